@@ -1,0 +1,177 @@
+/* polarquant.h — C ABI of the MI355X (gfx950) polar-key decode path.
+ *
+ * The reference has no C/FFI boundary for this path: its Python attention
+ * classes call a Triton JIT kernel and eager torch ops.  Each entry point below
+ * names the reference interface it replaces; the Python classes in
+ * polarquant_amd/ bind them through ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller, unless it is
+ *     documented as a host pointer;
+ *   - every call is asynchronous on `stream` (a hipStream_t passed as void*,
+ *     NULL = the default stream), performs no allocation and no
+ *     synchronisation, and never throws;
+ *   - the return value is PQ_OK (0) or a negative pq_status; argument errors are
+ *     detected on the host before anything is launched, so they can be tested
+ *     without a GPU;
+ *   - "half word" means a 16-bit float in the dtype given by `dtype`
+ *     (PQ_F16 = IEEE binary16, PQ_BF16 = bfloat16);
+ *   - head_dim is 128 (D = 64 dimension pairs (d, d+64)) and the group size G is
+ *     128 tokens, as in the reference (models/modeling_llama_polar.py:34-37).
+ */
+#ifndef POLARQUANT_H
+#define POLARQUANT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PQ_HEAD_DIM 128
+#define PQ_PAIRS 64
+#define PQ_GROUP 128
+#define PQ_MAX_REP 8          /* query heads per KV head (GQA ratio) supported by the kernels */
+#define PQ_PARTIAL_FLOATS 132 /* floats per split-K partial: m, l, 2 pad, acc[128] */
+
+typedef enum {
+    PQ_OK = 0,
+    PQ_ERR_NULL_POINTER = -1,
+    PQ_ERR_BAD_SHAPE = -2,      /* non-positive size, N % Nk != 0, rep > PQ_MAX_REP ... */
+    PQ_ERR_BAD_BITS = -3,       /* rbits/tbits outside [1,..], rbits + tbits > 8, tbits > 4 */
+    PQ_ERR_BAD_DTYPE = -4,
+    PQ_ERR_MISALIGNED = -5,     /* a pointer or stride breaks the alignment a kernel needs */
+    PQ_ERR_BAD_STRIDE = -6,
+    PQ_ERR_WORKSPACE = -7,      /* workspace too small / bad split count */
+    PQ_ERR_LAUNCH = -8,         /* hipLaunchKernel reported an error */
+    PQ_ERR_NO_DEVICE = -9
+} pq_status;
+
+typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
+
+/* flags for pq_quantize_groups */
+#define PQ_WRAP_FP32 1u /* add 2*pi in fp32 (eager CUDA semantics) instead of the
+                           dtype-rounded 6.28125 that eager CPU torch adds */
+
+/* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
+int pq_version(void);
+
+/* Human-readable text for a pq_status. Host-only. */
+const char *pq_status_string(int status);
+
+/* ---------------------------------------------------------------------------
+ * S — quantized-key decode scores.
+ * Replaces attention_decode_forward_triton_impl(query_states, indices, rscale,
+ * rmn, tscale, tmn, rbits, tbits) -> fp32 [B,N,1,Nb*G]
+ * (models/kernel4group.py:83-109, kernel :14-80).
+ *
+ *   q       [B,N,1,128]      half words, contiguous
+ *   codes   [B,Nk,Nb,128,64] u8, contiguous, code = (rho << tbits) + theta
+ *   rscale, rmn, tscale, tmn [B,Nk,Nb,1,64] half words, contiguous
+ *   out     [B,N,1,Nb*128]   fp32, contiguous
+ * out[b, kvh*rep + j, 0, g*128 + t] = sum_d (q[d] cos phi + q[d+64] sin phi) * r,
+ *   phi = tscale_d*(theta+0.5)+tmn_d, r = rscale_d*(rho+0.5)+rmn_d.  No 1/sqrt(d).
+ * Query head h reads KV head h / (N/Nk) (repeat-interleave, as HF repeat_kv).
+ * ------------------------------------------------------------------------- */
+int pq_decode_scores(const void *q, const uint8_t *codes, const void *rscale, const void *rmn,
+                     const void *tscale, const void *tmn, float *out,
+                     int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, void *stream);
+
+/* Host-only argument check of pq_decode_scores (same return codes, launches nothing). */
+int pq_validate_decode_scores(const void *q, const uint8_t *codes, const void *rscale, const void *rmn,
+                              const void *tscale, const void *tmn, const float *out,
+                              int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype);
+
+/* ---------------------------------------------------------------------------
+ * Q — polar quantizer (quantize-on-append and prompt quantization).
+ * Replaces LlamaPolarGroupAttention.quantize_and_pack_nbit(key_states)
+ * (models/modeling_llama_polar.py:135-157; models/modeling_qwen_polar.py:134-156).
+ *
+ *   k          post-RoPE keys, logical shape [B,Nk,Nb*128,128] half words, addressed
+ *              with element strides k_strides[4] = {batch, head, token, dim};
+ *              dim stride must be 1 (a transposed [B,L,Nk,128] view is fine)
+ *   k_strides  HOST pointer to 4 int64
+ *   codes      [B,Nk,Nb,128,64] u8 — written with group stride 128*64 inside a
+ *              (batch, head) plane of `out_group_capacity` groups, i.e. the plane
+ *              stride is out_group_capacity*128*64 (pass Nb for a dense output);
+ *              writing starts at group `out_group_offset` of each plane
+ *   rscale, rmn, tscale, tmn  [B,Nk,out_group_capacity,1,64] half words, same rule
+ * Arithmetic: every reference op is evaluated in fp32 and rounded to the key
+ * dtype before the next, which is what eager torch does on half tensors.
+ * Degenerate groups (scale == 0, quotient NaN/Inf) yield code 0.
+ * ------------------------------------------------------------------------- */
+int pq_quantize_groups(const void *k, const int64_t *k_strides, int dtype,
+                       int B, int Nk, int Nb, int rbits, int tbits, unsigned flags,
+                       uint8_t *codes, void *rscale, void *rmn, void *tscale, void *tmn,
+                       int out_group_capacity, int out_group_offset, void *stream);
+
+int pq_validate_quantize_groups(const void *k, const int64_t *k_strides, int dtype,
+                                int B, int Nk, int Nb, int rbits, int tbits, unsigned flags,
+                                const uint8_t *codes, const void *rscale, const void *rmn,
+                                const void *tscale, const void *tmn,
+                                int out_group_capacity, int out_group_offset);
+
+/* ---------------------------------------------------------------------------
+ * R+M+X+V — fused decode attention over the polar key cache.
+ * Replaces the decode branch of LlamaPolarGroupAttention.forward between the
+ * RoPE and o_proj (models/modeling_llama_polar.py:66-99; qwen :65-98): quantized
+ * scores, residual fp16 scores, concat, /sqrt(d), mask, fp32 softmax, P.V — in
+ * one pass over HBM with a split over the context and a merge kernel.
+ *
+ * The caller has already appended the step's new key to the residual buffer
+ * and the new value to the V cache (reference :77,98).
+ *
+ *   q        [B,N,128] half words, contiguous
+ *   codes    u8, (batch,head) plane stride = group_capacity*128*64; meta likewise
+ *            with plane stride group_capacity*64; may be NULL when no sequence has
+ *            a quantized group
+ *   n_groups number of quantized groups of every sequence (used when
+ *            n_groups_per_seq == NULL)
+ *   n_groups_per_seq  optional device int32 [B]: per-sequence group count (ragged)
+ *   k_resid  [B,Nk,resid_capacity,128] half words: fp16 keys not yet quantized
+ *   n_resid / n_resid_per_seq  residual key count, uniform or device int32 [B];
+ *            0..128
+ *   v        [B,Nk,v_capacity,128] half words; token t of sequence b is row t;
+ *            rows [0, n_groups*128 + n_resid) are read
+ *   mask     optional device u8 [B, mask_stride]: 1 = attend, 0 = masked; column t
+ *            is token t (reference attention_mask, :94-95); NULL = no mask
+ *   sm_scale multiplier applied to every score (1/sqrt(128) in the reference)
+ *   n_splits context splits per (batch, KV head) for the quantized part, >= 1;
+ *            use pq_decode_attn_plan to choose
+ *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
+ *   out      [B,N,128] half words
+ * ------------------------------------------------------------------------- */
+int pq_decode_attn(const void *q,
+                   const uint8_t *codes, const void *rscale, const void *rmn,
+                   const void *tscale, const void *tmn, int group_capacity,
+                   int n_groups, const int32_t *n_groups_per_seq,
+                   const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                   const void *v, int64_t v_capacity,
+                   const uint8_t *mask, int64_t mask_stride,
+                   float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                   int n_splits, void *workspace, size_t workspace_bytes,
+                   void *out, void *stream);
+
+int pq_validate_decode_attn(const void *q,
+                            const uint8_t *codes, const void *rscale, const void *rmn,
+                            const void *tscale, const void *tmn, int group_capacity,
+                            int n_groups, const int32_t *n_groups_per_seq,
+                            const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                            const void *v, int64_t v_capacity,
+                            const uint8_t *mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, const void *workspace, size_t workspace_bytes,
+                            const void *out);
+
+/* Suggested n_splits for a shape (host-only; `max_groups` = largest group count
+ * of any sequence, `n_cus` = compute units of the device or 0 for 256). */
+int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus);
+
+/* Bytes of workspace pq_decode_attn needs for (B, N, n_splits). Host-only. */
+size_t pq_decode_attn_workspace_bytes(int B, int N, int n_splits);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* POLARQUANT_H */

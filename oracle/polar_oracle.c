@@ -1,0 +1,195 @@
+/* CPU oracle (plain C) for the polar-key decode path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * An independent second restatement of the reference algorithm, written with
+ * scalar loops and libm so that it shares no code with oracle/polar_oracle.py
+ * (torch) or with the HIP product.  Only tests/, __graft_entry__.smoke() and
+ * bench.py's cpu_baseline leg may load the library built from this file.
+ *
+ * Reference lines followed:
+ *   po_quantize      models/modeling_llama_polar.py:135-157
+ *   po_scores        models/kernel4group.py:64-77 (semantics), :151-155 (formula)
+ *   po_decode_attn   models/modeling_llama_polar.py:77-99
+ *
+ * Pin status: see the header of oracle/polar_oracle.py; the two restatements
+ * are checked against each other bit-for-bit (codes, metadata) and to 1e-6
+ * (scores) in tests/test_oracle_pins.py.  The angle uses libm atan2f where the
+ * torch restatement uses torch.atan2 (Sleef): a last-ulp difference between the
+ * two can move a code across a bin edge; the tests count such flips.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ---- half / bfloat16 <-> float, round-to-nearest-even ---- */
+static float h2f(uint16_t h) {
+    uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1f, m = h & 0x3ffu, u;
+    if (e == 0) {
+        if (m == 0) u = s;
+        else { int sh = 0; while (!(m & 0x400u)) { m <<= 1; sh++; } m &= 0x3ffu; u = s | ((uint32_t)(113 - sh) << 23) | (m << 13); }
+    } else if (e == 31) u = s | 0x7f800000u | (m << 13);
+    else u = s | ((e + 112) << 23) | (m << 13);
+    float f; memcpy(&f, &u, 4); return f;
+}
+static uint16_t f2h(float f) {
+    uint32_t u; memcpy(&u, &f, 4);
+    uint32_t s = (u >> 16) & 0x8000u, e = (u >> 23) & 0xff, m = u & 0x7fffffu;
+    if (e == 255) return (uint16_t)(s | 0x7c00u | (m ? 0x200u : 0));
+    int ex = (int)e - 127 + 15;
+    if (ex >= 31) return (uint16_t)(s | 0x7c00u);
+    if (ex <= 0) {
+        if (ex < -10) return (uint16_t)s;
+        m |= 0x800000u;
+        int sh = 14 - ex;
+        uint32_t r = m >> sh, rem = m & ((1u << sh) - 1), half = 1u << (sh - 1);
+        if (rem > half || (rem == half && (r & 1))) r++;
+        return (uint16_t)(s | r);
+    }
+    uint32_t r = ((uint32_t)ex << 10) | (m >> 13), rem = m & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) r++;
+    return (uint16_t)(s | r);
+}
+static float b2f(uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; }
+static uint16_t f2b(float f) {
+    uint32_t u; memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1);
+    return (uint16_t)(u >> 16);
+}
+static inline float lo2f(uint16_t h, int bf) { return bf ? b2f(h) : h2f(h); }
+static inline uint16_t f2lo(float f, int bf) { return bf ? f2b(f) : f2h(f); }
+/* round a float through the low-precision type: one eager torch op's result */
+static inline float rnd(float f, int bf) { return lo2f(f2lo(f, bf), bf); }
+
+float po_half_to_float(uint16_t h) { return h2f(h); }
+uint16_t po_float_to_half(float f) { return f2h(f); }
+
+static uint8_t code_of(float v, float mn, float scale, int bits, int bf) {
+    float d = rnd(v - mn, bf);
+    float q = rnd(d / scale, bf);
+    q = floorf(q);
+    if (!(q == q) || isinf(q)) return 0;          /* NaN/Inf -> 0 (defined here; UB in the reference) */
+    if (q < 0) q = 0;
+    if (q > 255) q = 255;
+    int c = (int)q, top = (1 << bits) - 1;
+    return (uint8_t)(c > top ? top : c);
+}
+
+/* k: [B,Nk,L,2D] contiguous low-precision words.  Outputs contiguous:
+ * codes [B,Nk,Nb,G,D] u8; rscale,rmn,tscale,tmn [B,Nk,Nb,D] low-precision words. */
+int po_quantize(const uint16_t *k, int bf, int wrap_fp32, int B, int Nk, int L, int D, int G, int rbits, int tbits,
+                uint8_t *codes, uint16_t *rscale, uint16_t *rmn, uint16_t *tscale, uint16_t *tmn) {
+    if (L % G || rbits + tbits > 8) return -1;
+    /* torch-CPU casts the python scalar 2*pi to the tensor dtype before the add
+     * (6.28125 in both half and bfloat16); wrap_fp32 != 0 keeps it in fp32, which
+     * is what an eager CUDA add of a half tensor and a python scalar does. */
+    const float TWO_PI = wrap_fp32 ? (float)(2.0 * 3.14159265358979323846)
+                                   : rnd((float)(2.0 * 3.14159265358979323846), bf);
+    int Nb = L / G;
+    float *phi = (float *)malloc(sizeof(float) * G), *rad = (float *)malloc(sizeof(float) * G);
+    for (long bh = 0; bh < (long)B * Nk; bh++)
+        for (int nb = 0; nb < Nb; nb++)
+            for (int d = 0; d < D; d++) {
+                const uint16_t *base = k + ((bh * L) + (long)nb * G) * 2 * D;
+                float pmx = -INFINITY, pmn = INFINITY, rmx_ = -INFINITY, rmn_ = INFINITY;
+                for (int g = 0; g < G; g++) {
+                    float x = lo2f(base[(long)g * 2 * D + d], bf), y = lo2f(base[(long)g * 2 * D + D + d], bf);
+                    float p = rnd(atan2f(y, x), bf);                       /* :143 */
+                    if (p < 0) p = rnd(p + TWO_PI, bf);                    /* :144 */
+                    float r = rnd(sqrtf(x * x + y * y), bf);               /* :150 */
+                    phi[g] = p; rad[g] = r;
+                    if (p > pmx) pmx = p;
+                    if (p < pmn) pmn = p;
+                    if (r > rmx_) rmx_ = r;
+                    if (r < rmn_) rmn_ = r;
+                }
+                float ts = rnd(rnd(pmx - pmn, bf) / (float)(1 << tbits), bf);   /* :147 */
+                float rs = rnd(rnd(rmx_ - rmn_, bf) / (float)(1 << rbits), bf); /* :152 */
+                long mi = (bh * Nb + nb) * D + d;
+                tscale[mi] = f2lo(ts, bf); tmn[mi] = f2lo(pmn, bf);
+                rscale[mi] = f2lo(rs, bf); rmn[mi] = f2lo(rmn_, bf);
+                for (int g = 0; g < G; g++) {
+                    uint8_t th = code_of(phi[g], pmn, ts, tbits, bf);      /* :148 */
+                    uint8_t rh = code_of(rad[g], rmn_, rs, rbits, bf);     /* :153 */
+                    codes[((bh * Nb + nb) * G + g) * D + d] = (uint8_t)((rh << tbits) + th);  /* :155 */
+                }
+            }
+    free(phi); free(rad);
+    return 0;
+}
+
+/* scores[b,h,l] = sum_d (q[d] cos phi^ + q[d+D] sin phi^) * r^ ; out [B,N,Nb*G] fp32 */
+int po_scores(const uint16_t *q, int bf, const uint8_t *codes, const uint16_t *rscale, const uint16_t *rmn,
+              const uint16_t *tscale, const uint16_t *tmn, float *out,
+              int B, int N, int Nk, int Nb, int G, int D, int rbits, int tbits) {
+    (void)rbits;
+    int rep = N / Nk, nt = 1 << tbits;
+    double *lc = (double *)malloc(sizeof(double) * D * nt), *ls = (double *)malloc(sizeof(double) * D * nt);
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < N; h++) {
+            int kvh = h / rep;
+            const uint16_t *qq = q + ((long)b * N + h) * 2 * D;
+            for (int nb = 0; nb < Nb; nb++) {
+                long mi = (((long)b * Nk + kvh) * Nb + nb) * D;
+                for (int d = 0; d < D; d++)
+                    for (int t = 0; t < nt; t++) {
+                        double p = (double)lo2f(tscale[mi + d], bf) * (t + 0.5) + (double)lo2f(tmn[mi + d], bf);
+                        lc[d * nt + t] = cos(p); ls[d * nt + t] = sin(p);
+                    }
+                for (int g = 0; g < G; g++) {
+                    const uint8_t *c = codes + ((((long)b * Nk + kvh) * Nb + nb) * G + g) * D;
+                    double acc = 0;
+                    for (int d = 0; d < D; d++) {
+                        int th = c[d] & (nt - 1), rh = c[d] >> tbits;
+                        double r = (double)lo2f(rscale[mi + d], bf) * (rh + 0.5) + (double)lo2f(rmn[mi + d], bf);
+                        acc += ((double)lo2f(qq[d], bf) * lc[d * nt + th] + (double)lo2f(qq[D + d], bf) * ls[d * nt + th]) * r;
+                    }
+                    out[((long)b * N + h) * Nb * G + (long)nb * G + g] = (float)acc;
+                }
+            }
+        }
+    free(lc); free(ls);
+    return 0;
+}
+
+/* Full decode attention for one step (new k/v already appended by the caller).
+ * q [B,N,2D]; codes/meta as above (Nb groups, may be 0); kres [B,Nk,res,2D]; v [B,Nk,Nb*G+res,2D];
+ * mask [B,Nb*G+res] bytes (1 keep) or NULL; out [B,N,2D] low-precision words. */
+int po_decode_attn(const uint16_t *q, int bf, const uint8_t *codes, const uint16_t *rscale, const uint16_t *rmn,
+                   const uint16_t *tscale, const uint16_t *tmn, const uint16_t *kres, int res,
+                   const uint16_t *v, const uint8_t *mask, uint16_t *out,
+                   int B, int N, int Nk, int Nb, int G, int D, int rbits, int tbits) {
+    int rep = N / Nk, Lq = Nb * G, Lt = Lq + res, hd = 2 * D;
+    float *sq = (float *)malloc(sizeof(float) * (size_t)B * N * (Lq ? Lq : 1));
+    if (Nb) po_scores(q, bf, codes, rscale, rmn, tscale, tmn, sq, B, N, Nk, Nb, G, D, rbits, tbits);
+    double *s = (double *)malloc(sizeof(double) * Lt), *acc = (double *)malloc(sizeof(double) * hd);
+    double isq = 1.0 / sqrt((double)hd);
+    for (int b = 0; b < B; b++)
+        for (int h = 0; h < N; h++) {
+            int kvh = h / rep;
+            const uint16_t *qq = q + ((long)b * N + h) * hd;
+            for (int l = 0; l < Lq; l++) s[l] = (double)sq[((long)b * N + h) * Lq + l] * isq;
+            for (int l = 0; l < res; l++) {
+                const uint16_t *kk = kres + (((long)b * Nk + kvh) * res + l) * hd;
+                float a = 0;
+                for (int d = 0; d < hd; d++) a += lo2f(qq[d], bf) * lo2f(kk[d], bf);
+                s[Lq + l] = (double)rnd(a, bf) * isq;                      /* half matmul then .to(float32), :79 */
+            }
+            double mx = -INFINITY;
+            for (int l = 0; l < Lt; l++) {
+                if (mask && !mask[(long)b * Lt + l]) s[l] = -INFINITY;
+                if (s[l] > mx) mx = s[l];
+            }
+            double den = 0;
+            for (int l = 0; l < Lt; l++) { s[l] = exp(s[l] - mx); den += s[l]; }
+            for (int d = 0; d < hd; d++) acc[d] = 0;
+            for (int l = 0; l < Lt; l++) {
+                double p = (double)rnd((float)(s[l] / den), bf);           /* softmax(...).to(q.dtype), :97 */
+                const uint16_t *vv = v + (((long)b * Nk + kvh) * Lt + l) * hd;
+                for (int d = 0; d < hd; d++) acc[d] += p * lo2f(vv[d], bf);
+            }
+            for (int d = 0; d < hd; d++) out[((long)b * N + h) * hd + d] = f2lo((float)acc[d], bf);
+        }
+    free(sq); free(s); free(acc);
+    return 0;
+}

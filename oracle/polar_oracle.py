@@ -1,0 +1,283 @@
+"""CPU oracle for the polar-key decode path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, with torch-CPU library routines, the algorithm of the
+reference's polar-key decode path.  Only tests/, __graft_entry__.smoke() and
+bench.py's cpu_baseline leg may import it; the product (polarquant_amd/) never
+does.  Every function cites the reference lines it follows.
+
+Pin status (what proves each function is right, beyond retyping a formula;
+the checks live in tests/test_oracle_pins.py):
+
+  quantize_and_pack_nbit   pinned: brute-force fp64 quantizer on tiny inputs,
+                           closed-form known-answer group (angles on bin
+                           centres), min/max-element invariants, error bounds,
+                           cross-check against the independent C restatement
+                           (oracle/polar_oracle.c).  The reference holds no
+                           golden vectors for it.
+  dequantize_keys          pinned: closed form on the known-answer group,
+                           error bounds |phi-phi^|<=tscale/2, |r-r^|<=rscale/2.
+  decode_scores            pinned: textbook q.K^T (torch.matmul) on the
+                           dequantized keys, LUT identity |q|cos(phi-psi),
+                           pure-python brute force on one group, C cross-check.
+  decode_attention         pinned: composition of torch.matmul/softmax library
+                           routines; cross-checked against a one-shot softmax
+                           over the concatenated dequantized+residual keys.
+  prefill_cache/decode_step pinned: shape/bookkeeping property tests (quantized
+                           token count, residual length, kv_seq_len).
+  Degenerate groups (tscale==0 or rscale==0 -> 0/0) are undefined behaviour in
+  the reference (NaN -> uint8); this oracle defines the code as 0 there, which
+  is what torch-CPU's cast yields.  That choice is "parity unpinned".
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+GROUP_SIZE = 128
+
+
+# --------------------------------------------------------------------------
+# RoPE (HF rotate-half convention, transformers modeling_llama.apply_rotary_pos_emb)
+# used only to build synthetic post-RoPE keys.
+# --------------------------------------------------------------------------
+def rope_cos_sin(positions: torch.Tensor, head_dim: int, theta: float, dtype=torch.float32):
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+    freqs = positions.to(torch.float32)[:, None] * inv_freq[None, :]
+    emb = torch.cat([freqs, freqs], dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    h = x.shape[-1] // 2
+    return torch.cat([-x[..., h:], x[..., :h]], dim=-1)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [..., L, D]; cos/sin [L, D]."""
+    return x * cos + rotate_half(x) * sin
+
+
+# --------------------------------------------------------------------------
+# Q: polar quantizer  (models/modeling_llama_polar.py:135-157, identical to
+# models/modeling_qwen_polar.py:134-156 and models/kernel4group.py:126-139)
+# --------------------------------------------------------------------------
+def _to_u8_defined(x: torch.Tensor) -> torch.Tensor:
+    """floor(x).to(uint8) with NaN/Inf -> 0 made explicit (torch-CPU behaviour)."""
+    x = torch.floor(x)
+    x = torch.where(torch.isfinite(x), x, torch.zeros_like(x))
+    return x.to(torch.float32).clamp_(0, 255).to(torch.uint8)
+
+
+def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4,
+                           group_size: int = GROUP_SIZE):
+    """key_states [B,Nk,L,2*D] half/bf16 (post-RoPE) ->
+    (indices u8 [B,Nk,Nb,G,D], rscale, rmn, tscale, tmn [B,Nk,Nb,1,D] in key dtype).
+
+    Every op runs eagerly in the key dtype, exactly as the reference does
+    (modeling_llama_polar.py:141-155): x = dims [0,D), y = dims [D,2D).
+    """
+    B, N, L, D2 = key_states.shape
+    assert D2 % 2 == 0 and L % group_size == 0 and rbits + tbits <= 8
+    D, G = D2 // 2, group_size
+    ks = key_states.reshape(B, N, L // G, G, 2, D)
+
+    phi = torch.atan2(ks[:, :, :, :, 1, :], ks[:, :, :, :, 0, :])             # :143
+    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)                        # :144
+    tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]      # :146
+    tscale = (tmx - tmn) / (2 ** tbits)                                       # :147
+    theta = torch.clamp(_to_u8_defined((phi - tmn) / tscale), 0, 2 ** tbits - 1)  # :148
+
+    radii = torch.norm(ks, p=2, dim=-2)                                       # :150
+    rmx, rmn = radii.max(-2, keepdim=True)[0], radii.min(-2, keepdim=True)[0]  # :151
+    rscale = (rmx - rmn) / (2 ** rbits)                                       # :152
+    rho = torch.clamp(_to_u8_defined((radii - rmn) / rscale), 0, 2 ** rbits - 1)  # :153
+
+    indices = (rho << tbits) + theta                                          # :155
+    return indices, rscale, rmn, tscale, tmn
+
+
+def quantize_brute_fp64(key_states: torch.Tensor, rbits: int, tbits: int, group_size: int = GROUP_SIZE):
+    """Same quantizer in exact-ish fp64 arithmetic with no half rounding of the
+    intermediates.  Where it disagrees with quantize_and_pack_nbit the
+    disagreement is by definition a rounding "edge flip"."""
+    B, N, L, D2 = key_states.shape
+    D, G = D2 // 2, group_size
+    ks = key_states.to(torch.float64).reshape(B, N, L // G, G, 2, D)
+    x, y = ks[..., 0, :], ks[..., 1, :]
+    phi = torch.atan2(y, x)
+    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)
+    tmx, tmn = phi.amax(-2, keepdim=True), phi.amin(-2, keepdim=True)
+    tscale = (tmx - tmn) / (2 ** tbits)
+    theta = torch.clamp(torch.nan_to_num(torch.floor((phi - tmn) / tscale), nan=0.0, posinf=0.0), 0, 2 ** tbits - 1)
+    r = torch.sqrt(x * x + y * y)
+    rmx, rmn = r.amax(-2, keepdim=True), r.amin(-2, keepdim=True)
+    rscale = (rmx - rmn) / (2 ** rbits)
+    rho = torch.clamp(torch.nan_to_num(torch.floor((r - rmn) / rscale), nan=0.0, posinf=0.0), 0, 2 ** rbits - 1)
+    idx = (rho.to(torch.int64) << tbits) + theta.to(torch.int64)
+    return idx.to(torch.uint8), rscale, rmn, tscale, tmn
+
+
+# --------------------------------------------------------------------------
+# dequantize (models/kernel4group.py:151-153; fp32 bin centres as the Triton
+# kernel evaluates them, kernel4group.py:67,73)
+# --------------------------------------------------------------------------
+def dequantize_keys(indices, rscale, rmn, tscale, tmn, rbits: int = 4, tbits: int = 4,
+                    dtype=torch.float32) -> torch.Tensor:
+    """-> K^ [B,Nk,Nb*G,2*D] in `dtype` (fp32 or fp64): (r^ cos phi^ || r^ sin phi^)."""
+    B, Nk, Nb, G, D = indices.shape
+    theta = (indices & (2 ** tbits - 1)).to(dtype)
+    rho = (indices >> tbits).to(dtype)
+    phi = tscale.to(dtype) * (theta + 0.5) + tmn.to(dtype)
+    rad = rscale.to(dtype) * (rho + 0.5) + rmn.to(dtype)
+    k = torch.stack([rad * torch.cos(phi), rad * torch.sin(phi)], dim=-2)  # [B,Nk,Nb,G,2,D]
+    return k.reshape(B, Nk, Nb * G, 2 * D)
+
+
+def repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """HF repeat_kv: [B,Nk,L,D] -> [B,Nk*n_rep,L,D], query head h uses kv head h//n_rep."""
+    if n_rep == 1:
+        return x
+    B, Nk, L, D = x.shape
+    return x[:, :, None, :, :].expand(B, Nk, n_rep, L, D).reshape(B, Nk * n_rep, L, D)
+
+
+# --------------------------------------------------------------------------
+# S: quantized-key scores (models/kernel4group.py:14-109; oracle formula :151-155)
+# --------------------------------------------------------------------------
+def decode_scores(query_states, indices, rscale, rmn, tscale, tmn, rbits: int = 4, tbits: int = 4,
+                  dtype=torch.float32) -> torch.Tensor:
+    """query [B,N,1,2D] -> fp32/fp64 scores [B,N,1,Nb*G] = q . K^^T, no 1/sqrt(d)."""
+    B, N = query_states.shape[:2]
+    Nk = indices.shape[1]
+    khat = dequantize_keys(indices, rscale, rmn, tscale, tmn, rbits, tbits, dtype)
+    return torch.matmul(query_states.to(dtype), repeat_kv(khat, N // Nk).transpose(2, 3))
+
+
+def decode_scores_lut_python(query, indices, rscale, rmn, tscale, tmn, rbits, tbits, b, h, group):
+    """Pure-python float64 restatement of one program of the Triton kernel
+    (kernel4group.py:64-77): LUT over angle bins, gather, radius, sum over pairs.
+    Returns a list of G python floats for query head h, one 128-token group."""
+    B, Nk, Nb, G, D = indices.shape
+    N = query.shape[1]
+    kvh = h // (N // Nk)
+    out = []
+    q = query[b, h, 0].to(torch.float64).tolist()
+    ts = tscale[b, kvh, group, 0].to(torch.float64).tolist()
+    tm = tmn[b, kvh, group, 0].to(torch.float64).tolist()
+    rs = rscale[b, kvh, group, 0].to(torch.float64).tolist()
+    rm = rmn[b, kvh, group, 0].to(torch.float64).tolist()
+    idx = indices[b, kvh, group].tolist()
+    for g in range(G):
+        acc = 0.0
+        for d in range(D):
+            code = idx[g][d]
+            th, rh = code & ((1 << tbits) - 1), code >> tbits
+            phi = ts[d] * (th + 0.5) + tm[d]
+            rad = rs[d] * (rh + 0.5) + rm[d]
+            acc += (q[d] * math.cos(phi) + q[d + D] * math.sin(phi)) * rad
+        out.append(acc)
+    return out
+
+
+# --------------------------------------------------------------------------
+# R/M/X/V: full decode attention (models/modeling_llama_polar.py:61-101)
+# --------------------------------------------------------------------------
+def decode_attention(query_states, key_resid, indices, rscale, rmn, tscale, tmn, value_states,
+                     attention_mask: Optional[torch.Tensor] = None, rbits: int = 4, tbits: int = 4,
+                     score_dtype=torch.float32) -> torch.Tensor:
+    """One decode step's attention, AFTER the new key/value have been appended
+    to key_resid / value_states (modeling_llama_polar.py:77,98).
+
+    query [B,N,1,128]; key_resid [B,Nk,res,128] (res>=1) or None; quant tensors
+    or None; value_states [B,Nk,Lq+res,128]; attention_mask [B,Lq+res] of {0,1}.
+    Returns attn_output [B,N,1,128] in query dtype.
+    """
+    B, N, _, hd = query_states.shape
+    Nk = value_states.shape[1]
+    rep = N // Nk
+    parts = []
+    if indices is not None:
+        parts.append(decode_scores(query_states, indices, rscale, rmn, tscale, tmn, rbits, tbits,
+                                   score_dtype).to(torch.float32))                       # :66-75
+    if key_resid is not None and key_resid.shape[2] > 0:
+        # the reference multiplies in the model dtype then promotes (:79); the
+        # product of two halves summed in fp32 then rounded to half is what a
+        # half matmul yields, so do exactly that.
+        w = torch.matmul(query_states.float(), repeat_kv(key_resid, rep).float().transpose(2, 3))
+        parts.append(w.to(query_states.dtype).to(torch.float32))
+    attn = torch.cat(parts, dim=-1) / math.sqrt(hd)                                     # :80
+    if attention_mask is not None:
+        attn = attn + (1.0 - attention_mask[:, None, None, :].to(torch.float32)) * torch.finfo(torch.float32).min  # :94-95
+    p = torch.softmax(attn, dim=-1).to(query_states.dtype)                               # :97
+    out = torch.matmul(p.float(), repeat_kv(value_states, rep).float())                  # :99
+    return out.to(query_states.dtype)
+
+
+def decode_attention_exact(query_states, key_resid, indices, rscale, rmn, tscale, tmn, value_states,
+                           attention_mask=None, rbits=4, tbits=4) -> torch.Tensor:
+    """Same attention in fp64 with no intermediate half rounding; returns fp64
+    [B,N,1,128].  Used as the centre of the tolerance band for the HIP kernel."""
+    B, N, _, hd = query_states.shape
+    Nk = value_states.shape[1]
+    rep = N // Nk
+    ks = []
+    if indices is not None:
+        ks.append(dequantize_keys(indices, rscale, rmn, tscale, tmn, rbits, tbits, torch.float64))
+    if key_resid is not None and key_resid.shape[2] > 0:
+        ks.append(key_resid.to(torch.float64))
+    k = torch.cat(ks, dim=2)
+    attn = torch.matmul(query_states.to(torch.float64), repeat_kv(k, rep).transpose(2, 3)) / math.sqrt(hd)
+    if attention_mask is not None:
+        attn = attn.masked_fill(attention_mask[:, None, None, :] == 0, float("-inf"))
+    p = torch.softmax(attn, dim=-1)
+    return torch.matmul(p, repeat_kv(value_states.to(torch.float64), rep))
+
+
+# --------------------------------------------------------------------------
+# C/P/F: cache tuple bookkeeping (modeling_llama_polar.py:62,83-92,101,116-128)
+# --------------------------------------------------------------------------
+def prefill_cache(key_states, value_states, rbits=4, tbits=4, residual_length=GROUP_SIZE):
+    """Prompt keys/values [B,Nk,L,128] -> the reference's 8-tuple (:116-128)."""
+    L = key_states.shape[2]
+    r = L % residual_length
+    if r == 0:
+        k_full, k_quant = None, key_states
+    else:
+        k_full = key_states if L < residual_length else key_states[:, :, -r:, :]
+        k_quant = None if L < residual_length else key_states[:, :, :-r, :]
+    ind = rs = rm = ts = tm = None
+    if k_quant is not None:
+        ind, rs, rm, ts, tm = quantize_and_pack_nbit(k_quant.contiguous(), rbits, tbits, residual_length)
+    return (k_full, ind, rs, rm, ts, tm, value_states, L)
+
+
+def decode_step(query_states, key_states, value_states, past_key_value, attention_mask=None,
+                rbits=4, tbits=4, residual_length=GROUP_SIZE):
+    """One decode step on post-RoPE q/k/v [B,H,1,128] (:61-101) -> (attn_output, new tuple)."""
+    k_full, ind, rs, rm, ts, tm, v_full, kv_len = past_key_value
+    k_full = key_states if k_full is None else torch.cat([k_full, key_states], dim=2)       # :77
+    v_full = torch.cat([v_full, value_states], dim=2)                                       # :98
+    out = decode_attention(query_states, k_full, ind, rs, rm, ts, tm, v_full, attention_mask, rbits, tbits)
+    if k_full.shape[2] % residual_length == 0:                                              # :83
+        i2, rs2, rm2, ts2, tm2 = quantize_and_pack_nbit(k_full.contiguous(), rbits, tbits, residual_length)
+        cat = lambda a, b: b if a is None else torch.cat([a, b], dim=2)
+        ind, rs, rm, ts, tm = cat(ind, i2), cat(rs, rs2), cat(rm, rm2), cat(ts, ts2), cat(tm, tm2)
+        k_full = None
+    return out, (k_full, ind, rs, rm, ts, tm, v_full, kv_len + 1)
+
+
+# --------------------------------------------------------------------------
+# fp16 un-quantized decode attention: the baseline the reference benchmarks
+# against (benchmark/models/modeling_llama_exp.py:39-54)
+# --------------------------------------------------------------------------
+def fp16_decode_attention(query_states, key_states, value_states, attention_mask=None):
+    B, N, _, hd = query_states.shape
+    rep = N // key_states.shape[1]
+    attn = torch.matmul(query_states.float(), repeat_kv(key_states, rep).float().transpose(2, 3))
+    attn = attn.to(query_states.dtype).float() / math.sqrt(hd)
+    if attention_mask is not None:
+        attn = attn + (1.0 - attention_mask[:, None, None, :].float()) * torch.finfo(torch.float32).min
+    p = torch.softmax(attn, dim=-1).to(query_states.dtype)
+    return torch.matmul(p.float(), repeat_kv(value_states, rep).float()).to(query_states.dtype)

@@ -1,0 +1,229 @@
+// Device-side building blocks shared by the polar-key kernels (gfx950, wave64).
+//
+// Work decomposition used by every kernel here:
+//   * one wavefront owns one 128-token group at a time and works through it in
+//     two 64-token tiles, lane == token;
+//   * per group the wavefront first builds, with lane == dimension pair d, an
+//     angle lookup table in its private slice of LDS:
+//         LUT[d][theta][j] = rscale_d * (q_j[d] cos phi + q_j[d+64] sin phi),
+//         phi = tscale_d * (theta + 0.5) + tmn_d          (kernel4group.py:67-69)
+//     for the `rep` query heads j that share the KV head;
+//   * in the tile loop every lane walks the 64 pair codes of its token.  All
+//     lanes look at the same pair d at the same time, so the LDS address differs
+//     between lanes only by theta: equal theta is a broadcast, different theta
+//     are different banks.  The radius bin centre r = rscale*(rho+0.5)+rmn
+//     (kernel4group.py:73) is applied as (rho + c_d) with the wave-uniform
+//     c_d = (rmn_d + rscale_d/2)/rscale_d, because rscale_d is already folded
+//     into the table.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+namespace pq {
+
+constexpr int kPairs = 64;
+constexpr int kGroup = 128;
+constexpr int kHeadDim = 128;
+constexpr int kWave = 64;
+
+struct F16 {};
+struct BF16 {};
+
+template <typename T> __device__ __forceinline__ float lo2f(uint16_t w);
+template <> __device__ __forceinline__ float lo2f<F16>(uint16_t w) {
+    return __half2float(__ushort_as_half(w));
+}
+template <> __device__ __forceinline__ float lo2f<BF16>(uint16_t w) {
+    return __uint_as_float(static_cast<uint32_t>(w) << 16);
+}
+template <typename T> __device__ __forceinline__ uint16_t f2lo(float f);
+template <> __device__ __forceinline__ uint16_t f2lo<F16>(float f) {
+    return __half_as_ushort(__float2half_rn(f));
+}
+template <> __device__ __forceinline__ uint16_t f2lo<BF16>(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).  Unlike
+// "#pragma unroll" the indices are constants when the body is instantiated, so
+// register arrays indexed by them never fall back to scratch memory.
+template <int I> struct IC { static constexpr int value = I; constexpr operator int() const { return I; } };
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) { f(IC<I>{}); static_for<N, I + 1>(f); }
+}
+
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+    return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
+
+// Geometry of the per-wave lookup table for TB angle bits and REPP (1,2,4,8)
+// padded query heads.  An entry holds min(REPP,4) floats; REPP == 8 keeps two
+// tables ("halves") of 4-float entries.  Within pair d the entry of angle bin
+// theta sits at slot theta ^ (d & (NB-1)): the XOR spreads the 64 lanes of the
+// build phase (lane == d, fixed theta) over all banks, and is undone for free in
+// the tile loop by XOR-ing four codes at a time with a compile-time constant.
+template <int TB, int REPP>
+struct Lut {
+    static constexpr int NB = 1 << TB;
+    static constexpr int ENTRY = REPP < 4 ? REPP : 4;
+    static constexpr int HALVES = REPP / ENTRY;
+    static constexpr int EB = ENTRY * 4;          // entry bytes
+    static constexpr int SH = ENTRY == 1 ? 2 : (ENTRY == 2 ? 3 : 4);
+    static constexpr int PB = NB * EB;            // bytes per pair
+    static constexpr int HB = kPairs * PB;        // bytes per half
+    static constexpr int BYTES = HALVES * HB;
+    static_assert(TB + SH <= 8, "theta*entry_bytes must fit a byte");
+};
+
+// LDS is addressed with 32-bit byte addresses in address space 3 so that the
+// compiler emits ds_read_b128/ds_write_b128 with the pair offset folded into
+// the instruction's immediate offset field.
+struct __attribute__((aligned(16))) Entry4 { float x, y, z, w; };
+struct __attribute__((aligned(8))) Entry2 { float x, y; };
+typedef __attribute__((address_space(3))) Entry4 lds_e4;
+typedef __attribute__((address_space(3))) Entry2 lds_e2;
+typedef __attribute__((address_space(3))) float lds_f1;
+typedef __attribute__((address_space(3))) void lds_void;
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wint-to-pointer-cast"
+
+template <typename P>
+__device__ __forceinline__ P* lds_ptr(uint32_t addr) { return (P*)(addr); }
+
+__device__ __forceinline__ uint32_t lds_addr(void* p) {
+    return (uint32_t)(uintptr_t)((lds_void*)p);
+}
+
+// Build the table for one group.  lane == pair d.
+//   qx[j], qy[j]: q_j[d], q_j[d+64] (0 for padded heads)
+//   returns c_d for this lane's pair.
+template <typename T, int TB, int REPP>
+__device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (&qx)[REPP], const float (&qy)[REPP],
+                                           uint16_t w_rscale, uint16_t w_rmn, uint16_t w_tscale, uint16_t w_tmn) {
+    using L = Lut<TB, REPP>;
+    const float ts = lo2f<T>(w_tscale), tm = lo2f<T>(w_tmn);
+    const float rs = lo2f<T>(w_rscale), rm = lo2f<T>(w_rmn);
+    float s, c, sd, cd;
+    sincosf(__builtin_fmaf(ts, 0.5f, tm), &s, &c);
+    sincosf(ts, &sd, &cd);
+    const float rmp = __builtin_fmaf(rs, 0.5f, rm);
+    float a, cdv;
+    if (rs != 0.0f) { a = rs; cdv = rmp / rs; }
+    else            { a = rmp * 0x1p-40f; cdv = 0x1p40f; }   // (rho + 2^40) * 2^-40 == 1 exactly
+    float ax[REPP], ay[REPP];
+#pragma unroll
+    for (int j = 0; j < REPP; j++) { ax[j] = qx[j] * a; ay[j] = qy[j] * a; }
+    const uint32_t base = lut + lane * L::PB + ((lane & (L::NB - 1)) << L::SH);
+#pragma unroll
+    for (int k = 0; k < L::NB; k++) {
+        float e[REPP];
+#pragma unroll
+        for (int j = 0; j < REPP; j++) e[j] = __builtin_fmaf(ax[j], c, ay[j] * s);
+        const uint32_t off = base ^ (k << L::SH);
+        if constexpr (L::ENTRY == 1) {
+            *lds_ptr<lds_f1>(off) = e[0];
+        } else if constexpr (L::ENTRY == 2) {
+            lds_e2* p = lds_ptr<lds_e2>(off);
+            p->x = e[0]; p->y = e[1];
+        } else {
+#pragma unroll
+            for (int h = 0; h < L::HALVES; h++) {
+                lds_e4* p = lds_ptr<lds_e4>(off + h * L::HB);
+                p->x = e[h * 4]; p->y = e[h * 4 + 1]; p->z = e[h * 4 + 2]; p->w = e[h * 4 + 3];
+            }
+        }
+        const float c2 = __builtin_fmaf(c, cd, -(s * sd));
+        const float s2 = __builtin_fmaf(s, cd, c * sd);
+        c = c2; s = s2;
+    }
+    return cdv;
+}
+
+// Score one token against the table.  `codes` holds the token's 64 pair codes as
+// 16 little-endian words; cds[d] are the wave-uniform c_d.  acc[j] += ...
+// The 64 table reads are issued in batches of 8 codes, one batch ahead of the
+// FMAs that consume them, so that 8-16 LDS reads are always in flight.
+template <int TB, int REPP>
+__device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes)[16], const float (&cds)[kPairs],
+                                            float (&acc)[REPP]) {
+    using L = Lut<TB, REPP>;
+    constexpr uint32_t TM4 = ((1u << TB) - 1u) * 0x01010101u;
+    constexpr uint32_t RM4 = (0xFFu >> TB) * 0x01010101u;
+    constexpr int nbm = L::NB - 1;
+    constexpr int BW = REPP == 8 ? 1 : 2;      // code words per batch
+    constexpr int NBATCH = 16 / BW;
+    float e[2][BW * 4][REPP];
+    uint32_t r4s[2][BW];
+
+    auto load = [&](auto BI) {
+        constexpr int bi = decltype(BI)::value, buf = bi & 1;
+        static_for<BW>([&](auto CC) {
+            constexpr int cc = decltype(CC)::value, c = bi * BW + cc;
+            const uint32_t w = codes[c];
+            // byte i of kc: XOR pattern of pair 4c+i, already scaled to bytes
+            constexpr uint32_t kc = ((uint32_t)(((4 * c + 0) & nbm) << L::SH)) | ((uint32_t)(((4 * c + 1) & nbm) << L::SH) << 8) |
+                                    ((uint32_t)(((4 * c + 2) & nbm) << L::SH) << 16) | ((uint32_t)(((4 * c + 3) & nbm) << L::SH) << 24);
+            uint32_t a4 = ((w & TM4) << L::SH) ^ kc;   // byte i: LDS byte offset of theta_i inside pair 4c+i
+            uint32_t r4 = (w >> TB) & RM4;             // byte i: rho_i
+            // keep the packed forms: byte i is then picked by v_bfe_u32 / v_cvt_f32_ubyte<i>
+            asm volatile("" : "+v"(a4), "+v"(r4));
+            r4s[buf][cc] = r4;
+            static_for<4>([&](auto II) {
+                constexpr int i = decltype(II)::value, d = 4 * c + i;
+                const uint32_t off = (a4 >> (8 * i)) & 0xFFu;
+                const uint32_t addr = lut + off + d * L::PB;
+                if constexpr (L::ENTRY == 1) {
+                    e[buf][cc * 4 + i][0] = *lds_ptr<lds_f1>(addr);
+                } else if constexpr (L::ENTRY == 2) {
+                    const lds_e2* p = lds_ptr<lds_e2>(addr);
+                    e[buf][cc * 4 + i][0] = p->x; e[buf][cc * 4 + i][1] = p->y;
+                } else {
+                    static_for<L::HALVES>([&](auto HH) {
+                        constexpr int h = decltype(HH)::value;
+                        const lds_e4* p = lds_ptr<lds_e4>(addr + h * L::HB);
+                        e[buf][cc * 4 + i][h * 4] = p->x; e[buf][cc * 4 + i][h * 4 + 1] = p->y;
+                        e[buf][cc * 4 + i][h * 4 + 2] = p->z; e[buf][cc * 4 + i][h * 4 + 3] = p->w;
+                    });
+                }
+            });
+        });
+    };
+    auto compute = [&](auto BI) {
+        constexpr int bi = decltype(BI)::value, buf = bi & 1;
+        static_for<BW>([&](auto CC) {
+            constexpr int cc = decltype(CC)::value, c = bi * BW + cc;
+            const uint32_t r4 = r4s[buf][cc];
+            static_for<4>([&](auto II) {
+                constexpr int i = decltype(II)::value;
+                const float t = static_cast<float>((r4 >> (8 * i)) & 0xFFu) + cds[4 * c + i];
+                static_for<REPP>([&](auto JJ) {
+                    constexpr int j = decltype(JJ)::value;
+                    acc[j] = __builtin_fmaf(e[buf][cc * 4 + i][j], t, acc[j]);
+                });
+            });
+        });
+    };
+    load(IC<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<NBATCH>([&](auto BI) {
+        constexpr int bi = decltype(BI)::value;
+        if constexpr (bi + 1 < NBATCH) load(IC<bi + 1>{});
+        compute(BI);
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+#pragma clang diagnostic pop
+
+// Broadcast the 64 per-pair c_d values (lane d holds c_d) into wave-uniform registers.
+__device__ __forceinline__ void broadcast_cd(float cdv, float (&cds)[kPairs]) {
+#pragma unroll
+    for (int d = 0; d < kPairs; d++) cds[d] = readlane_f(cdv, d);
+}
+
+}  // namespace pq

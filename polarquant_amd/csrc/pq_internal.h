@@ -1,0 +1,39 @@
+// Host-side launcher prototypes shared between the C-ABI translation unit and
+// the kernel translation units.  Each returns a hipError_t cast to int (0 = ok).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace pq {
+
+int launch_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
+                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, hipStream_t st);
+
+int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int Nk, int Nb, int rbits, int tbits,
+                    unsigned flags, uint8_t* codes, void* rscale, void* rmn, void* tscale, void* tmn,
+                    int cap, int off, hipStream_t st);
+
+struct AttnArgs {
+    const void* q;
+    const uint8_t* codes;
+    const void *rscale, *rmn, *tscale, *tmn;
+    int group_capacity, n_groups;
+    const int32_t* n_groups_per_seq;
+    const void* k_resid;
+    int resid_capacity, n_resid;
+    const int32_t* n_resid_per_seq;
+    const void* v;
+    int64_t v_capacity;
+    const uint8_t* mask;
+    int64_t mask_stride;
+    float sm_scale;
+    int B, N, Nk, tbits, dtype, n_splits;
+    float* workspace;
+    void* out;
+};
+int launch_attn(const AttnArgs& a, hipStream_t st);
+
+inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 : 8; }
+
+}  // namespace pq

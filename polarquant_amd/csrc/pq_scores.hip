@@ -1,0 +1,105 @@
+// Quantized-key decode scores: the HIP counterpart of the reference's Triton
+// score kernel (models/kernel4group.py:14-80).  One wavefront per
+// (batch, KV head, 128-token group); output fp32 [B,N,1,Nb*128].
+#include "pq_device.h"
+#include "pq_internal.h"
+
+namespace pq {
+
+template <typename T, int TB, int REPP>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) void scores_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
+                                                       const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
+                                                       const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
+                                                       float* __restrict__ out, int N, int Nk, int Nb, int rep) {
+    using L = Lut<TB, REPP>;
+    __shared__ __attribute__((aligned(16))) char lut_mem[L::BYTES];
+    const uint32_t lut = lds_addr(lut_mem);
+    const int lane = threadIdx.x;
+    const int grp = blockIdx.x;
+    const int bh = blockIdx.y;             // b*Nk + kvh
+    const int b = bh / Nk, kvh = bh - b * Nk;
+    const size_t gidx = static_cast<size_t>(bh) * Nb + grp;
+
+    // token codes of tile 0 and 1 (issued first: longest latency)
+    const uint4* crow = reinterpret_cast<const uint4*>(codes + gidx * (kGroup * kPairs));
+    uint4 cw[2][4];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) cw[t][i] = crow[(t * kWave + lane) * 4 + i];
+
+    float qx[REPP], qy[REPP];
+    const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) {
+        const bool ok = j < rep;
+        qx[j] = ok ? lo2f<T>(qb[j * kHeadDim + lane]) : 0.0f;
+        qy[j] = ok ? lo2f<T>(qb[j * kHeadDim + kPairs + lane]) : 0.0f;
+    }
+    const size_t mi = gidx * kPairs + lane;
+    const float cdv = build_lut<T, TB, REPP>(lut, lane, qx, qy, rscale[mi], rmn[mi], tscale[mi], tmn[mi]);
+    float cds[kPairs];
+    broadcast_cd(cdv, cds);
+    __syncthreads();
+
+    float* ob = out + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * (static_cast<size_t>(Nb) * kGroup) +
+                static_cast<size_t>(grp) * kGroup + lane;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        uint32_t cwords[16];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            cwords[4 * i + 0] = cw[t][i].x; cwords[4 * i + 1] = cw[t][i].y;
+            cwords[4 * i + 2] = cw[t][i].z; cwords[4 * i + 3] = cw[t][i].w;
+        }
+        float acc[REPP];
+#pragma unroll
+        for (int j = 0; j < REPP; j++) acc[j] = 0.0f;
+        score_token<TB, REPP>(lut, cwords, cds, acc);
+        // pin the sums: without this the optimizer sinks each head's FMAs into its
+        // "j < rep" store branch and keeps every table entry alive until then
+#pragma unroll
+        for (int j = 0; j < REPP; j++) asm volatile("" : "+v"(acc[j]));
+#pragma unroll
+        for (int j = 0; j < REPP; j++)
+            if (j < rep) ob[static_cast<size_t>(j) * Nb * kGroup + t * kWave] = acc[j];
+    }
+}
+
+template <typename T, int TB>
+static int launch_tb(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
+                     const void* tmn, float* out, int B, int N, int Nk, int Nb, hipStream_t st) {
+    const int rep = N / Nk;
+    dim3 grid(Nb, B * Nk), block(kWave);
+#define PQ_LAUNCH(REPP)                                                                                         \
+    hipLaunchKernelGGL((scores_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)q, codes,             \
+                       (const uint16_t*)rscale, (const uint16_t*)rmn, (const uint16_t*)tscale,                  \
+                       (const uint16_t*)tmn, out, N, Nk, Nb, rep)
+    switch (rep_pad(rep)) {
+        case 1: PQ_LAUNCH(1); break;
+        case 2: PQ_LAUNCH(2); break;
+        case 4: PQ_LAUNCH(4); break;
+        default: PQ_LAUNCH(8); break;
+    }
+#undef PQ_LAUNCH
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_t(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
+                    const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, hipStream_t st) {
+    switch (tbits) {
+        case 1: return launch_tb<T, 1>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
+        case 2: return launch_tb<T, 2>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
+        case 3: return launch_tb<T, 3>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
+        default: return launch_tb<T, 4>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
+    }
+}
+
+int launch_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
+                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, hipStream_t st) {
+    return dtype == 0 ? launch_t<F16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, st)
+                      : launch_t<BF16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, st);
+}
+
+}  // namespace pq

@@ -1,0 +1,120 @@
+"""Seeded synthetic workloads for the polar-key decode path.
+
+All tensors are generated on the CPU with a seeded torch.Generator so that a
+CPU checker and the GPU kernels see identical bits; callers move them to the
+GPU.  Keys follow the benchmark recipe: N(0,1) with 4 of the 128 channels
+scaled x8 (outliers), then HF rotate-half RoPE at positions 0..L-1, then cast
+to the model dtype.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+HEAD_DIM = 128
+GROUP = 128
+
+
+@dataclass
+class Shape:
+    name: str
+    batch: int
+    n_heads: int
+    n_kv_heads: int
+    context: int
+    rbits: int
+    tbits: int
+    rope_theta: float
+    seed: int
+    ragged: bool = False
+
+
+# index k == BASELINE configs[k] (config 4, the end-to-end model, has its own builder)
+CONFIGS = [
+    Shape("cfg0-llama2-7b-scores-b1-4k", 1, 32, 32, 4096, 4, 4, 1e4, 1000),
+    Shape("cfg1-llama3-8b-b16-32k", 16, 32, 8, 32768, 4, 4, 5e5, 1001),
+    Shape("cfg2-qwen2.5-7b-ragged-b64", 64, 28, 4, 8192, 3, 3, 1e6, 1002, ragged=True),
+    Shape("cfg3-llama3-8b-b1-128k", 1, 32, 8, 131072, 4, 4, 5e5, 1003),
+]
+
+
+def _rope_tables(L: int, theta: float, start: int = 0):
+    inv_freq = 1.0 / (theta ** (torch.arange(0, HEAD_DIM, 2, dtype=torch.float32) / HEAD_DIM))
+    pos = torch.arange(start, start + L, dtype=torch.float32)
+    ang = pos[:, None] * inv_freq[None, :]
+    emb = torch.cat([ang, ang], dim=-1)
+    return emb.cos(), emb.sin()
+
+
+def _rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    h = HEAD_DIM // 2
+    rot = torch.cat([-x[..., h:], x[..., :h]], dim=-1)
+    return x * cos + rot * sin
+
+
+def make_keys(B: int, Nk: int, L: int, theta: float, gen: torch.Generator, dtype=torch.float16,
+              chunk: int = 8192) -> torch.Tensor:
+    """Post-RoPE keys [B,Nk,L,128] in `dtype`, with 4 outlier channels x8."""
+    outliers = torch.randperm(HEAD_DIM, generator=gen)[:4]
+    out = torch.empty(B, Nk, L, HEAD_DIM, dtype=dtype)
+    for s in range(0, L, chunk):
+        n = min(chunk, L - s)
+        k = torch.randn(B, Nk, n, HEAD_DIM, generator=gen, dtype=torch.float32)
+        k[..., outliers] *= 8.0
+        cos, sin = _rope_tables(n, theta, s)
+        out[:, :, s:s + n] = _rope(k, cos, sin).to(dtype)
+    return out
+
+
+def make_half(shape, gen: torch.Generator, dtype=torch.float16, chunk_elems: int = 1 << 26) -> torch.Tensor:
+    """N(0,1) tensor in `dtype`, generated in bounded fp32 chunks."""
+    out = torch.empty(shape, dtype=dtype)
+    flat = out.view(-1)
+    for s in range(0, flat.numel(), chunk_elems):
+        n = min(chunk_elems, flat.numel() - s)
+        flat[s:s + n] = torch.randn(n, generator=gen, dtype=torch.float32).to(dtype)
+    return out
+
+
+def ragged_lengths(B: int, gen: torch.Generator, lo: int = 512, hi: int = 8192) -> torch.Tensor:
+    return torch.randint(lo, hi + 1, (B,), generator=gen)
+
+
+@dataclass
+class DecodeInputs:
+    shape: Shape
+    q: torch.Tensor                 # [B,N,1,128]
+    k: torch.Tensor                 # [B,Nk,L,128] post-RoPE keys (context)
+    v: torch.Tensor                 # [B,Nk,L,128]
+    lengths: Optional[torch.Tensor]  # [B] for ragged shapes
+
+
+def make_decode_inputs(shape: Shape, dtype=torch.float16, context: Optional[int] = None,
+                       batch: Optional[int] = None) -> DecodeInputs:
+    """Inputs of one decode step for `shape`; `context`/`batch` override the
+    full size (tests use reduced sizes of the same recipe and seed)."""
+    g = torch.Generator().manual_seed(shape.seed)
+    B = batch or shape.batch
+    L = context or shape.context
+    k = make_keys(B, shape.n_kv_heads, L, shape.rope_theta, g, dtype)
+    q = make_half((B, shape.n_heads, 1, HEAD_DIM), g, dtype)
+    v = make_half((B, shape.n_kv_heads, L, HEAD_DIM), g, dtype)
+    lengths = None
+    if shape.ragged:
+        lengths = ragged_lengths(B, g, min(512, L), L)
+    return DecodeInputs(shape, q, k, v, lengths)
+
+
+def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], resid_tokens: List[int],
+                      rbits: int = 4, tbits: int = 4, code_bytes_per_pair: float = 1.0) -> int:
+    """HBM bytes one fused decode-attention step must move: one byte per pair
+    code (the stored layout), 4 half metadata words per (group, pair), fp16 V
+    for every token, fp16 residual keys, plus q in / out."""
+    total = 0
+    for lq, res in zip(quant_tokens, resid_tokens):
+        total += n_kv_heads * (int(lq * 64 * code_bytes_per_pair) + (lq // GROUP) * 4 * 64 * 2
+                               + (lq + res) * HEAD_DIM * 2 + res * HEAD_DIM * 2)
+    total += 2 * len(quant_tokens) * n_heads * HEAD_DIM * 2
+    return total
