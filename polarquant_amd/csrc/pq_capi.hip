@@ -70,10 +70,47 @@ int pq_decode_scores(const void* q, const uint8_t* codes, const void* rscale, co
 
 }  // extern "C"
 
+extern "C" {
+
+int pq_validate_quantize_groups(const void* k, const int64_t* k_strides, int dtype,
+                                int B, int Nk, int Nb, int rbits, int tbits, unsigned flags,
+                                const uint8_t* codes, const void* rscale, const void* rmn,
+                                const void* tscale, const void* tmn,
+                                int out_group_capacity, int out_group_offset) {
+    if (!k || !k_strides || !codes || !rscale || !rmn || !tscale || !tmn) return PQ_ERR_NULL_POINTER;
+    if (B <= 0 || Nk <= 0 || Nb <= 0 || Nb > 65535 * 32 || static_cast<long long>(B) * Nk > 65535)
+        return PQ_ERR_BAD_SHAPE;
+    if (rbits < 1 || tbits < 1 || rbits + tbits > 8) return PQ_ERR_BAD_BITS;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32)) return PQ_ERR_BAD_SHAPE;
+    if (k_strides[3] != 1) return PQ_ERR_BAD_STRIDE;
+    if (k_strides[0] < 0 || k_strides[1] < 0 || k_strides[2] < PQ_HEAD_DIM) return PQ_ERR_BAD_STRIDE;
+    if (out_group_offset < 0 || out_group_capacity < out_group_offset + Nb) return PQ_ERR_BAD_STRIDE;
+    // 8-byte vector loads of 4 halves: base and every stride must keep that alignment
+    if (!aligned(k, 8) || (k_strides[0] & 3) || (k_strides[1] & 3) || (k_strides[2] & 3)) return PQ_ERR_MISALIGNED;
+    if (!aligned(codes, 4) || !aligned(rscale, 8) || !aligned(rmn, 8) || !aligned(tscale, 8) || !aligned(tmn, 8))
+        return PQ_ERR_MISALIGNED;
+    return PQ_OK;
+}
+
+int pq_quantize_groups(const void* k, const int64_t* k_strides, int dtype,
+                       int B, int Nk, int Nb, int rbits, int tbits, unsigned flags,
+                       uint8_t* codes, void* rscale, void* rmn, void* tscale, void* tmn,
+                       int out_group_capacity, int out_group_offset, void* stream) {
+    if (int rc = pq_validate_quantize_groups(k, k_strides, dtype, B, Nk, Nb, rbits, tbits, flags, codes, rscale, rmn,
+                                             tscale, tmn, out_group_capacity, out_group_offset))
+        return rc;
+    if (Nb > 65535 * 32) return PQ_ERR_BAD_SHAPE;
+    const int err = pq::launch_quantize(k, k_strides, dtype, B, Nk, Nb, rbits, tbits, flags, codes, rscale, rmn,
+                                        tscale, tmn, out_group_capacity, out_group_offset,
+                                        static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+}  // extern "C"
+
 // ---- TEMPORARY: remaining entry points are filled in next ----
 extern "C" {
-int pq_quantize_groups(const void*, const int64_t*, int, int, int, int, int, int, unsigned, uint8_t*, void*, void*, void*, void*, int, int, void*) { return PQ_ERR_LAUNCH; }
-int pq_validate_quantize_groups(const void*, const int64_t*, int, int, int, int, int, int, unsigned, const uint8_t*, const void*, const void*, const void*, const void*, int, int) { return PQ_ERR_LAUNCH; }
 int pq_decode_attn(const void*, const uint8_t*, const void*, const void*, const void*, const void*, int, int, const int32_t*, const void*, int, int, const int32_t*, const void*, int64_t, const uint8_t*, int64_t, float, int, int, int, int, int, int, int, void*, size_t, void*, void*) { return PQ_ERR_LAUNCH; }
 int pq_validate_decode_attn(const void*, const uint8_t*, const void*, const void*, const void*, const void*, int, int, const int32_t*, const void*, int, int, const int32_t*, const void*, int64_t, const uint8_t*, int64_t, float, int, int, int, int, int, int, int, const void*, size_t, const void*) { return PQ_ERR_LAUNCH; }
 int pq_decode_attn_plan(int, int, int, int) { return 1; }

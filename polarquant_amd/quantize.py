@@ -1,0 +1,55 @@
+"""Polar quantizer: HIP counterpart of `quantize_and_pack_nbit`
+(reference: models/modeling_llama_polar.py:135-157)."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _ffi
+from .kernel4group import _dtype_code, _stream_ptr
+
+GROUP = 128
+PAIRS = 64
+
+
+def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4, group_size: int = GROUP,
+                           wrap_fp32: bool = False,
+                           out: Optional[Tuple[torch.Tensor, ...]] = None, group_offset: int = 0):
+    """key_states [B,Nk,L,128] half/bf16 on the GPU (any batch/head/token strides, unit dim stride)
+    -> (indices u8 [B,Nk,Nb,128,64], rscale, rmn, tscale, tmn [B,Nk,Nb,1,64]).
+
+    `out`, if given, is a 5-tuple of pre-allocated cache tensors
+    ([B,Nk,cap,128,64] u8 and four [B,Nk,cap,1,64]) that receive the Nb new groups
+    at group index `group_offset`; nothing is allocated then.
+    """
+    if not key_states.is_cuda:
+        raise RuntimeError("polarquant_amd: the quantizer needs tensors on the GPU (no CPU fallback)")
+    B, Nk, L, D2 = key_states.shape
+    assert D2 == 2 * PAIRS and group_size == GROUP, "head_dim 128 and group size 128 only"
+    assert L % GROUP == 0 and rbits + tbits <= 8
+    Nb = L // GROUP
+    dt = _dtype_code(key_states)
+    if key_states.stride(3) != 1 or any(s % 4 for s in key_states.stride()[:3]) or key_states.data_ptr() % 8:
+        key_states = key_states.contiguous()
+    dev = key_states.device
+    if out is None:
+        codes = torch.empty((B, Nk, Nb, GROUP, PAIRS), dtype=torch.uint8, device=dev)
+        meta = [torch.empty((B, Nk, Nb, 1, PAIRS), dtype=key_states.dtype, device=dev) for _ in range(4)]
+        cap, off = Nb, 0
+    else:
+        codes, meta = out[0], list(out[1:])
+        cap, off = codes.shape[2], group_offset
+        assert codes.is_contiguous() and all(m.is_contiguous() for m in meta)
+    strides = (ctypes.c_int64 * 4)(*key_states.stride())
+    with torch.cuda.device(dev):
+        rc = _ffi.lib().pq_quantize_groups(key_states.data_ptr(), ctypes.cast(strides, ctypes.c_void_p), dt, B, Nk, Nb,
+                                           rbits, tbits, _ffi.PQ_WRAP_FP32 if wrap_fp32 else 0,
+                                           codes.data_ptr(), *[m.data_ptr() for m in meta], cap, off,
+                                           _stream_ptr(dev))
+    _ffi.check(rc, "pq_quantize_groups")
+    if out is None:
+        return (codes, *meta)
+    sl = slice(off, off + Nb)
+    return (codes[:, :, sl], *[m[:, :, sl] for m in meta])

@@ -1,0 +1,116 @@
+"""GPU parity of pq_quantize_groups (through the C ABI) against the CPU oracle.
+
+Bar: packed codes and the four metadata tensors bit-exact.  Any disagreement
+is an "edge flip"; flips are counted and the target (asserted) is 0.
+"""
+import pytest
+import torch
+
+from oracle import polar_oracle as po
+from polarquant_amd import workloads as wl
+from polarquant_amd.quantize import quantize_and_pack_nbit
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["codes", "rscale", "rmn", "tscale", "tmn"]
+
+
+def _bits(t):
+    return t if t.dtype == torch.uint8 else t.view(torch.int16)
+
+
+def count_flips(got, ref):
+    """-> dict name -> number of differing elements (metadata compared by value so that -0.0 == +0.0)."""
+    out = {}
+    for n, g, r in zip(NAMES, got, ref):
+        g = g.cpu()
+        if g.dtype == torch.uint8:
+            out[n] = int((g != r).sum())
+        else:
+            out[n] = int(((g.float() != r.float()) & ~(g.float().isnan() & r.float().isnan())).sum())
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (2, 4), (5, 3), (4, 2)])
+def test_quantize_bit_exact(gpu, dtype, rbits, tbits):
+    print("case", dtype, rbits, tbits, flush=True)
+    g = torch.Generator().manual_seed(21)
+    k = wl.make_keys(2, 4, 1024, 5e5, g, dtype)
+    ref = po.quantize_and_pack_nbit(k, rbits, tbits)
+    got = quantize_and_pack_nbit(k.to(gpu), rbits, tbits)
+    torch.cuda.synchronize()
+    assert [tuple(t.shape) for t in got] == [tuple(t.shape) for t in ref]
+    flips = count_flips(got, ref)
+    print("flips", flips, flush=True)
+    assert all(v == 0 for v in flips.values()), flips
+
+
+def test_quantize_cfg0_full_flip_count(gpu):
+    """BASELINE configs[0] keys: [1,32,4096,128] fp16, RoPE theta 1e4, 4/4 bits."""
+    sh = wl.CONFIGS[0]
+    inp = wl.make_decode_inputs(sh)
+    ref = po.quantize_and_pack_nbit(inp.k, 4, 4)
+    got = quantize_and_pack_nbit(inp.k.to(gpu), 4, 4)
+    flips = count_flips(got, ref)
+    print("cfg0 flips", flips, "of", ref[0].numel(), "codes", flush=True)
+    assert all(v == 0 for v in flips.values()), flips
+
+
+def test_quantize_strided_transposed_view(gpu):
+    """Keys arrive as a transposed view of the [B,L,Nk,128] projection output
+    (modeling_llama_polar.py:54); the kernel reads them in place."""
+    g = torch.Generator().manual_seed(5)
+    B, Nk, L = 2, 4, 256
+    k_blhd = wl.make_half((B, L, Nk, 128), g)
+    k = k_blhd.transpose(1, 2)
+    ref = po.quantize_and_pack_nbit(k.contiguous(), 4, 4)
+    kd = k_blhd.to(gpu).transpose(1, 2)
+    assert not kd.is_contiguous()
+    got = quantize_and_pack_nbit(kd, 4, 4)
+    assert all(v == 0 for v in count_flips(got, ref).values())
+
+
+def test_quantize_into_cache_slot(gpu):
+    """Quantize-on-append writes one group into a pre-allocated cache at a group offset."""
+    g = torch.Generator().manual_seed(6)
+    B, Nk, cap = 2, 2, 5
+    k = wl.make_keys(B, Nk, 256, 1e4, g)
+    ref = po.quantize_and_pack_nbit(k, 4, 4)
+    codes = torch.zeros(B, Nk, cap, 128, 64, dtype=torch.uint8, device=gpu)
+    meta = [torch.zeros(B, Nk, cap, 1, 64, dtype=torch.float16, device=gpu) for _ in range(4)]
+    got = quantize_and_pack_nbit(k.to(gpu), 4, 4, out=(codes, *meta), group_offset=2)
+    assert all(v == 0 for v in count_flips(got, ref).values())
+    assert int(codes[:, :, :2].sum()) == 0 and int(codes[:, :, 4:].sum()) == 0
+    assert torch.equal(codes[:, :, 2:4].cpu(), ref[0])
+
+
+def test_quantize_special_values(gpu):
+    """Zeros, axis-aligned keys, constant groups (scale == 0 -> code 0), negative zero, tiny and huge values."""
+    g = torch.Generator().manual_seed(9)
+    k = wl.make_half((1, 2, 256, 128), g)
+    k[0, 0, :128, :8] = 0.0                      # x == 0 for pairs 0..7 in group 0
+    k[0, 0, :128, 64 + 8:64 + 16] = 0.0          # y == 0 for pairs 8..15
+    k[0, 0, :128, 16] = 1.5; k[0, 0, :128, 64 + 16] = -2.0   # constant pair -> both scales 0
+    k[0, 0, :128, 17] = 0.0; k[0, 0, :128, 64 + 17] = 0.0    # origin
+    k[0, 1, :128, 18] = -0.0
+    k[0, 1, 5, 19] = 6.0e-8; k[0, 1, 6, 64 + 19] = -6.0e-8    # subnormal halves
+    k[0, 1, 7, 20] = 60000.0; k[0, 1, 8, 64 + 20] = -60000.0
+    ref = po.quantize_and_pack_nbit(k, 4, 4)
+    got = quantize_and_pack_nbit(k.to(gpu), 4, 4)
+    flips = count_flips(got, ref)
+    assert all(v == 0 for v in flips.values()), flips
+
+
+def test_quantize_wrap_fp32_flag(gpu):
+    """PQ_WRAP_FP32 adds 2*pi in fp32 (what an eager GPU add of a half tensor and a
+    python float does); checked against the plain-C oracle's same switch."""
+    from oracle import c_oracle as co
+    g = torch.Generator().manual_seed(2)
+    k = wl.make_keys(1, 2, 512, 1e4, g)
+    ref = co.quantize(k, 4, 4, wrap_fp32=True)
+    got = quantize_and_pack_nbit(k.to(gpu), 4, 4, wrap_fp32=True)
+    flips = count_flips(got, ref)
+    # libm atan2f (C oracle) vs the SLEEF restatement may differ in the last ulp: allow a handful, report them
+    print("wrap_fp32 flips vs C oracle", flips, flush=True)
+    assert flips["codes"] <= 4 and flips["rscale"] == 0 and flips["rmn"] == 0
