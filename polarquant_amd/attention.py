@@ -1,0 +1,99 @@
+"""Fused polar-key decode attention (HIP) behind a torch-tensor interface.
+
+`polar_decode_attention` computes what the decode branch of the reference's
+LlamaPolarGroupAttention.forward computes between RoPE and o_proj
+(models/modeling_llama_polar.py:66-99), in one pass over HBM.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _ffi
+from .kernel4group import _dtype_code, _stream_ptr
+
+GROUP = 128
+_WORKSPACES = {}
+
+
+def _num_cus(device: torch.device) -> int:
+    return torch.cuda.get_device_properties(device).multi_processor_count
+
+
+def plan_splits(B: int, Nk: int, max_groups: int, device: torch.device) -> int:
+    return _ffi.lib().pq_decode_attn_plan(B, Nk, max(max_groups, 1), _num_cus(device))
+
+
+def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
+    """A cached fp32 workspace for the split-K partials (grown on demand, one per device)."""
+    need = _ffi.lib().pq_decode_attn_workspace_bytes(B, N, n_splits)
+    key = (device.type, device.index)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() * 4 < need:
+        ws = torch.empty((need + 3) // 4, dtype=torch.float32, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def polar_decode_attention(
+    query_states: torch.Tensor,               # [B,N,1,128] or [B,N,128]
+    indices: Optional[torch.Tensor],          # [B,Nk,cap,128,64] u8 (cap >= used groups) or None
+    rscale: Optional[torch.Tensor], rmn: Optional[torch.Tensor],
+    tscale: Optional[torch.Tensor], tmn: Optional[torch.Tensor],   # [B,Nk,cap,1,64]
+    key_resid: Optional[torch.Tensor],        # [B,Nk,res_cap,128] fp16 keys not yet quantized (new key included)
+    value_states: torch.Tensor,               # [B,Nk,v_cap,128]; rows [0, n_groups*128 + n_resid) are used
+    n_groups: int, n_resid: int,
+    attention_mask: Optional[torch.Tensor] = None,   # [B, >= n_groups*128 + n_resid] of {0,1}
+    rbits: int = 4, tbits: int = 4, sm_scale: Optional[float] = None,
+    n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
+    n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """-> attention output [B,N,1,128] in the query dtype."""
+    if not query_states.is_cuda:
+        raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
+    dev = query_states.device
+    B, N = query_states.shape[:2]
+    hd = query_states.shape[-1]
+    Nk = value_states.shape[1]
+    assert hd == 128
+    dt = _dtype_code(query_states)
+    q = query_states.reshape(B, N, hd)
+    if not q.is_contiguous():
+        q = q.contiguous()
+    assert value_states.is_contiguous() and value_states.dtype == query_states.dtype
+    v_cap = value_states.shape[2]
+    if indices is not None:
+        assert indices.is_contiguous() and all(m.is_contiguous() for m in (rscale, rmn, tscale, tmn))
+        g_cap = indices.shape[2]
+        cptr = [indices.data_ptr(), rscale.data_ptr(), rmn.data_ptr(), tscale.data_ptr(), tmn.data_ptr()]
+    else:
+        g_cap, cptr = 0, [None] * 5
+    if key_resid is not None:
+        assert key_resid.is_contiguous() and key_resid.dtype == query_states.dtype
+        r_cap, kptr = key_resid.shape[2], key_resid.data_ptr()
+    else:
+        r_cap, kptr = 0, None
+    mptr, mstride = None, 0
+    if attention_mask is not None:
+        m8 = attention_mask if attention_mask.dtype == torch.uint8 else (attention_mask != 0).to(torch.uint8)
+        m8 = m8.contiguous()
+        mptr, mstride = m8.data_ptr(), m8.stride(0)
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(hd)
+    max_groups = g_cap if n_groups_per_seq is not None else n_groups
+    if n_splits is None:
+        n_splits = plan_splits(B, Nk, max_groups, dev)
+    ws = workspace_for(B, N, n_splits, dev)
+    if out is None:
+        out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
+    gps = n_groups_per_seq.data_ptr() if n_groups_per_seq is not None else None
+    rps = n_resid_per_seq.data_ptr() if n_resid_per_seq is not None else None
+    with torch.cuda.device(dev):
+        rc = _ffi.lib().pq_decode_attn(
+            q.data_ptr(), *cptr, g_cap, n_groups, gps, kptr, r_cap, n_resid, rps,
+            value_states.data_ptr(), v_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
+            n_splits, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
+    _ffi.check(rc, "pq_decode_attn")
+    return out

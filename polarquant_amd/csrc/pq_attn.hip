@@ -1,0 +1,384 @@
+// Fused polar-key decode attention: quantized-key scores, fp16 residual-key
+// scores, 1/sqrt(d), mask, softmax and P.V in one pass over HBM
+// (reference decode branch: models/modeling_llama_polar.py:66-99), split over
+// the context, followed by a small merge kernel.
+//
+// attn_kernel: grid (n_splits + 1, B*Nk), one wavefront per block.
+//   block x <  n_splits : the x-th slice of the sequence's quantized groups
+//   block x == n_splits : the fp16 residual keys (0..128 tokens)
+// Each wavefront walks its tokens in 64-token tiles, lane == token, and keeps
+// flash-style running state (m, l, acc) for the `rep` query heads of its KV
+// head.  P.V runs on the matrix cores: for 16 tokens at a time
+//     D[dim][head] += V^T[dim][token] * P[token][head]
+// with v_mfma_f32_16x16x16 (f16 or bf16), heads padded to the 16 columns.
+// The V operand is built from plain 16-byte row loads (lane (g,n) loads dims
+// 8n..8n+7 of tokens 4g..4g+3) by a 4x4 in-register transpose with v_perm_b32;
+// P goes through a 1 KiB LDS staging buffer.
+// The running maximum m is only raised when a score exceeds it by more than
+// kLazyThreshold (in log2 units): probabilities stay below 2^8, and the
+// 32-register rescale of the accumulators is skipped on almost every tile.
+//
+// merge_kernel: grid B*N, 128 threads (one per output dim): combines the
+// n_splits + 1 partials (m, l, acc[128]) of a query head and writes half words.
+#include "pq_device.h"
+#include "pq_internal.h"
+
+namespace pq {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLazyThreshold = 8.0f;
+constexpr int kPartialFloats = 132;   // m, l, pad, pad, acc[128]
+constexpr float kLog2e = 1.44269504088896340736f;
+
+template <typename T> __device__ __forceinline__ floatx4 mfma16(uint2 a, uint2 b, floatx4 c);
+template <> __device__ __forceinline__ floatx4 mfma16<F16>(uint2 a, uint2 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ floatx4 mfma16<BF16>(uint2 a, uint2 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+template <int REPP>
+struct AttnState {
+    float m[REPP];        // running maximum (log2 units), wave-uniform
+    float l[REPP];        // per-lane partial sum of probabilities
+    floatx4 acc[8];       // lane (g,n): acc[e][i] = out_head_n[dim 8*(4g+i)+e]
+};
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wint-to-pointer-cast"
+
+// Softmax update and P.V for one 64-token tile.
+//   t[j]   scaled score (log2 units) of this lane's token for head j; -inf = masked/invalid
+//   vv     this lane's V operand loads: vv[tb][i] = dims 8n..8n+7 of token 16*tb + 4*g + i
+//   pbuf   LDS address of the [REPP][64] 16-bit staging buffer
+template <typename T, int REPP>
+__device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[REPP], const uint4 (&vv)[4][4],
+                                                uint32_t pbuf, int lane) {
+    bool raise = false;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) raise |= t[j] > st.m[j] + kLazyThreshold;
+    if (__any(raise)) {
+        float alpha[REPP];
+#pragma unroll
+        for (int j = 0; j < REPP; j++) {
+            const float mn = fmaxf(st.m[j], wave_max(t[j]));
+            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2f(st.m[j] - mn);
+            st.m[j] = mn;
+            st.l[j] *= alpha[j];
+        }
+        float a = alpha[0];
+#pragma unroll
+        for (int j = 1; j < REPP; j++) a = ((lane & 15) == j) ? alpha[j] : a;
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.acc[e] *= a;
+    }
+#pragma unroll
+    for (int j = 0; j < REPP; j++) {
+        const float ms = (st.m[j] == -INFINITY) ? 0.0f : st.m[j];
+        const float p = exp2f(t[j] - ms);
+        st.l[j] += p;
+        *lds_ptr<__attribute__((address_space(3))) uint16_t>(pbuf + (j * kWave + lane) * 2) = f2lo<T>(p);
+    }
+    asm volatile("" ::: "memory");
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t prow = pbuf + ((n & (REPP - 1)) * kWave + 4 * g) * 2;
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) {
+        const __attribute__((address_space(3))) uint2* pp = lds_ptr<__attribute__((address_space(3))) uint2>(prow + tb * 32);
+        uint2 pb;
+        pb.x = pp->x; pb.y = pp->y;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+            auto word = [&](const uint4& v) { return (e >> 1) == 0 ? v.x : (e >> 1) == 1 ? v.y : (e >> 1) == 2 ? v.z : v.w; };
+            uint2 va;
+            va.x = __builtin_amdgcn_perm(word(vv[tb][1]), word(vv[tb][0]), sel);
+            va.y = __builtin_amdgcn_perm(word(vv[tb][3]), word(vv[tb][2]), sel);
+            st.acc[e] = mfma16<T>(va, pb, st.acc[e]);
+        }
+    }
+    asm volatile("" ::: "memory");
+    // keep the next tile's loads behind this tile's matrix work: hoisting them
+    // here would double the registers held by V operands
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Hot-loop loads go through buffer resources: the address is a wave-uniform
+// base held in scalar registers plus one fixed 32-bit lane offset plus a scalar
+// offset that carries the loop position, so no per-lane 64-bit pointer has to
+// be kept or advanced, and rows past the end of a tensor read as zero instead
+// of faulting (which is what the partly filled residual tile relies on).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(voff), static_cast<int>(soff), 0);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// Issue the V operand loads of the 64-token tile that starts at byte offset
+// `tile_off` of the (batch, KV head) plane: lane (g,n) loads dims 8n..8n+7 of
+// tokens 16*tb + 4*g + i.  voff = g*1024 + n*16.
+__device__ __forceinline__ void load_v_tile(uint4 (&vv)[4][4], __amdgpu_buffer_rsrc_t rv, uint32_t voff, uint32_t tile_off) {
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            vv[tb][i] = buf_load16(rv, voff, tile_off + static_cast<uint32_t>((16 * tb + i) * kHeadDim * 2));
+}
+
+template <typename T, int TB, int REPP>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 3)))
+void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
+                 const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
+                 const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
+                 int group_capacity, int n_groups, const int32_t* __restrict__ n_groups_per_seq,
+                 const uint16_t* __restrict__ k_resid, int resid_capacity, int n_resid,
+                 const int32_t* __restrict__ n_resid_per_seq,
+                 const uint16_t* __restrict__ v, int64_t v_capacity,
+                 const uint8_t* __restrict__ mask, int64_t mask_stride,
+                 float scale_log2, int N, int Nk, int rep, int n_splits, float* __restrict__ ws) {
+    using L = Lut<TB, REPP>;
+    // the table region doubles as the fp32 query buffer of the residual block
+    constexpr int kLutBytes = L::BYTES > REPP * kHeadDim * 4 ? L::BYTES : REPP * kHeadDim * 4;
+    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
+    const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
+
+    const int lane = threadIdx.x;
+    const int split = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / Nk, kvh = bh - b * Nk;
+
+    int nb = n_groups_per_seq ? n_groups_per_seq[b] : n_groups;
+    nb = nb < 0 ? 0 : (nb > group_capacity ? group_capacity : nb);
+    int nres = n_resid_per_seq ? n_resid_per_seq[b] : n_resid;
+    nres = nres < 0 ? 0 : (nres > resid_capacity ? resid_capacity : nres);
+    int64_t n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
+    n_tokens = n_tokens > v_capacity ? v_capacity : n_tokens;   // never read past the (batch, head) plane of V
+
+    const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
+                                                static_cast<uint32_t>(n_tokens * (kHeadDim * 2)));
+    const uint32_t voff_v = static_cast<uint32_t>(lane >> 4) * (4 * kHeadDim * 2) + static_cast<uint32_t>(lane & 15) * 16;
+    const bool has_mask = mask != nullptr;
+    const __amdgpu_buffer_rsrc_t rm = make_rsrc(has_mask ? mask + static_cast<size_t>(b) * mask_stride : nullptr,
+                                                has_mask ? static_cast<uint32_t>(n_tokens < mask_stride ? n_tokens : mask_stride) : 0u);
+
+    AttnState<REPP> st;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) { st.m[j] = -INFINITY; st.l[j] = 0.0f; }
+#pragma unroll
+    for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    if (split < n_splits) {
+        // ---------------- quantized groups [g0, g1) ----------------
+        const int gps = (nb + n_splits - 1) / n_splits;
+        const int g0 = split * gps;
+        const int g1 = (g0 + gps) < nb ? (g0 + gps) : nb;
+        if (g0 < g1) {
+            float qx[REPP], qy[REPP];
+#pragma unroll
+            for (int j = 0; j < REPP; j++) {
+                const bool ok = j < rep;
+                qx[j] = ok ? lo2f<T>(qb[j * kHeadDim + lane]) : 0.0f;
+                qy[j] = ok ? lo2f<T>(qb[j * kHeadDim + kPairs + lane]) : 0.0f;
+            }
+            const size_t plane = static_cast<size_t>(bh) * group_capacity;
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(codes + plane * (kGroup * kPairs),
+                                                        static_cast<uint32_t>(nb) * (kGroup * kPairs));
+            const uint32_t voff_c = static_cast<uint32_t>(lane) * kPairs;
+            // software pipeline: codes of the next tile and metadata of the next group are in flight
+            uint4 cnext[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(g0) * (kGroup * kPairs) + 16 * i);
+            const uint16_t* prs = rscale + plane * kPairs + lane;
+            const uint16_t* prm = rmn + plane * kPairs + lane;
+            const uint16_t* pts = tscale + plane * kPairs + lane;
+            const uint16_t* ptm = tmn + plane * kPairs + lane;
+            uint16_t mrs = prs[g0 * kPairs], mrm = prm[g0 * kPairs], mts = pts[g0 * kPairs], mtm = ptm[g0 * kPairs];
+            for (int grp = g0; grp < g1; grp++) {
+                asm volatile("" ::: "memory");
+                const float cdv = build_lut<T, TB, REPP>(lut, lane, qx, qy, mrs, mrm, mts, mtm);
+                float cds[kPairs];
+                broadcast_cd(cdv, cds);
+                asm volatile("" ::: "memory");
+                if (grp + 1 < g1) {
+                    const int o = (grp + 1) * kPairs;
+                    mrs = prs[o]; mrm = prm[o]; mts = pts[o]; mtm = ptm[o];
+                }
+#pragma unroll
+                for (int half = 0; half < 2; half++) {
+                    const int tt = 2 * grp + half;
+                    const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
+                    uint4 vv[4][4];
+                    load_v_tile(vv, rv, voff_v, tok0 * (kHeadDim * 2));
+                    uint32_t cw[16];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        cw[4 * i] = cnext[i].x; cw[4 * i + 1] = cnext[i].y; cw[4 * i + 2] = cnext[i].z; cw[4 * i + 3] = cnext[i].w;
+                    }
+                    if (half == 0 || grp + 1 < g1) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++)
+                            cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(tt + 1) * (kWave * kPairs) + 16 * i);
+                    }
+                    float s[REPP];
+#pragma unroll
+                    for (int j = 0; j < REPP; j++) s[j] = 0.0f;
+                    score_token<TB, REPP>(lut, cw, cds, s);
+                    const bool keep = has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(tok0), 0) != 0) : true;
+#pragma unroll
+                    for (int j = 0; j < REPP; j++) s[j] = keep ? s[j] * scale_log2 : -INFINITY;
+                    softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
+                }
+            }
+        }
+    } else if (nres > 0) {
+        // ---------------- fp16 residual keys ----------------
+        // q as fp32 in LDS: [REPP][128]
+#pragma unroll
+        for (int j = 0; j < REPP; j++) {
+            const bool ok = j < rep;
+            *lds_ptr<lds_f1>(lut + (j * kHeadDim + lane) * 4) = ok ? lo2f<T>(qb[j * kHeadDim + lane]) : 0.0f;
+            *lds_ptr<lds_f1>(lut + (j * kHeadDim + kWave + lane) * 4) = ok ? lo2f<T>(qb[j * kHeadDim + kWave + lane]) : 0.0f;
+        }
+        asm volatile("" ::: "memory");
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
+                                                    static_cast<uint32_t>(nres) * (kHeadDim * 2));
+        const int n_tiles = (nres + kWave - 1) / kWave;
+        for (int tt = 0; tt < n_tiles; tt++) {
+            const int tok = tt * kWave + lane;
+            const bool valid = tok < nres;
+            const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
+            uint4 vv[4][4];
+            load_v_tile(vv, rv, voff_v, arow * (kHeadDim * 2));
+            float s[REPP];
+#pragma unroll
+            for (int j = 0; j < REPP; j++) s[j] = 0.0f;
+#pragma unroll 4
+            for (int c = 0; c < 16; c++) {
+                const uint4 kw = buf_load16(rk, static_cast<uint32_t>(tok) * (kHeadDim * 2), 16 * c);
+                const uint32_t w[4] = {kw.x, kw.y, kw.z, kw.w};
+                float kf[8];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    kf[2 * i] = lo2f<T>(static_cast<uint16_t>(w[i] & 0xffffu));
+                    kf[2 * i + 1] = lo2f<T>(static_cast<uint16_t>(w[i] >> 16));
+                }
+#pragma unroll
+                for (int j = 0; j < REPP; j++) {
+                    const lds_e4* qa = lds_ptr<lds_e4>(lut + (j * kHeadDim + 8 * c) * 4);
+                    const lds_e4* qc = lds_ptr<lds_e4>(lut + (j * kHeadDim + 8 * c + 4) * 4);
+                    s[j] = __builtin_fmaf(qa->x, kf[0], s[j]); s[j] = __builtin_fmaf(qa->y, kf[1], s[j]);
+                    s[j] = __builtin_fmaf(qa->z, kf[2], s[j]); s[j] = __builtin_fmaf(qa->w, kf[3], s[j]);
+                    s[j] = __builtin_fmaf(qc->x, kf[4], s[j]); s[j] = __builtin_fmaf(qc->y, kf[5], s[j]);
+                    s[j] = __builtin_fmaf(qc->z, kf[6], s[j]); s[j] = __builtin_fmaf(qc->w, kf[7], s[j]);
+                }
+            }
+            const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(arow), 0) != 0) : true);
+#pragma unroll
+            for (int j = 0; j < REPP; j++) {
+                // the reference multiplies q.K^T in the model dtype before promoting (:79)
+                const float sr = lo2f<T>(f2lo<T>(s[j]));
+                s[j] = keep ? sr * scale_log2 : -INFINITY;
+            }
+            softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
+        }
+    }
+
+    // ---------------- write the partial ----------------
+    float lsum[REPP];
+#pragma unroll
+    for (int j = 0; j < REPP; j++) lsum[j] = wave_sum(st.l[j]);
+    const int g = lane >> 4, n = lane & 15;
+    if (n < rep) {
+        float mm = st.m[0], ll = lsum[0];
+#pragma unroll
+        for (int j = 1; j < REPP; j++) { mm = (n == j) ? st.m[j] : mm; ll = (n == j) ? lsum[j] : ll; }
+        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * (n_splits + 1) + split) * kPartialFloats;
+        if (g == 0) { pw[0] = mm; pw[1] = ll; }
+        float* pa = pw + 4 + 32 * g;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *reinterpret_cast<float4*>(pa + 8 * i) = make_float4(st.acc[0][i], st.acc[1][i], st.acc[2][i], st.acc[3][i]);
+            *reinterpret_cast<float4*>(pa + 8 * i + 4) = make_float4(st.acc[4][i], st.acc[5][i], st.acc[6][i], st.acc[7][i]);
+        }
+    }
+}
+#pragma clang diagnostic pop
+
+template <typename T>
+__global__ __launch_bounds__(kHeadDim) void merge_kernel(const float* __restrict__ ws, int n_part, uint16_t* __restrict__ out) {
+    const int bn = blockIdx.x, d = threadIdx.x;
+    const float* p = ws + static_cast<size_t>(bn) * n_part * kPartialFloats;
+    float M = -INFINITY;
+    for (int s = 0; s < n_part; s++) M = fmaxf(M, p[s * kPartialFloats]);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < n_part; s++) {
+        const float m = p[s * kPartialFloats];
+        if (m == -INFINITY) continue;
+        const float w = exp2f(m - M);
+        den = __builtin_fmaf(w, p[s * kPartialFloats + 1], den);
+        num = __builtin_fmaf(w, p[s * kPartialFloats + 4 + d], num);
+    }
+    out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : 0.0f);
+}
+
+template <typename T, int TB>
+static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
+    const int rep = a.N / a.Nk;
+    dim3 grid(a.n_splits + 1, a.B * a.Nk), block(kWave);
+    const float scale_log2 = a.sm_scale * kLog2e;
+#define PQ_LAUNCH(REPP)                                                                                              \
+    hipLaunchKernelGGL((attn_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,                \
+                       (const uint16_t*)a.rscale, (const uint16_t*)a.rmn, (const uint16_t*)a.tscale,                 \
+                       (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
+                       (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
+                       (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.N, a.Nk, rep,        \
+                       a.n_splits, a.workspace)
+    switch (rep_pad(rep)) {
+        case 1: PQ_LAUNCH(1); break;
+        case 2: PQ_LAUNCH(2); break;
+        case 4: PQ_LAUNCH(4); break;
+        default: PQ_LAUNCH(8); break;
+    }
+#undef PQ_LAUNCH
+    int err = static_cast<int>(hipGetLastError());
+    if (err) return err;
+    hipLaunchKernelGGL(merge_kernel<T>, dim3(a.B * a.N), dim3(kHeadDim), 0, st, a.workspace, a.n_splits + 1,
+                       (uint16_t*)a.out);
+    return static_cast<int>(hipGetLastError());
+}
+
+template <typename T>
+static int launch_attn_t(const AttnArgs& a, hipStream_t st) {
+    switch (a.tbits) {
+        case 1: return launch_attn_tb<T, 1>(a, st);
+        case 2: return launch_attn_tb<T, 2>(a, st);
+        case 3: return launch_attn_tb<T, 3>(a, st);
+        default: return launch_attn_tb<T, 4>(a, st);
+    }
+}
+
+int launch_attn(const AttnArgs& a, hipStream_t st) {
+    return a.dtype == 0 ? launch_attn_t<F16>(a, st) : launch_attn_t<BF16>(a, st);
+}
+
+}  // namespace pq

@@ -109,10 +109,88 @@ int pq_quantize_groups(const void* k, const int64_t* k_strides, int dtype,
 
 }  // extern "C"
 
-// ---- TEMPORARY: remaining entry points are filled in next ----
 extern "C" {
-int pq_decode_attn(const void*, const uint8_t*, const void*, const void*, const void*, const void*, int, int, const int32_t*, const void*, int, int, const int32_t*, const void*, int64_t, const uint8_t*, int64_t, float, int, int, int, int, int, int, int, void*, size_t, void*, void*) { return PQ_ERR_LAUNCH; }
-int pq_validate_decode_attn(const void*, const uint8_t*, const void*, const void*, const void*, const void*, int, int, const int32_t*, const void*, int, int, const int32_t*, const void*, int64_t, const uint8_t*, int64_t, float, int, int, int, int, int, int, int, const void*, size_t, const void*) { return PQ_ERR_LAUNCH; }
-int pq_decode_attn_plan(int, int, int, int) { return 1; }
-size_t pq_decode_attn_workspace_bytes(int, int, int) { return 0; }
+
+int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus) {
+    if (B <= 0 || Nk <= 0 || max_groups <= 0) return 1;
+    if (n_cus <= 0) n_cus = 256;
+    // one wavefront per (batch, KV head, split); about 8 fit a CU next to their lookup tables.
+    // Aim for one resident wavefront per slot so that all slices run concurrently and finish together.
+    const long long slots = static_cast<long long>(n_cus) * 8;
+    long long n = slots / (static_cast<long long>(B) * Nk);
+    if (n < 1) n = 1;
+    if (n > max_groups) n = max_groups;
+    if (n > 65534) n = 65534;
+    return static_cast<int>(n);
 }
+
+size_t pq_decode_attn_workspace_bytes(int B, int N, int n_splits) {
+    if (B <= 0 || N <= 0 || n_splits <= 0) return 0;
+    return static_cast<size_t>(B) * N * (static_cast<size_t>(n_splits) + 1) * PQ_PARTIAL_FLOATS * sizeof(float);
+}
+
+int pq_validate_decode_attn(const void* q,
+                            const uint8_t* codes, const void* rscale, const void* rmn,
+                            const void* tscale, const void* tmn, int group_capacity,
+                            int n_groups, const int32_t* n_groups_per_seq,
+                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                            const void* v, int64_t v_capacity,
+                            const uint8_t* mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, const void* workspace, size_t workspace_bytes,
+                            const void* out) {
+    if (!q || !v || !workspace || !out) return PQ_ERR_NULL_POINTER;
+    if (int rc = check_heads(B, N, Nk)) return rc;
+    if (static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
+    if (int rc = check_bits(rbits, tbits)) return rc;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (group_capacity < 0 || resid_capacity < 0 || n_groups < 0 || n_resid < 0 || v_capacity <= 0)
+        return PQ_ERR_BAD_STRIDE;
+    const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
+    if (any_groups && (!codes || !rscale || !rmn || !tscale || !tmn)) return PQ_ERR_NULL_POINTER;
+    const bool any_resid = n_resid_per_seq ? resid_capacity > 0 : n_resid > 0;
+    if (any_resid && !k_resid) return PQ_ERR_NULL_POINTER;
+    if (!n_groups_per_seq && n_groups > group_capacity) return PQ_ERR_BAD_STRIDE;
+    if (!n_resid_per_seq && n_resid > resid_capacity) return PQ_ERR_BAD_STRIDE;
+    if (!n_groups_per_seq && !n_resid_per_seq &&
+        static_cast<int64_t>(n_groups) * PQ_GROUP + n_resid > v_capacity) return PQ_ERR_BAD_STRIDE;
+    // with per-sequence counts (device arrays) the kernel clamps each sequence to the capacities instead
+    if (mask && mask_stride <= 0) return PQ_ERR_BAD_STRIDE;
+    if (mask && !n_groups_per_seq && !n_resid_per_seq &&
+        mask_stride < static_cast<int64_t>(n_groups) * PQ_GROUP + n_resid) return PQ_ERR_BAD_STRIDE;
+    if (!(sm_scale == sm_scale)) return PQ_ERR_BAD_SHAPE;
+    if (n_splits < 1 || n_splits > 65534) return PQ_ERR_WORKSPACE;
+    if (workspace_bytes < pq_decode_attn_workspace_bytes(B, N, n_splits)) return PQ_ERR_WORKSPACE;
+    if (!aligned(q, 2) || !aligned(v, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return PQ_ERR_MISALIGNED;
+    if (codes && !aligned(codes, 16)) return PQ_ERR_MISALIGNED;
+    if (k_resid && !aligned(k_resid, 16)) return PQ_ERR_MISALIGNED;
+    return PQ_OK;
+}
+
+int pq_decode_attn(const void* q,
+                   const uint8_t* codes, const void* rscale, const void* rmn,
+                   const void* tscale, const void* tmn, int group_capacity,
+                   int n_groups, const int32_t* n_groups_per_seq,
+                   const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                   const void* v, int64_t v_capacity,
+                   const uint8_t* mask, int64_t mask_stride,
+                   float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                   int n_splits, void* workspace, size_t workspace_bytes,
+                   void* out, void* stream) {
+    if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+                                         k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
+                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, workspace,
+                                         workspace_bytes, out))
+        return rc;
+    pq::AttnArgs a;
+    a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
+    a.group_capacity = group_capacity; a.n_groups = n_groups; a.n_groups_per_seq = n_groups_per_seq;
+    a.k_resid = k_resid; a.resid_capacity = resid_capacity; a.n_resid = n_resid; a.n_resid_per_seq = n_resid_per_seq;
+    a.v = v; a.v_capacity = v_capacity; a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
+    a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
+    a.workspace = static_cast<float*>(workspace); a.out = out;
+    const int err = pq::launch_attn(a, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -100,6 +100,31 @@ __device__ __forceinline__ uint32_t lds_addr(void* p) {
     return (uint32_t)(uintptr_t)((lds_void*)p);
 }
 
+// sin and cos of a bin-centre angle.  Three-constant Cody-Waite reduction by
+// pi/2 with fused multiply-adds (accurate for |x| up to ~1e6, far beyond any
+// half-precision tscale*(theta+0.5)+tmn), then the classic single-precision
+// minimax polynomials on [-pi/4, pi/4]; absolute error below 2e-7.  Straight-line
+// code: the library sincosf carries a Payne-Hanek branch the table build
+// neither needs nor can afford in registers.
+__device__ __forceinline__ void sincos_bin(float x, float* sn, float* cs) {
+    const float k = __builtin_rintf(x * 0.636619772367581343f);
+    float r = __builtin_fmaf(-k, 0x1.921fb6p+0f, x);
+    r = __builtin_fmaf(-k, -0x1.777a5cp-25f, r);
+    r = __builtin_fmaf(-k, -0x1.ee59dap-50f, r);
+    const float z = r * r;
+    float ps = __builtin_fmaf(z, -1.9515295891e-4f, 8.3321608736e-3f);
+    ps = __builtin_fmaf(ps, z, -1.6666654611e-1f);
+    const float s0 = __builtin_fmaf(ps * z, r, r);
+    float pc = __builtin_fmaf(z, 2.443315711809948e-5f, -1.388731625493765e-3f);
+    pc = __builtin_fmaf(pc, z, 4.166664568298827e-2f);
+    const float c0 = __builtin_fmaf(pc * z, z, __builtin_fmaf(z, -0.5f, 1.0f));
+    const int q = static_cast<int>(k);
+    const float ss = (q & 1) ? c0 : s0;
+    const float cc = (q & 1) ? s0 : c0;
+    *sn = (q & 2) ? -ss : ss;
+    *cs = ((q + 1) & 2) ? -cc : cc;
+}
+
 // Build the table for one group.  lane == pair d.
 //   qx[j], qy[j]: q_j[d], q_j[d+64] (0 for padded heads)
 //   returns c_d for this lane's pair.
@@ -110,8 +135,8 @@ __device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (
     const float ts = lo2f<T>(w_tscale), tm = lo2f<T>(w_tmn);
     const float rs = lo2f<T>(w_rscale), rm = lo2f<T>(w_rmn);
     float s, c, sd, cd;
-    sincosf(__builtin_fmaf(ts, 0.5f, tm), &s, &c);
-    sincosf(ts, &sd, &cd);
+    sincos_bin(__builtin_fmaf(ts, 0.5f, tm), &s, &c);
+    sincos_bin(ts, &sd, &cd);
     const float rmp = __builtin_fmaf(rs, 0.5f, rm);
     float a, cdv;
     if (rs != 0.0f) { a = rs; cdv = rmp / rs; }
@@ -147,8 +172,8 @@ __device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (
 
 // Score one token against the table.  `codes` holds the token's 64 pair codes as
 // 16 little-endian words; cds[d] are the wave-uniform c_d.  acc[j] += ...
-// The 64 table reads are issued in batches of 8 codes, one batch ahead of the
-// FMAs that consume them, so that 8-16 LDS reads are always in flight.
+// The 64 table reads are issued in batches of 4 or 8 codes, one batch ahead of the
+// FMAs that consume them, so that 4-16 LDS reads are always in flight.
 template <int TB, int REPP>
 __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes)[16], const float (&cds)[kPairs],
                                             float (&acc)[REPP]) {
@@ -156,7 +181,7 @@ __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes
     constexpr uint32_t TM4 = ((1u << TB) - 1u) * 0x01010101u;
     constexpr uint32_t RM4 = (0xFFu >> TB) * 0x01010101u;
     constexpr int nbm = L::NB - 1;
-    constexpr int BW = REPP == 8 ? 1 : 2;      // code words per batch
+    constexpr int BW = REPP >= 4 ? 1 : 2;      // code words per batch
     constexpr int NBATCH = 16 / BW;
     float e[2][BW * 4][REPP];
     uint32_t r4s[2][BW];
@@ -217,6 +242,10 @@ __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes
         compute(BI);
         __builtin_amdgcn_sched_barrier(0);
     });
+    // pin the sums here: otherwise the optimizer sinks the FMA chains into whatever
+    // conditional code consumes them and keeps all 64 table entries alive until then
+#pragma unroll
+    for (int j = 0; j < REPP; j++) asm volatile("" : "+v"(acc[j]));
 }
 #pragma clang diagnostic pop
 

@@ -56,10 +56,6 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) v
 #pragma unroll
         for (int j = 0; j < REPP; j++) acc[j] = 0.0f;
         score_token<TB, REPP>(lut, cwords, cds, acc);
-        // pin the sums: without this the optimizer sinks each head's FMAs into its
-        // "j < rep" store branch and keeps every table entry alive until then
-#pragma unroll
-        for (int j = 0; j < REPP; j++) asm volatile("" : "+v"(acc[j]));
 #pragma unroll
         for (int j = 0; j < REPP; j++)
             if (j < rep) ob[static_cast<size_t>(j) * Nb * kGroup + t * kWave] = acc[j];

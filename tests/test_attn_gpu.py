@@ -1,0 +1,160 @@
+"""GPU parity of pq_decode_attn (through the C ABI) against the CPU oracle.
+
+Bar: attention output within rtol 1e-2 / atol 1e-3 of the reference path
+(fp16).  Two references are used: the literal restatement (half-rounded
+softmax, as the reference computes) and an fp64 evaluation with no
+intermediate rounding; the kernel must meet the bar against both.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import polar_oracle as po
+from polarquant_amd import workloads as wl
+from polarquant_amd.attention import polar_decode_attention
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def _close(got, ref, rtol=RTOL, atol=ATOL):
+    got, ref = got.double(), ref.double()
+    err = (got - ref).abs()
+    bad = err > atol + rtol * ref.abs()
+    return int(bad.sum()), float(err.max())
+
+
+def _case(gpu, B, N, Nk, n_groups, n_resid, rbits, tbits, dtype, theta=5e5, mask_pad=0, seed=0, n_splits=None,
+          caps=(0, 0, 0)):
+    g = torch.Generator().manual_seed(seed)
+    L = n_groups * 128 + n_resid
+    k = wl.make_keys(B, Nk, max(L, 1), theta, g, dtype)
+    q = wl.make_half((B, N, 1, 128), g, dtype)
+    v = wl.make_half((B, Nk, L, 128), g, dtype)
+    quant = (None,) * 5
+    if n_groups:
+        quant = po.quantize_and_pack_nbit(k[:, :, :n_groups * 128].contiguous(), rbits, tbits)
+    kres = k[:, :, n_groups * 128:L].contiguous() if n_resid else None
+    mask = None
+    if mask_pad:
+        mask = torch.ones(B, L, dtype=torch.int64)
+        for b in range(B):
+            mask[b, :(mask_pad * (b + 1)) % L] = 0      # left padding, different per sequence
+    ref = po.decode_attention(q, kres, *quant, v, mask, rbits, tbits)
+    ref64 = po.decode_attention_exact(q, kres, *quant, v, mask, rbits, tbits)
+    # device tensors, optionally with spare capacity behind the used part
+    gc, rc, vc = caps
+    dq = [None] * 5
+    if n_groups:
+        cap = n_groups + gc
+        dq = [torch.zeros((B, Nk, cap) + tuple(t.shape[3:]), dtype=t.dtype, device=gpu) for t in quant]
+        for d, t in zip(dq, quant):
+            d[:, :, :n_groups] = t.to(gpu)
+    dk = None
+    if n_resid:
+        dk = torch.zeros(B, Nk, n_resid + rc, 128, dtype=dtype, device=gpu)
+        dk[:, :, :n_resid] = kres.to(gpu)
+    dv = torch.zeros(B, Nk, L + vc, 128, dtype=dtype, device=gpu)
+    dv[:, :, :L] = v.to(gpu)
+    if vc:
+        dv[:, :, L:] = float("nan")     # rows past the end must never contribute
+    out = polar_decode_attention(q.to(gpu), *dq, dk, dv, n_groups, n_resid,
+                                 attention_mask=None if mask is None else mask.to(gpu),
+                                 rbits=rbits, tbits=tbits, n_splits=n_splits)
+    torch.cuda.synchronize()
+    out = out.cpu()
+    assert out.shape == (B, N, 1, 128) and out.dtype == dtype
+    assert torch.isfinite(out.float()).all()
+    return out, ref, ref64
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,Nk,rbits,tbits", [(32, 8, 4, 4), (32, 32, 4, 4), (28, 4, 3, 3), (16, 8, 4, 4), (12, 2, 3, 3)])
+def test_attn_matches_oracle(gpu, dtype, N, Nk, rbits, tbits):
+    print("case", dtype, N, Nk, rbits, tbits, flush=True)
+    out, ref, ref64 = _case(gpu, 2, N, Nk, 6, 37, rbits, tbits, dtype, seed=1)
+    rtol, atol = (RTOL, ATOL) if dtype == torch.float16 else (2e-2, 4e-3)   # bf16 has 8 mantissa bits
+    nbad, emax = _close(out, ref64, rtol, atol)
+    print("max err vs fp64", emax, flush=True)
+    assert nbad == 0
+    nbad, emax = _close(out, ref, rtol, atol)
+    assert nbad == 0
+
+
+@pytest.mark.parametrize("n_groups,n_resid", [(0, 1), (0, 64), (0, 128), (1, 0), (1, 1), (3, 127), (5, 128), (2, 65)])
+def test_attn_residual_edges(gpu, n_groups, n_resid):
+    """Empty quantized part, empty residual, full 128-token residual (the step before a flush)."""
+    print("case", n_groups, n_resid, flush=True)
+    out, ref, ref64 = _case(gpu, 2, 32, 8, n_groups, n_resid, 4, 4, torch.float16, seed=2)
+    assert _close(out, ref64)[0] == 0 and _close(out, ref)[0] == 0
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 3, 7, 16])
+def test_attn_split_invariance(gpu, n_splits):
+    out, ref, ref64 = _case(gpu, 1, 32, 8, 16, 5, 4, 4, torch.float16, seed=3, n_splits=n_splits)
+    assert _close(out, ref64)[0] == 0
+
+
+def test_attn_left_padding_mask(gpu):
+    out, ref, ref64 = _case(gpu, 3, 32, 8, 4, 19, 4, 4, torch.float16, seed=4, mask_pad=150)
+    assert _close(out, ref64)[0] == 0 and _close(out, ref)[0] == 0
+
+
+def test_attn_spare_capacity(gpu):
+    """Cache tensors larger than the used part (pre-allocated arena); unused V rows hold NaN."""
+    out, ref, ref64 = _case(gpu, 2, 32, 8, 3, 40, 4, 4, torch.float16, seed=5, caps=(5, 88, 300))
+    assert _close(out, ref64)[0] == 0
+
+
+def test_attn_ragged_lengths(gpu):
+    """Per-sequence context lengths (continuous batching): groups and residual counts per sequence."""
+    g = torch.Generator().manual_seed(8)
+    B, N, Nk, rb, tb = 6, 28, 4, 3, 3
+    lens = torch.tensor([129, 512, 700, 1023, 128, 77])
+    Lmax = int(lens.max())
+    k = wl.make_keys(B, Nk, Lmax, 1e6, g)
+    q = wl.make_half((B, N, 1, 128), g)
+    v = wl.make_half((B, Nk, Lmax, 128), g)
+    gcap = Lmax // 128
+    codes = torch.zeros(B, Nk, gcap, 128, 64, dtype=torch.uint8)
+    meta = [torch.zeros(B, Nk, gcap, 1, 64, dtype=torch.float16) for _ in range(4)]
+    kres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16)
+    refs = []
+    for b in range(B):
+        L = int(lens[b]); ng, nr = L // 128, L % 128
+        quant = (None,) * 5
+        if ng:
+            quant = po.quantize_and_pack_nbit(k[b:b + 1, :, :ng * 128].contiguous(), rb, tb)
+            codes[b, :, :ng] = quant[0][0]
+            for m, t in zip(meta, quant[1:]):
+                m[b, :, :ng] = t[0]
+        kr = k[b:b + 1, :, ng * 128:L].contiguous() if nr else None
+        if nr:
+            kres[b, :, :nr] = kr[0]
+        refs.append(po.decode_attention_exact(q[b:b + 1], kr, *quant, v[b:b + 1, :, :L], None, rb, tb))
+    ref64 = torch.cat(refs, 0)
+    out = polar_decode_attention(q.to(gpu), codes.to(gpu), *[m.to(gpu) for m in meta], kres.to(gpu), v.to(gpu),
+                                 0, 0, rbits=rb, tbits=tb,
+                                 n_groups_per_seq=(lens // 128).int().to(gpu), n_resid_per_seq=(lens % 128).int().to(gpu),
+                                 n_splits=3)
+    torch.cuda.synchronize()
+    assert _close(out.cpu(), ref64)[0] == 0
+
+
+def test_attn_sharp_softmax(gpu):
+    """A query aligned with one key: the softmax is dominated by a single token
+    whose score is far above the rest, in a late tile (exercises the lazy rescale)."""
+    g = torch.Generator().manual_seed(12)
+    B, N, Nk, ng = 1, 32, 8, 8
+    L = ng * 128 + 3
+    k = wl.make_keys(B, Nk, L, 5e5, g)
+    v = wl.make_half((B, Nk, L, 128), g)
+    q = wl.make_half((B, N, 1, 128), g)
+    for h in range(N):
+        q[0, h, 0] = (k[0, h // 4, 700 + h] * 1.5).half()
+    quant = po.quantize_and_pack_nbit(k[:, :, :ng * 128].contiguous())
+    kres = k[:, :, ng * 128:].contiguous()
+    ref64 = po.decode_attention_exact(q, kres, *quant, v)
+    out = polar_decode_attention(q.to(gpu), *[t.to(gpu) for t in quant], kres.to(gpu), v.to(gpu), ng, 3, n_splits=2)
+    assert _close(out.cpu(), ref64)[0] == 0
