@@ -1,0 +1,247 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused polar decode attention, Llama-3-8B shape, batch 16, 32k context.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one pass of the hot path over one batch: the fused decode
+attention of one layer (quantized-key scores + residual key + softmax + P.V)
+for 16 sequences x 32 query heads over 32768 cached tokens (4-bit radius /
+4-bit angle codes, fp16 values), inputs resident in HBM.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b16 32k"
+
+# HBM bytes per launch of the dominant kernel at this workload, from two
+# `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
+# read for a copy kernel of known size; see profiles/attn_kernel_cfg1_pmc.md.
+# None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def build_cfg1(dev, dtype=torch.float16):
+    """configs[1] resident in HBM: polar 4/4 key cache of 256 groups per (sequence, KV head),
+    fp16 V cache, one new token whose key sits in the fp16 residual buffer."""
+    from polarquant_amd import workloads as wl
+    from polarquant_amd.quantize import quantize_and_pack_nbit
+
+    sh = wl.CONFIGS[1]
+    B, N, Nk, L = sh.batch, sh.n_heads, sh.n_kv_heads, sh.context
+    Nb = L // 128
+    g = torch.Generator(device=dev).manual_seed(sh.seed)
+    codes = torch.empty(B, Nk, Nb, 128, 64, dtype=torch.uint8, device=dev)
+    meta = [torch.empty(B, Nk, Nb, 1, 64, dtype=dtype, device=dev) for _ in range(4)]
+    inv_freq = 1.0 / (sh.rope_theta ** (torch.arange(0, 128, 2, dtype=torch.float32, device=dev) / 128))
+    ang = torch.arange(L, dtype=torch.float32, device=dev)[:, None] * inv_freq[None, :]
+    cos, sin = torch.cat([ang, ang], -1).cos(), torch.cat([ang, ang], -1).sin()
+    outl = torch.randperm(128, generator=g, device=dev)[:4]
+    for b in range(B):                      # keys of one sequence at a time: 64 MiB fp16
+        k = torch.randn(1, Nk, L, 128, generator=g, device=dev, dtype=torch.float32)
+        k[..., outl] *= 8.0
+        k = (k * cos + torch.cat([-k[..., 64:], k[..., :64]], -1) * sin).to(dtype)
+        quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=(codes[b:b + 1], *[m[b:b + 1] for m in meta]))
+    v = torch.empty(B, Nk, L + 1, 128, dtype=dtype, device=dev)
+    for b in range(B):
+        v[b] = torch.randn(Nk, L + 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    q = torch.randn(B, N, 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    k_new = torch.randn(B, Nk, 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    kres = torch.zeros(B, Nk, 128, 128, dtype=dtype, device=dev)
+    kres[:, :, :1] = k_new
+    return dict(shape=sh, q=q, codes=codes, meta=meta, kres=kres, v=v, n_groups=Nb, n_resid=1)
+
+
+def time_events(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps      # ms per call
+
+
+def kernel_duration_ms(launch, steps):
+    """Average duration of one launch, each launch bracketed by its own pair of
+    events on the launching stream."""
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    for a, b in evs:
+        a.record()
+        launch()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in evs) / steps
+
+
+def cpu_baseline(w):
+    """The reference path on the host cores: dequantize-then-matmul scores, /sqrt(d),
+    fp32 softmax, P.V (oracle restatement of modeling_llama_polar.py:66-99 and
+    kernel4group.py:151-155), on one of the 16 sequences, scaled to the batch."""
+    from oracle import polar_oracle as po
+    sh = w["shape"]
+    b = 0
+    cq = w["q"][b:b + 1].cpu()
+    quant = [w["codes"][b:b + 1].cpu()] + [m[b:b + 1].cpu() for m in w["meta"]]
+    kres = w["kres"][b:b + 1, :, :w["n_resid"]].cpu()
+    v = w["v"][b:b + 1].cpu()
+    threads = torch.get_num_threads()
+    po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)        # warm-up
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 20):
+        t0 = time.perf_counter()
+        ref = po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return ref, {
+        "value": round(med * sh.batch * 1e6, 1), "unit": "us/step", "cores": threads, "kind": "port",
+        "sample": "sequence 0 of %d (8 KV heads x 32768 tokens), median of %d runs of the torch-CPU restatement "
+                  "of the reference path (dequantize, matmul, softmax, P.V), scaled x%d to the batch"
+                  % (sh.batch, len(times), sh.batch),
+    }
+
+
+def fp16_baselines(w, steps, warmup):
+    """Un-quantized fp16 decode attention on the same GPU: (i) the reference's eager
+    path (benchmark/models/modeling_llama_exp.py:42-52: cat + repeat_kv + matmul,
+    softmax, matmul) and (ii) torch's fused scaled_dot_product_attention."""
+    import torch.nn.functional as F
+    sh = w["shape"]
+    B, N, Nk, L = sh.batch, sh.n_heads, sh.n_kv_heads, sh.context
+    dev = w["q"].device
+    g = torch.Generator(device=dev).manual_seed(1)
+    kc = torch.empty(B, Nk, L, 128, dtype=torch.float16, device=dev)
+    for b in range(B):
+        kc[b] = torch.randn(Nk, L, 128, generator=g, device=dev).half()
+    vc = w["v"][:, :, :L].contiguous()
+    q, kn, vn = w["q"], w["kres"][:, :, :1].contiguous(), w["v"][:, :, L:L + 1].contiguous()
+    rep = N // Nk
+
+    def repeat_kv(x):
+        b, h, s, d = x.shape
+        return x[:, :, None].expand(b, h, rep, s, d).reshape(b, h * rep, s, d)
+
+    def eager():
+        k = torch.cat([kc, kn], dim=2)
+        v = torch.cat([vc, vn], dim=2)
+        a = torch.matmul(q, repeat_kv(k).transpose(2, 3)) / math.sqrt(128)
+        a = torch.softmax(a, dim=-1, dtype=torch.float32).to(q.dtype)
+        return torch.matmul(a, repeat_kv(v))
+
+    kf, vf = torch.cat([kc, kn], dim=2), torch.cat([vc, vn], dim=2)
+
+    def sdpa():
+        return F.scaled_dot_product_attention(q, kf, vf, enable_gqa=True)
+
+    out = {}
+    try:
+        out["fp16_eager_us"] = round(time_events(eager, max(3, steps // 4), 2) * 1e3, 1)
+    except Exception as e:                      # noqa: BLE001 - report, do not fail the bench
+        out["fp16_eager_error"] = str(e)[:200]
+    try:
+        out["fp16_sdpa_us"] = round(time_events(sdpa, steps, warmup) * 1e3, 1)
+    except Exception as e:                      # noqa: BLE001
+        out["fp16_sdpa_error"] = str(e)[:200]
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-baselines", action="store_true", help="skip the CPU and fp16 baselines")
+    ap.add_argument("--splits", type=int, default=0, help="override the context split count")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported"
+              % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    from polarquant_amd import _ffi, workloads as wl
+    from polarquant_amd.attention import plan_splits, polar_decode_attention, workspace_for
+    from polarquant_amd.kernel4group import _stream_ptr
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _ffi.lib()
+    w = build_cfg1(dev)
+    sh = w["shape"]
+    B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
+    n_splits = args.splits or plan_splits(B, Nk, w["n_groups"], dev)
+    ws = workspace_for(B, N, n_splits, dev)
+    out = torch.empty(B, N, 1, 128, dtype=torch.float16, device=dev)
+    sm_scale = 1.0 / math.sqrt(128)
+
+    def step():
+        polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"],
+                               rbits=sh.rbits, tbits=sh.tbits, n_splits=n_splits, out=out)
+
+    common = [w["q"].data_ptr(), w["codes"].data_ptr(), *[m.data_ptr() for m in w["meta"]], w["codes"].shape[2],
+              w["n_groups"], None, w["kres"].data_ptr(), w["kres"].shape[2], w["n_resid"], None,
+              w["v"].data_ptr(), w["v"].shape[2], None, 0, sm_scale, B, N, Nk, sh.rbits, sh.tbits, _ffi.PQ_F16,
+              n_splits, ws.data_ptr(), ws.numel() * 4]
+
+    def partials_only():
+        rc = lib.pq_decode_attn_partials(*common, _stream_ptr(dev))
+        assert rc == 0, rc
+
+    ms = time_events(step, args.steps, args.warmup)
+    k_ms = kernel_duration_ms(partials_only, args.steps)
+
+    alg_bytes = wl.algorithmic_bytes(Nk, N, [w["n_groups"] * 128] * B, [w["n_resid"]] * B, sh.rbits, sh.tbits)
+    achieved = alg_bytes / (k_ms * 1e-3) / 1e9
+    result = {
+        "metric": METRIC, "value": round(ms * 1e3, 2), "unit": "us/step", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: fused polar decode attention, Llama-3-8B shape (32 q heads / 8 KV heads, "
+                               "head_dim 128), batch 16, context 32768, 4-bit radius / 4-bit angle, 128-token groups, "
+                               "fp16 V, one decode step of one layer",
+                   "n_splits": n_splits, "algorithmic_bytes": alg_bytes},
+        "hbm_gbps": round(alg_bytes / (ms * 1e-3) / 1e9, 1),
+        "pct_of_hbm_peak": round(100 * alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
+        "roofline": {"bound": "hbm", "kernel": "attn_kernel<F16,4,4>", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES},
+    }
+    if not args.no_baselines:
+        ref, cpu = cpu_baseline(w)
+        result["cpu_baseline"] = cpu
+        got = out[0:1].cpu()
+        err = (got.double() - ref.double()).abs()
+        result["parity_vs_cpu_sample"] = {"max_abs_err": float(err.max()),
+                                          "within_rtol1e-2_atol1e-3": bool((err <= 1e-3 + 1e-2 * ref.double().abs()).all())}
+        fp = fp16_baselines(w, args.steps, args.warmup)
+        result.update(fp)
+        for key in ("fp16_eager_us", "fp16_sdpa_us"):
+            if key in fp:
+                result["speedup_vs_" + key[:-3]] = round(fp[key] / (ms * 1e3), 2)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -164,6 +164,26 @@ int pq_validate_decode_attn(const void *q,
                             int n_splits, const void *workspace, size_t workspace_bytes,
                             const void *out);
 
+/* The two launches of pq_decode_attn as separate calls, same arguments and
+ * checks: pq_decode_attn_partials writes the n_splits + 1 partial results
+ * (running maximum, probability sum, un-normalised output) of every query head
+ * into `workspace`; pq_decode_attn_merge combines them into `out`.  They exist so
+ * that a caller can time, overlap or graph-capture the two kernels separately;
+ * pq_decode_attn(...) == partials(...) followed by merge(...) on the same stream.
+ * No reference counterpart beyond that of pq_decode_attn. */
+int pq_decode_attn_partials(const void *q,
+                            const uint8_t *codes, const void *rscale, const void *rmn,
+                            const void *tscale, const void *tmn, int group_capacity,
+                            int n_groups, const int32_t *n_groups_per_seq,
+                            const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                            const void *v, int64_t v_capacity,
+                            const uint8_t *mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, void *workspace, size_t workspace_bytes, void *stream);
+
+int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
+                         void *out, void *stream);
+
 /* Suggested n_splits for a shape (host-only; `max_groups` = largest group count
  * of any sequence, `n_cus` = compute units of the device or 0 for 256). */
 int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus);

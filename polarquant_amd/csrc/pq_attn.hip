@@ -360,10 +360,6 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
         default: PQ_LAUNCH(8); break;
     }
 #undef PQ_LAUNCH
-    int err = static_cast<int>(hipGetLastError());
-    if (err) return err;
-    hipLaunchKernelGGL(merge_kernel<T>, dim3(a.B * a.N), dim3(kHeadDim), 0, st, a.workspace, a.n_splits + 1,
-                       (uint16_t*)a.out);
     return static_cast<int>(hipGetLastError());
 }
 
@@ -377,8 +373,16 @@ static int launch_attn_t(const AttnArgs& a, hipStream_t st) {
     }
 }
 
-int launch_attn(const AttnArgs& a, hipStream_t st) {
+int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
     return a.dtype == 0 ? launch_attn_t<F16>(a, st) : launch_attn_t<BF16>(a, st);
+}
+
+int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st) {
+    if (dtype == 0)
+        hipLaunchKernelGGL(merge_kernel<F16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits + 1, (uint16_t*)out);
+    else
+        hipLaunchKernelGGL(merge_kernel<BF16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits + 1, (uint16_t*)out);
+    return static_cast<int>(hipGetLastError());
 }
 
 }  // namespace pq

@@ -167,6 +167,45 @@ int pq_validate_decode_attn(const void* q,
     return PQ_OK;
 }
 
+int pq_decode_attn_partials(const void* q,
+                            const uint8_t* codes, const void* rscale, const void* rmn,
+                            const void* tscale, const void* tmn, int group_capacity,
+                            int n_groups, const int32_t* n_groups_per_seq,
+                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                            const void* v, int64_t v_capacity,
+                            const uint8_t* mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, void* workspace, size_t workspace_bytes, void* stream) {
+    // `out` is not touched by this half: validate with a stand-in non-null, aligned pointer
+    if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+                                         k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
+                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, workspace,
+                                         workspace_bytes, workspace))
+        return rc;
+    pq::AttnArgs a;
+    a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
+    a.group_capacity = group_capacity; a.n_groups = n_groups; a.n_groups_per_seq = n_groups_per_seq;
+    a.k_resid = k_resid; a.resid_capacity = resid_capacity; a.n_resid = n_resid; a.n_resid_per_seq = n_resid_per_seq;
+    a.v = v; a.v_capacity = v_capacity; a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
+    a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
+    a.workspace = static_cast<float*>(workspace); a.out = nullptr;
+    const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+int pq_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
+                         void* out, void* stream) {
+    if (!workspace || !out) return PQ_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0) return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (n_splits < 1 || n_splits > 65534) return PQ_ERR_WORKSPACE;
+    if (workspace_bytes < pq_decode_attn_workspace_bytes(B, N, n_splits)) return PQ_ERR_WORKSPACE;
+    if (!aligned(workspace, 16) || !aligned(out, 2)) return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_attn_merge(static_cast<const float*>(workspace), B, N, n_splits, dtype, out,
+                                          static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 int pq_decode_attn(const void* q,
                    const uint8_t* codes, const void* rscale, const void* rmn,
                    const void* tscale, const void* tmn, int group_capacity,
@@ -177,20 +216,13 @@ int pq_decode_attn(const void* q,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                    int n_splits, void* workspace, size_t workspace_bytes,
                    void* out, void* stream) {
-    if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+    if (!out) return PQ_ERR_NULL_POINTER;
+    if (int rc = pq_decode_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                          mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, workspace,
-                                         workspace_bytes, out))
+                                         workspace_bytes, stream))
         return rc;
-    pq::AttnArgs a;
-    a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
-    a.group_capacity = group_capacity; a.n_groups = n_groups; a.n_groups_per_seq = n_groups_per_seq;
-    a.k_resid = k_resid; a.resid_capacity = resid_capacity; a.n_resid = n_resid; a.n_resid_per_seq = n_resid_per_seq;
-    a.v = v; a.v_capacity = v_capacity; a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
-    a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
-    a.workspace = static_cast<float*>(workspace); a.out = out;
-    const int err = pq::launch_attn(a, static_cast<hipStream_t>(stream));
-    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+    return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
 
 }  // extern "C"

@@ -32,7 +32,8 @@ struct AttnArgs {
     float* workspace;
     void* out;
 };
-int launch_attn(const AttnArgs& a, hipStream_t st);
+int launch_attn_partials(const AttnArgs& a, hipStream_t st);
+int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st);
 
 inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 : 8; }
 
