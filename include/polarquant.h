@@ -165,7 +165,7 @@ int pq_validate_decode_attn(const void *q,
                             const void *out);
 
 /* The two launches of pq_decode_attn as separate calls, same arguments and
- * checks: pq_decode_attn_partials writes the n_splits + 1 partial results
+ * checks: pq_decode_attn_partials writes the n_splits partial results
  * (running maximum, probability sum, un-normalised output) of every query head
  * into `workspace`; pq_decode_attn_merge combines them into `out`.  They exist so
  * that a caller can time, overlap or graph-capture the two kernels separately;

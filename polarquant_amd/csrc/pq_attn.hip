@@ -3,9 +3,14 @@
 // (reference decode branch: models/modeling_llama_polar.py:66-99), split over
 // the context, followed by a small merge kernel.
 //
-// attn_kernel: grid (n_splits + 1, B*Nk), one wavefront per block.
-//   block x <  n_splits : the x-th slice of the sequence's quantized groups
-//   block x == n_splits : the fp16 residual keys (0..128 tokens)
+// attn_kernel: grid (n_splits, B*Nk), one wavefront per block: block x works
+// through the x-th slice of the sequence's quantized groups; the last block of
+// a (batch, KV head) then also takes the fp16 residual keys (0..128 tokens).
+// The kernel is built for ONE resident wavefront per SIMD (4 per CU) with deep
+// software prefetch instead of many wavefronts: V operands are double-buffered
+// a whole 64-token tile ahead, which keeps ~40 KiB of loads in flight per
+// wavefront; pq_decode_attn_plan sizes n_splits so that B*Nk*n_splits fills
+// those slots exactly once.
 // Each wavefront walks its tokens in 64-token tiles, lane == token, and keeps
 // flash-style running state (m, l, acc) for the `rep` query heads of its KV
 // head.  P.V runs on the matrix cores: for 16 tokens at a time
@@ -19,7 +24,7 @@
 // 32-register rescale of the accumulators is skipped on almost every tile.
 //
 // merge_kernel: grid B*N, 128 threads (one per output dim): combines the
-// n_splits + 1 partials (m, l, acc[128]) of a query head and writes half words.
+// n_splits partials (m, l, acc[128]) of a query head and writes half words.
 #include "pq_device.h"
 #include "pq_internal.h"
 
@@ -144,7 +149,7 @@ __device__ __forceinline__ void load_v_tile(uint4 (&vv)[4][4], __amdgpu_buffer_r
 }
 
 template <typename T, int TB, int REPP>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 3)))
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(1, 2)))
 void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                  const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
                  const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
@@ -187,7 +192,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
-    if (split < n_splits) {
+    {
         // ---------------- quantized groups [g0, g1) ----------------
         const int gps = (nb + n_splits - 1) / n_splits;
         const int g0 = split * gps;
@@ -213,6 +218,9 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             const uint16_t* pts = tscale + plane * kPairs + lane;
             const uint16_t* ptm = tmn + plane * kPairs + lane;
             uint16_t mrs = prs[g0 * kPairs], mrm = prm[g0 * kPairs], mts = pts[g0 * kPairs], mtm = ptm[g0 * kPairs];
+            // V operands are double-buffered by tile parity: tile t+1 is requested before tile t is scored
+            uint4 vv[2][4][4];
+            load_v_tile(vv[0], rv, voff_v, static_cast<uint32_t>(2 * g0) * kWave * (kHeadDim * 2));
             for (int grp = g0; grp < g1; grp++) {
                 asm volatile("" ::: "memory");
                 const float cdv = build_lut<T, TB, REPP>(lut, lane, qx, qy, mrs, mrm, mts, mtm);
@@ -227,8 +235,8 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                 for (int half = 0; half < 2; half++) {
                     const int tt = 2 * grp + half;
                     const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
-                    uint4 vv[4][4];
-                    load_v_tile(vv, rv, voff_v, tok0 * (kHeadDim * 2));
+                    // past the last tile of this slice the loads run off the buffer's end and return zeros
+                    load_v_tile(vv[half ^ 1], rv, voff_v, (half == 0 || grp + 1 < g1) ? (tok0 + kWave) * (kHeadDim * 2) : 0xFFFFFF00u);
                     uint32_t cw[16];
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -246,12 +254,14 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     const bool keep = has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(tok0), 0) != 0) : true;
 #pragma unroll
                     for (int j = 0; j < REPP; j++) s[j] = keep ? s[j] * scale_log2 : -INFINITY;
-                    softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
+                    softmax_pv_tile<T, REPP>(st, s, vv[half], pbuf, lane);
                 }
             }
         }
-    } else if (nres > 0) {
+    }
+    if (split == n_splits - 1 && nres > 0) {
         // ---------------- fp16 residual keys ----------------
+        asm volatile("" ::: "memory");
         // q as fp32 in LDS: [REPP][128]
 #pragma unroll
         for (int j = 0; j < REPP; j++) {
@@ -312,7 +322,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
         float mm = st.m[0], ll = lsum[0];
 #pragma unroll
         for (int j = 1; j < REPP; j++) { mm = (n == j) ? st.m[j] : mm; ll = (n == j) ? lsum[j] : ll; }
-        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * (n_splits + 1) + split) * kPartialFloats;
+        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * n_splits + split) * kPartialFloats;
         if (g == 0) { pw[0] = mm; pw[1] = ll; }
         float* pa = pw + 4 + 32 * g;
 #pragma unroll
@@ -326,25 +336,56 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 
 template <typename T>
 __global__ __launch_bounds__(kHeadDim) void merge_kernel(const float* __restrict__ ws, int n_part, uint16_t* __restrict__ out) {
+    // one block per query head, thread == output dim.  The partial headers (m, l)
+    // are fetched by one thread each, so that all loads of the block are issued
+    // at once instead of one dependent load per partial.
+    __shared__ float wgt[1024];
+    __shared__ float red[2][kHeadDim / kWave];
     const int bn = blockIdx.x, d = threadIdx.x;
     const float* p = ws + static_cast<size_t>(bn) * n_part * kPartialFloats;
     float M = -INFINITY;
-    for (int s = 0; s < n_part; s++) M = fmaxf(M, p[s * kPartialFloats]);
+    for (int s = d; s < n_part; s += kHeadDim) M = fmaxf(M, p[static_cast<size_t>(s) * kPartialFloats]);
+    M = wave_max(M);
+    if ((d & (kWave - 1)) == 0) red[0][d / kWave] = M;
+    __syncthreads();
+    M = fmaxf(red[0][0], red[0][1]);
     float num = 0.0f, den = 0.0f;
-    for (int s = 0; s < n_part; s++) {
-        const float m = p[s * kPartialFloats];
-        if (m == -INFINITY) continue;
-        const float w = exp2f(m - M);
-        den = __builtin_fmaf(w, p[s * kPartialFloats + 1], den);
-        num = __builtin_fmaf(w, p[s * kPartialFloats + 4 + d], num);
+    for (int s0 = 0; s0 < n_part; s0 += 1024) {
+        const int cnt = (n_part - s0) < 1024 ? (n_part - s0) : 1024;
+        __syncthreads();
+        for (int s = d; s < cnt; s += kHeadDim) {
+            const float m = p[static_cast<size_t>(s0 + s) * kPartialFloats];
+            const float w = (m == -INFINITY) ? 0.0f : exp2f(m - M);
+            wgt[s] = w;
+            den = __builtin_fmaf(w, p[static_cast<size_t>(s0 + s) * kPartialFloats + 1], den);
+        }
+        __syncthreads();
+        const float* pa = p + static_cast<size_t>(s0) * kPartialFloats + 4 + d;
+        int s = 0;
+        for (; s + 8 <= cnt; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = pa[static_cast<size_t>(s + u) * kPartialFloats];
+#pragma unroll
+            for (int u = 0; u < 8; u++) num = wgt[s + u] != 0.0f ? __builtin_fmaf(wgt[s + u], v[u], num) : num;
+        }
+        for (; s < cnt; s++) {
+            const float v = pa[static_cast<size_t>(s) * kPartialFloats];
+            num = wgt[s] != 0.0f ? __builtin_fmaf(wgt[s], v, num) : num;
+        }
     }
+    den = wave_sum(den);
+    __syncthreads();
+    if ((d & (kWave - 1)) == 0) red[1][d / kWave] = den;
+    __syncthreads();
+    den = red[1][0] + red[1][1];
     out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : 0.0f);
 }
 
 template <typename T, int TB>
 static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     const int rep = a.N / a.Nk;
-    dim3 grid(a.n_splits + 1, a.B * a.Nk), block(kWave);
+    dim3 grid(a.n_splits, a.B * a.Nk), block(kWave);
     const float scale_log2 = a.sm_scale * kLog2e;
 #define PQ_LAUNCH(REPP)                                                                                              \
     hipLaunchKernelGGL((attn_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,                \
@@ -379,9 +420,9 @@ int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
 
 int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st) {
     if (dtype == 0)
-        hipLaunchKernelGGL(merge_kernel<F16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits + 1, (uint16_t*)out);
+        hipLaunchKernelGGL(merge_kernel<F16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
     else
-        hipLaunchKernelGGL(merge_kernel<BF16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits + 1, (uint16_t*)out);
+        hipLaunchKernelGGL(merge_kernel<BF16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
     return static_cast<int>(hipGetLastError());
 }
 

@@ -114,9 +114,10 @@ extern "C" {
 int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || max_groups <= 0) return 1;
     if (n_cus <= 0) n_cus = 256;
-    // one wavefront per (batch, KV head, split); about 8 fit a CU next to their lookup tables.
-    // Aim for one resident wavefront per slot so that all slices run concurrently and finish together.
-    const long long slots = static_cast<long long>(n_cus) * 8;
+    // one wavefront per (batch, KV head, split), and the kernel keeps one wavefront per SIMD
+    // (4 per CU).  Fill those slots exactly once, so that all slices run concurrently and
+    // finish together; a few more blocks than slots would cost a whole second round.
+    const long long slots = static_cast<long long>(n_cus) * 4;
     long long n = slots / (static_cast<long long>(B) * Nk);
     if (n < 1) n = 1;
     if (n > max_groups) n = max_groups;
@@ -126,7 +127,7 @@ int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus) {
 
 size_t pq_decode_attn_workspace_bytes(int B, int N, int n_splits) {
     if (B <= 0 || N <= 0 || n_splits <= 0) return 0;
-    return static_cast<size_t>(B) * N * (static_cast<size_t>(n_splits) + 1) * PQ_PARTIAL_FLOATS * sizeof(float);
+    return static_cast<size_t>(B) * N * static_cast<size_t>(n_splits) * PQ_PARTIAL_FLOATS * sizeof(float);
 }
 
 int pq_validate_decode_attn(const void* q,
