@@ -28,8 +28,7 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # HBM bytes per launch of the dominant kernel at this workload, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
 # read for a copy kernel of known size; see profiles/attn_kernel_cfg1_pmc.md.
-# None until measured.
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = int(672030 * 2.0 * 1024 + 2176 * 1.0 * 1024)
 
 
 def build_cfg1(dev, dtype=torch.float16):
@@ -169,6 +168,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-baselines", action="store_true", help="skip the CPU and fp16 baselines")
     ap.add_argument("--splits", type=int, default=0, help="override the context split count")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run 3 plain 1 GiB device copies (torch clone): under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` "
+                         "their counter values give the scale factor for the attention kernel's")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported"
@@ -205,6 +207,13 @@ def main():
     def partials_only():
         rc = lib.pq_decode_attn_partials(*common, _stream_ptr(dev))
         assert rc == 0, rc
+
+    if args.copy_calib:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(3)
+        for _ in range(3):
+            dst = src.clone()
+        torch.cuda.synchronize()
+        del src, dst
 
     ms = time_events(step, args.steps, args.warmup)
     k_ms = kernel_duration_ms(partials_only, args.steps)

@@ -1,0 +1,132 @@
+"""The C ABI without a GPU: the library loads, exports every symbol that
+include/polarquant.h declares, and its host-side argument checks return the
+documented error codes.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from polarquant_amd import _ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+P = 0x7f0000000000          # a fake, 4 KiB-aligned "device pointer": the validators never dereference
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _ffi.lib()
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "polarquant.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    names = _declared_functions()
+    assert len(names) >= 12
+    raw = ctypes.CDLL(_ffi.LIB_PATH)
+    for n in names:
+        assert hasattr(raw, n), "libpolarquant_hip.so does not export %s" % n
+        assert n in _ffi.SIGNATURES, "%s is declared in the header but has no ctypes signature" % n
+    assert set(_ffi.SIGNATURES) == set(names)
+
+
+def test_version_and_status_strings(lib):
+    assert lib.pq_version() >= 100
+    for code in range(0, -10, -1):
+        assert lib.pq_status_string(code)
+    assert b"unknown" in lib.pq_status_string(-99)
+
+
+def test_validate_decode_scores(lib):
+    ok = [P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0]
+    assert lib.pq_validate_decode_scores(*ok) == 0
+
+    def bad(i, v):
+        a = list(ok); a[i] = v
+        return lib.pq_validate_decode_scores(*a)
+    assert bad(0, None) == -1 and bad(6, None) == -1                 # null pointers
+    assert bad(7, 0) == -2 and bad(9, 5) == -2 and bad(10, 0) == -2   # B<=0, N % Nk, Nb<=0
+    assert bad(8, 72) == -2                                          # rep 9 > 8
+    assert bad(11, 5) == -3 and bad(12, 5) == -3 and bad(12, 0) == -3  # r+t>8, tbits>4, tbits<1
+    assert bad(13, 2) == -4                                          # dtype
+    assert bad(1, P + 4) == -5 and bad(6, P + 2) == -5               # misaligned codes / out
+    # the launching entry point runs the same checks before touching the device
+    assert lib.pq_decode_scores(*ok[:11], 5, 4, 0, None) == -3
+
+
+def test_validate_quantize_groups(lib):
+    strides = (ctypes.c_int64 * 4)(8 * 256 * 128, 256 * 128, 128, 1)
+    sp = ctypes.cast(strides, ctypes.c_void_p)
+    ok = [P, sp, 0, 2, 8, 2, 4, 4, 0, P, P, P, P, P, 2, 0]
+    assert lib.pq_validate_quantize_groups(*ok) == 0
+
+    def bad(i, v):
+        a = list(ok); a[i] = v
+        return lib.pq_validate_quantize_groups(*a)
+    assert bad(0, None) == -1 and bad(1, None) == -1 and bad(9, None) == -1
+    assert bad(3, 0) == -2 and bad(5, 0) == -2
+    assert bad(6, 5) == -3 and bad(7, 0) == -3
+    assert bad(2, 7) == -4
+    assert bad(8, 2) == -2                           # unknown flag bit
+    assert bad(14, 1) == -6 and bad(15, 1) == -6     # capacity < offset + Nb
+    assert bad(0, P + 2) == -5                       # key pointer not 8-byte aligned
+    for i, s in enumerate([(8 * 256 * 128, 256 * 128, 128, 2), (8 * 256 * 128, 256 * 128, 64, 1),
+                           (8 * 256 * 128 + 2, 256 * 128, 128, 1)]):
+        st = (ctypes.c_int64 * 4)(*s)
+        a = list(ok); a[1] = ctypes.cast(st, ctypes.c_void_p)
+        assert lib.pq_validate_quantize_groups(*a) == (-6 if i < 2 else -5)
+    # transposed [B,L,Nk,128] view: token stride Nk*128
+    st = (ctypes.c_int64 * 4)(256 * 8 * 128, 128, 8 * 128, 1)
+    a = list(ok); a[1] = ctypes.cast(st, ctypes.c_void_p)
+    assert lib.pq_validate_quantize_groups(*a) == 0
+
+
+def test_validate_decode_attn_and_plan(lib):
+    B, N, Nk, ns = 2, 32, 8, 4
+    wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
+    assert wsb == B * N * ns * 132 * 4
+    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, 1024, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, P, wsb, P]
+    assert lib.pq_validate_decode_attn(*ok) == 0
+
+    def bad(i, v):
+        a = list(ok); a[i] = v
+        return lib.pq_validate_decode_attn(*a)
+    assert bad(0, None) == -1 and bad(13, None) == -1 and bad(25, None) == -1 and bad(27, None) == -1
+    assert bad(1, None) == -1            # groups > 0 but no codes
+    assert bad(9, None) == -1            # residual > 0 but no residual keys
+    assert bad(7, 5) == -6               # n_groups > capacity
+    assert bad(11, 129) == -6            # n_resid > capacity
+    assert bad(14, 3 * 128 + 4) == -6    # V capacity below tokens
+    assert bad(24, 0) == -7 and bad(26, wsb - 1) == -7
+    assert bad(20, 5) == -2 and bad(22, 5) == -3 and bad(23, 3) == -4
+    assert bad(13, P + 8) == -5
+    a = list(ok); a[15] = P; a[16] = 100          # mask row shorter than the context
+    assert lib.pq_validate_decode_attn(*a) == -6
+    # no quantized groups yet: codes may be NULL
+    a = list(ok); a[1:6] = [None] * 5; a[6] = 0; a[7] = 0
+    assert lib.pq_validate_decode_attn(*a) == 0
+    # plan: fills 4 wavefront slots per CU exactly once, never more splits than groups
+    assert lib.pq_decode_attn_plan(16, 8, 256, 256) == 8
+    assert lib.pq_decode_attn_plan(1, 8, 1024, 256) == 128
+    assert lib.pq_decode_attn_plan(64, 4, 64, 256) == 4
+    assert lib.pq_decode_attn_plan(1, 8, 3, 256) == 3
+    assert lib.pq_decode_attn_plan(512, 8, 64, 256) == 1
+    assert lib.pq_decode_attn_merge(None, 0, 1, 1, 1, 0, None, None) == -1
+
+
+def test_python_wrappers_refuse_cpu_tensors():
+    import torch
+    from polarquant_amd.attention import polar_decode_attention
+    from polarquant_amd.kernel4group import attention_decode_forward_triton_impl
+    from polarquant_amd.quantize import quantize_and_pack_nbit
+    k = torch.zeros(1, 1, 128, 128, dtype=torch.float16)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        quantize_and_pack_nbit(k)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        attention_decode_forward_triton_impl(k[:, :, :1], torch.zeros(1, 1, 1, 128, 64, dtype=torch.uint8), *[k[:, :, :1, :64].unsqueeze(2)] * 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        polar_decode_attention(k[:, :, :1], None, None, None, None, None, k, k, 0, 1)

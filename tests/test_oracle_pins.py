@@ -1,0 +1,271 @@
+"""Pins for the CPU oracle (oracle/polar_oracle.py, oracle/polar_oracle.c).
+
+The reference ships no tests, fixtures or golden vectors for this path, so every
+pin here is built from what the mathematics fixes: closed-form known answers,
+invariants of min/max quantization, error bounds, brute force in fp64 / pure
+python, library routines (torch.matmul, torch.softmax, HF rotate_half), and the
+agreement of two independent restatements (torch vs plain C).  None of the checks
+retypes the oracle's own formula.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import c_oracle as co
+from oracle import polar_oracle as po
+from polarquant_amd import workloads as wl
+
+
+def _keys(B, Nk, L, seed, dtype=torch.float16, theta=1e4):
+    g = torch.Generator().manual_seed(seed)
+    return wl.make_keys(B, Nk, L, theta, g, dtype), g
+
+
+# ------------------------------------------------------------------ quantizer
+def test_quantizer_known_answer_group():
+    """Keys placed on exact bin centres: the codes are known in closed form.
+    Pair d of token i is r_i (cos a_i, sin a_i) with a_i = a0 + (k_i + 0.5) * w, r_i = r0 + (m_i + 0.5) * u,
+    plus two tokens pinning the range ends; fp16 rounding of x, y moves the angle by ~1e-3 rad,
+    far less than half a bin."""
+    tb, rb = 4, 4
+    G, D = 128, 64
+    a0, a1, r0, r1 = 0.5, 2.5, 1.0, 3.0
+    w, u = (a1 - a0) / 2 ** tb, (r1 - r0) / 2 ** rb
+    g = torch.Generator().manual_seed(0)
+    kk = torch.randint(0, 2 ** tb, (G, D), generator=g)
+    mm = torch.randint(0, 2 ** rb, (G, D), generator=g)
+    ang = a0 + (kk.double() + 0.5) * w
+    rad = r0 + (mm.double() + 0.5) * u
+    # token 0 / 1 carry the extreme angle and radius of every pair
+    ang[0], rad[0], kk[0], mm[0] = a0, r0, 0, 0
+    ang[1], rad[1], kk[1], mm[1] = a1, r1, 2 ** tb - 1, 2 ** rb - 1
+    x, y = rad * torch.cos(ang), rad * torch.sin(ang)
+    keys = torch.cat([x, y], dim=-1).to(torch.float16).reshape(1, 1, G, 2 * D)
+    want = ((mm << tb) + kk).to(torch.uint8)
+    for quant in (po.quantize_and_pack_nbit, co.quantize):
+        codes, rscale, rmn, tscale, tmn = quant(keys, rb, tb)
+        assert torch.equal(codes[0, 0, 0], want)
+        assert torch.allclose(tmn.float(), torch.full_like(tmn.float(), a0), atol=2e-3)
+        assert torch.allclose(rmn.float(), torch.full_like(rmn.float(), r0), atol=2e-3)
+        assert torch.allclose(tscale.float(), torch.full_like(tscale.float(), w), atol=2e-4)
+        assert torch.allclose(rscale.float(), torch.full_like(rscale.float(), u), atol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (2, 5)])
+def test_quantizer_invariants(dtype, rbits, tbits):
+    k, _ = _keys(2, 3, 256, 1, dtype)
+    codes, rscale, rmn, tscale, tmn = po.quantize_and_pack_nbit(k, rbits, tbits)
+    theta, rho = codes & (2 ** tbits - 1), codes >> tbits
+    assert int(codes.max()) < 2 ** (rbits + tbits)
+    ks = k.reshape(2, 3, 2, 128, 2, 64).float()
+    x, y = ks[..., 0, :], ks[..., 1, :]
+    rad = torch.sqrt(x * x + y * y)
+    # the token with the smallest radius gets rho == 0, the largest gets the top code (clamp of exactly 2^b)
+    assert bool((rho.gather(3, rad.argmin(3, keepdim=True)) == 0).all())
+    assert bool((rho.gather(3, rad.argmax(3, keepdim=True)) == 2 ** rbits - 1).all())
+    phi = torch.atan2(y.double(), x.double())
+    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)
+    assert bool((theta.gather(3, phi.argmin(3, keepdim=True)) == 0).all())
+    assert bool((theta.gather(3, phi.argmax(3, keepdim=True)) == 2 ** tbits - 1).all())
+    # scale * 2^b reproduces the range up to the dtype's rounding
+    eps = 2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7
+    rng = (phi.amax(3, keepdim=True) - phi.amin(3, keepdim=True)).float()
+    assert bool(((tscale.float() * 2 ** tbits - rng).abs() <= 8 * eps * rng.clamp_min(1.0)).all())
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, 2e-3), (torch.bfloat16, 3e-2)])
+def test_dequantize_error_bounds(dtype, tol):
+    """|phi - phi^| <= tscale/2 and |r - r^| <= rscale/2, up to the dtype's rounding of the intermediates."""
+    k, _ = _keys(1, 2, 256, 2, dtype)
+    q = po.quantize_and_pack_nbit(k, 4, 4)
+    codes, rscale, rmn, tscale, tmn = q
+    khat = po.dequantize_keys(*q, dtype=torch.float64).reshape(1, 2, 2, 128, 2, 64)
+    ks = k.reshape(1, 2, 2, 128, 2, 64).double()
+    r, rh = ks.pow(2).sum(-2).sqrt(), khat.pow(2).sum(-2).sqrt()
+    assert bool(((r - rh).abs() <= rscale.double() / 2 + tol * (1 + r)).all())
+    phi = torch.atan2(ks[..., 1, :], ks[..., 0, :]); phi = torch.where(phi < 0, phi + 2 * math.pi, phi)
+    ph = torch.atan2(khat[..., 1, :], khat[..., 0, :]); ph = torch.where(ph < 0, ph + 2 * math.pi, ph)
+    d = (phi - ph).abs(); d = torch.minimum(d, 2 * math.pi - d)
+    assert bool((d <= tscale.double() / 2 + tol * 4).all())
+
+
+def test_quantizer_vs_fp64_brute_force_counts_edge_flips():
+    """The half-precision eager quantizer against exact-ish fp64 arithmetic: they may
+    only disagree by one bin, on elements that sit on a bin edge ("edge flips")."""
+    k, _ = _keys(1, 4, 512, 3)
+    codes = po.quantize_and_pack_nbit(k, 4, 4)[0]
+    brute = po.quantize_brute_fp64(k, 4, 4)[0]
+    dt = (codes & 15).int() - (brute & 15).int()
+    dr = (codes >> 4).int() - (brute >> 4).int()
+    assert int(dt.abs().max()) <= 1 and int(dr.abs().max()) <= 1
+    flips = int((codes != brute).sum())
+    print("edge flips half-vs-fp64: %d of %d" % (flips, codes.numel()))
+    assert flips < 0.03 * codes.numel()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (5, 3)])
+def test_c_and_torch_restatements_agree(dtype, rbits, tbits):
+    """Two independent restatements (torch eager ops with SLEEF atan2 / scalar C with libm atan2f)."""
+    k, _ = _keys(2, 4, 1024, 4, dtype)
+    a = po.quantize_and_pack_nbit(k, rbits, tbits)
+    b = co.quantize(k, rbits, tbits)
+    assert all(x.shape == y.shape for x, y in zip(a, b))
+    # radius side shares no transcendental: bit-exact
+    assert torch.equal(a[1].view(torch.int16), b[1].view(torch.int16))
+    assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
+    # angle side: a last-ulp difference of the two arctangents can move a value across a rounding tie
+    flips = int((a[0] != b[0]).sum())
+    meta = int((a[3].view(torch.int16) != b[3].view(torch.int16)).sum()) + int((a[4].view(torch.int16) != b[4].view(torch.int16)).sum())
+    print("torch-vs-C flips: codes %d / %d, angle metadata %d" % (flips, a[0].numel(), meta))
+    assert flips <= 1e-4 * a[0].numel() and meta <= 8
+
+
+def test_rope_pair_convention_matches_hf_rotate_half():
+    """x = dims [0,64), y = dims [64,128) is the HF rotate-half pairing: rotating a
+    key by RoPE turns pair (d, d+64) by the angle pos * inv_freq[d] and keeps its radius."""
+    hf = pytest.importorskip("transformers.models.llama.modeling_llama")
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(1, 2, 16, 128, generator=g)
+    cos, sin = po.rope_cos_sin(torch.arange(16), 128, 1e4)
+    ours = po.apply_rope(x, cos, sin)
+    theirs = x * cos + hf.rotate_half(x) * sin
+    assert torch.equal(ours, theirs)
+    assert torch.equal(wl._rope(x, cos, sin), theirs)
+    inv = 1.0 / (1e4 ** (torch.arange(0, 128, 2).float() / 128))
+    a0 = torch.atan2(x[..., 64:], x[..., :64]).double()
+    a1 = torch.atan2(ours[..., 64:], ours[..., :64]).double()
+    turn = (torch.arange(16).double()[:, None] * inv.double()[None, :])
+    d = torch.remainder(a1 - a0 - turn + math.pi, 2 * math.pi) - math.pi
+    assert float(d.abs().max()) < 1e-5
+    assert torch.allclose(x[..., :64] ** 2 + x[..., 64:] ** 2, ours[..., :64] ** 2 + ours[..., 64:] ** 2, atol=1e-4)
+
+
+# --------------------------------------------------------------------- scores
+def test_scores_vs_pure_python_lut_loop():
+    k, g = _keys(1, 2, 256, 6)
+    q = wl.make_half((1, 4, 1, 128), g)
+    quant = po.quantize_and_pack_nbit(k, 4, 4)
+    s = po.decode_scores(q, *quant, dtype=torch.float64)
+    for h, grp in [(0, 0), (3, 1)]:
+        brute = torch.tensor(po.decode_scores_lut_python(q, *quant, 4, 4, 0, h, grp), dtype=torch.float64)
+        assert torch.allclose(s[0, h, 0, grp * 128:(grp + 1) * 128], brute, rtol=0, atol=1e-9)
+
+
+def test_scores_polar_identity():
+    """q . K^ = sum_d |q_d| r^ cos(phi^ - psi_d): the angle table in polar form."""
+    k, g = _keys(1, 1, 128, 7)
+    q = wl.make_half((1, 1, 1, 128), g)
+    quant = po.quantize_and_pack_nbit(k, 4, 4)
+    codes, rscale, rmn, tscale, tmn = quant
+    s = po.decode_scores(q, *quant, dtype=torch.float64)[0, 0, 0]
+    qx, qy = q[0, 0, 0, :64].double(), q[0, 0, 0, 64:].double()
+    qn, psi = torch.sqrt(qx * qx + qy * qy), torch.atan2(qy, qx)
+    phi = tscale[0, 0, 0].double() * ((codes[0, 0, 0] & 15).double() + 0.5) + tmn[0, 0, 0].double()
+    rad = rscale[0, 0, 0].double() * ((codes[0, 0, 0] >> 4).double() + 0.5) + rmn[0, 0, 0].double()
+    alt = (qn * rad * torch.cos(phi - psi)).sum(-1)
+    assert torch.allclose(s, alt, rtol=0, atol=1e-9)
+
+
+@pytest.mark.parametrize("N,Nk", [(8, 8), (8, 2), (7, 1)])
+def test_scores_c_vs_torch_and_gqa_mapping(N, Nk):
+    k, g = _keys(2, Nk, 256, 8)
+    q = wl.make_half((2, N, 1, 128), g)
+    quant = po.quantize_and_pack_nbit(k, 3, 3)
+    s_t = po.decode_scores(q, *quant, rbits=3, tbits=3, dtype=torch.float64)
+    s_c = co.scores(q, *quant, rbits=3, tbits=3)
+    assert float((s_t - s_c.double()).abs().max()) < 1e-4
+    # query head h must read KV head h // rep (repeat-interleave): score it alone against that head
+    rep = N // Nk
+    for h in (0, N - 1):
+        one = po.decode_scores(q[:, h:h + 1], *[t[:, h // rep:h // rep + 1] for t in quant], rbits=3, tbits=3,
+                               dtype=torch.float64)
+        # BLAS may block the two matmuls differently: equal to rounding, not bit-for-bit
+        assert torch.allclose(one[:, 0], s_t[:, h], rtol=0, atol=1e-10)
+
+
+def test_scores_approximate_the_unquantized_keys():
+    """Sanity of the whole quantize -> score chain: 4/4-bit polar keys reproduce q.K^T to a few percent."""
+    k, g = _keys(1, 4, 512, 9)
+    q = wl.make_half((1, 4, 1, 128), g)
+    quant = po.quantize_and_pack_nbit(k, 4, 4)
+    s = po.decode_scores(q, *quant, dtype=torch.float64)
+    exact = torch.matmul(q.double(), k.double().transpose(2, 3))
+    rel = (s - exact).norm() / exact.norm()
+    assert float(rel) < 0.12
+
+
+# ------------------------------------------------------------------ attention
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_attention_three_ways(with_mask):
+    """Literal restatement vs one-shot fp64 softmax over concatenated keys vs the C loop."""
+    B, N, Nk, ng, nr = 2, 8, 2, 2, 37
+    k, g = _keys(B, Nk, ng * 128 + nr, 10)
+    q = wl.make_half((B, N, 1, 128), g)
+    v = wl.make_half((B, Nk, ng * 128 + nr, 128), g)
+    quant = po.quantize_and_pack_nbit(k[:, :, :ng * 128].contiguous(), 4, 4)
+    kres = k[:, :, ng * 128:].contiguous()
+    mask = None
+    if with_mask:
+        mask = torch.ones(B, ng * 128 + nr, dtype=torch.int64)
+        mask[0, :70] = 0
+        mask[1, :5] = 0
+    a = po.decode_attention(q, kres, *quant, v, mask)
+    b = po.decode_attention_exact(q, kres, *quant, v, mask)
+    c = co.decode_attn(q, *quant, kres, v, mask)
+    assert float((a.double() - b).abs().max()) < 2e-3
+    assert float((c.double() - b).abs().max()) < 2e-3
+    assert float((a.double() - c.double()).abs().max()) < 2e-3
+
+
+def test_fp16_baseline_is_plain_softmax_attention():
+    k, g = _keys(1, 2, 200, 11)
+    q = wl.make_half((1, 4, 1, 128), g)
+    v = wl.make_half((1, 2, 200, 128), g)
+    out = po.fp16_decode_attention(q, k, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), po.repeat_kv(k, 2).float(), po.repeat_kv(v, 2).float())
+    assert float((out.float() - ref).abs().max()) < 5e-3
+
+
+# ---------------------------------------------------------- cache bookkeeping
+@pytest.mark.parametrize("L", [1, 127, 128, 129, 300, 384])
+def test_prefill_cache_split(L):
+    k, g = _keys(1, 2, L, 12)
+    v = wl.make_half((1, 2, L, 128), g)
+    kf, ind, rs, rm, ts, tm, vv, n = po.prefill_cache(k, v)
+    nq = 0 if L < 128 else L - L % 128
+    assert n == L and vv.shape[2] == L
+    assert (ind is None) == (nq == 0)
+    if nq:
+        assert ind.shape == (1, 2, nq // 128, 128, 64) and rs.shape == (1, 2, nq // 128, 1, 64)
+    assert (kf is None) == (L % 128 == 0)
+    if kf is not None:
+        assert kf.shape[2] == L - nq and torch.equal(kf, k[:, :, nq:])
+
+
+def test_decode_steps_bookkeeping_and_equivalence():
+    """n decode steps from a prompt: quantized tokens = L - L%128 + 128*flushes, residual in [0,127]
+    after every step, kv_seq_len = L + n; and every step's output equals one-shot attention over
+    the dequantized cache + residual keys (softmax over all L + n tokens)."""
+    L, steps = 250, 140
+    k, g = _keys(1, 2, L + steps, 13)
+    v = wl.make_half((1, 2, L + steps, 128), g)
+    qs = wl.make_half((1, 4, steps, 128), g)
+    cache = po.prefill_cache(k[:, :, :L], v[:, :, :L])
+    for i in range(steps):
+        t = L + i
+        out, cache = po.decode_step(qs[:, :, i:i + 1], k[:, :, t:t + 1], v[:, :, t:t + 1], cache)
+        kf, ind = cache[0], cache[1]
+        nres = 0 if kf is None else kf.shape[2]
+        nq = 0 if ind is None else ind.shape[2] * 128
+        assert cache[-1] == t + 1 and cache[6].shape[2] == t + 1
+        assert 0 <= nres <= 127 and nq + nres == t + 1 and nq % 128 == 0
+        if i in (0, 5, 6, steps - 1):
+            # tokens that were quantized at the time of THIS step's scoring: the flush happens after scoring
+            nq_before = ((t + 1) // 128) * 128 if (t + 1) % 128 else t + 1 - 128
+            nq_before = max(nq_before, 0) if L >= 128 or t + 1 > 128 else 0
+            quant = po.quantize_and_pack_nbit(k[:, :, :nq_before].contiguous()) if nq_before else (None,) * 5
+            ref = po.decode_attention_exact(qs[:, :, i:i + 1], k[:, :, nq_before:t + 1], *quant, v[:, :, :t + 1])
+            assert float((out.double() - ref).abs().max()) < 2e-3
