@@ -1,0 +1,487 @@
+"""Host-side mirror of the reference's polar attention classes and model shell.
+
+Reference interfaces mirrored here (same names, argument meaning, return values):
+  * `*PolarGroupAttention.forward(hidden_states, attention_mask=None, past_key_value=None,
+    position_embeddings=None, **kwargs) -> (attn_output, past_key_value)` with the 8-tuple cache
+    `(key_states_full | None, indices | None, rscale, rmn, tscale, tmn, value_states_full, kv_seq_len)`
+    (models/modeling_llama_polar.py:31-157, models/modeling_qwen_polar.py:30-156);
+  * `*PolarDecoderLayer`, `*PolarModel`, `*PolarForCausalLM` (modeling_llama_polar.py:447-562);
+  * `generate`, `sample`, `top_k_top_p_filtering` (modeling_llama_polar.py:565-666).
+
+Differences that do not show at the interface: the decode branch is ONE fused HIP
+launch pair (scores + softmax + P.V, then the split merge) instead of ~12 eager
+kernels, and the cache tensors handed back in the tuple are views into a
+pre-allocated per-layer arena, so appending a token or a quantized group is O(1)
+instead of a torch.cat of the whole cache (reference :86-90,98).  The tuple is a
+`PolarCache` (a tuple subclass) that remembers its arena; a plain tuple in the
+reference's format is accepted too and is copied into a fresh arena.
+
+The modules are self-contained torch.nn modules whose parameter names match the
+HF Llama / Qwen2 checkpoints (model.layers.N.self_attn.q_proj.weight, ...), so a
+HF state_dict loads with load_state_dict; they do not import `transformers`.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .attention import polar_decode_attention
+from .quantize import quantize_and_pack_nbit
+
+GROUP = 128
+
+
+# ----------------------------------------------------------------------------- config
+@dataclass
+class PolarConfig:
+    hidden_size: int = 4096
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    num_hidden_layers: int = 32
+    intermediate_size: int = 14336
+    vocab_size: int = 128256
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 500000.0
+    head_dim: int = 128
+    attention_bias: bool = False        # q/k/v bias (Qwen2: True)
+    mlp_bias: bool = False
+    tie_word_embeddings: bool = False
+    eos_token_id: List[int] = field(default_factory=lambda: [128001])
+    # polar cache
+    rbits: int = 4
+    tbits: int = 4
+    cache_capacity: int = 0             # tokens to pre-allocate per layer (0: prompt + 1024, grown by doubling)
+
+    @staticmethod
+    def llama3_8b(**kw) -> "PolarConfig":
+        return PolarConfig(**kw)
+
+    @staticmethod
+    def llama2_7b(**kw) -> "PolarConfig":
+        return PolarConfig(num_key_value_heads=32, intermediate_size=11008, vocab_size=32000, rope_theta=1e4,
+                           eos_token_id=[2], **kw)
+
+    @staticmethod
+    def qwen25_7b(**kw) -> "PolarConfig":
+        return PolarConfig(hidden_size=3584, num_attention_heads=28, num_key_value_heads=4, num_hidden_layers=28,
+                           intermediate_size=18944, vocab_size=152064, rms_norm_eps=1e-6, rope_theta=1e6,
+                           attention_bias=True, eos_token_id=[151645, 151643], **kw)
+
+
+def _cfg(config, name, default=None):
+    return getattr(config, name, default)
+
+
+# ----------------------------------------------------------------------------- rope helpers (HF conventions)
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    x1, x2 = x[..., : x.shape[-1] // 2], x[..., x.shape[-1] // 2:]
+    return torch.cat((-x2, x1), dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim: int = 1):
+    cos, sin = cos.unsqueeze(unsqueeze_dim), sin.unsqueeze(unsqueeze_dim)
+    return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
+
+
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+    b, h, s, d = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    return hidden_states[:, :, None, :, :].expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
+
+
+def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
+    """(models/modeling_llama_polar.py:23-28) kept for callers that expand the code cache themselves;
+    the HIP kernels handle any GQA ratio natively and never need it."""
+    b, h, nb, s, d = hidden_states.shape
+    if n_rep == 1:
+        return hidden_states
+    return hidden_states[:, :, None].expand(b, h, n_rep, nb, s, d).reshape(b, h * n_rep, nb, s, d)
+
+
+class RotaryEmbedding(nn.Module):
+    def __init__(self, head_dim: int, base: float):
+        super().__init__()
+        inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+        self.register_buffer("inv_freq", inv_freq, persistent=False)
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, position_ids: torch.Tensor):
+        freqs = position_ids[:, :, None].float() * self.inv_freq[None, None, :].float().to(x.device)
+        emb = torch.cat((freqs, freqs), dim=-1)
+        return emb.cos().to(x.dtype), emb.sin().to(x.dtype)
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden_size: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.variance_epsilon = eps
+
+    def forward(self, x):
+        dt = x.dtype
+        x = x.float()
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * x.to(dt)
+
+
+class MLP(nn.Module):
+    def __init__(self, config):
+        super().__init__()
+        h, i, b = config.hidden_size, config.intermediate_size, _cfg(config, "mlp_bias", False)
+        self.gate_proj = nn.Linear(h, i, bias=b)
+        self.up_proj = nn.Linear(h, i, bias=b)
+        self.down_proj = nn.Linear(i, h, bias=b)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+# ----------------------------------------------------------------------------- cache
+class _Arena:
+    """Pre-allocated per-layer polar KV cache.  codes/meta/v grow by doubling."""
+
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits):
+        self.B, self.Nk, self.dtype, self.device = B, Nk, dtype, device
+        self.rbits, self.tbits = rbits, tbits
+        self.n_groups = self.n_resid = self.kv_len = 0
+        self.kres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
+        self._alloc(max(capacity_tokens, GROUP))
+
+    def _alloc(self, cap_tokens):
+        gcap = (cap_tokens + GROUP - 1) // GROUP
+        vcap = gcap * GROUP + GROUP
+        B, Nk, dev, dt = self.B, self.Nk, self.device, self.dtype
+        codes = torch.empty(B, Nk, gcap, GROUP, 64, dtype=torch.uint8, device=dev)
+        meta = [torch.empty(B, Nk, gcap, 1, 64, dtype=dt, device=dev) for _ in range(4)]
+        v = torch.empty(B, Nk, vcap, 128, dtype=dt, device=dev)
+        if self.kv_len:
+            codes[:, :, :self.n_groups] = self.codes[:, :, :self.n_groups]
+            for new, old in zip(meta, self.meta):
+                new[:, :, :self.n_groups] = old[:, :, :self.n_groups]
+            v[:, :, :self.kv_len] = self.v[:, :, :self.kv_len]
+        self.codes, self.meta, self.v, self.gcap, self.vcap = codes, meta, v, gcap, vcap
+
+    def reserve(self, tokens):
+        if tokens > self.vcap or (tokens // GROUP) > self.gcap:
+            self._alloc(max(2 * self.vcap, tokens))
+
+    def quantize_into(self, keys):
+        """keys [B,Nk,n*128,128] (any strides with unit dim stride) -> groups appended."""
+        n = keys.shape[2] // GROUP
+        quantize_and_pack_nbit(keys, self.rbits, self.tbits, out=(self.codes, *self.meta), group_offset=self.n_groups)
+        self.n_groups += n
+
+    def as_tuple(self) -> "PolarCache":
+        kf = self.kres[:, :, :self.n_resid] if self.n_resid else None
+        if self.n_groups:
+            q5 = [self.codes[:, :, :self.n_groups]] + [m[:, :, :self.n_groups] for m in self.meta]
+        else:
+            q5 = [None] * 5
+        return PolarCache((kf, *q5, self.v[:, :, :self.kv_len], self.kv_len), self)
+
+
+class PolarCache(tuple):
+    """The reference's 8-tuple, plus the arena its tensors are views of."""
+
+    def __new__(cls, items, arena):
+        obj = super().__new__(cls, items)
+        obj.arena = arena
+        return obj
+
+
+_MASK_CACHE = {"key": None, "u8": None}
+
+
+def _mask_u8(mask: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """attention_mask [B, L] of {0,1} (any dtype) -> uint8, converted once per step, not once per layer."""
+    if mask is None:
+        return None
+    if mask.dtype == torch.uint8:
+        return mask
+    key = (mask.data_ptr(), tuple(mask.shape), mask._version, mask.dtype)
+    if _MASK_CACHE["key"] != key:
+        _MASK_CACHE["key"], _MASK_CACHE["u8"] = key, (mask != 0).to(torch.uint8)
+    return _MASK_CACHE["u8"]
+
+
+# ----------------------------------------------------------------------------- attention
+class PolarGroupAttention(nn.Module):
+    """Polar-key attention with the reference's forward signature and cache tuple."""
+
+    def __init__(self, config, layer_idx: Optional[int] = None):
+        super().__init__()
+        self.config, self.layer_idx = config, layer_idx
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.head_dim = _cfg(config, "head_dim", None) or self.hidden_size // self.num_heads
+        self.num_key_value_heads = _cfg(config, "num_key_value_heads", self.num_heads)
+        self.num_key_value_groups = self.num_heads // self.num_key_value_heads
+        self.is_causal = True
+        qkv_bias = _cfg(config, "attention_bias", False)
+        self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=qkv_bias)
+        self.k_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=qkv_bias)
+        self.v_proj = nn.Linear(self.hidden_size, self.num_key_value_heads * self.head_dim, bias=qkv_bias)
+        self.o_proj = nn.Linear(self.num_heads * self.head_dim, self.hidden_size, bias=False)
+        # reference :34-37
+        self.rbits = _cfg(config, "rbits", 4)
+        self.tbits = _cfg(config, "tbits", 4)
+        self.group_size = 128
+        self.residual_length = 128
+        self.capture = None   # test hook: a list that receives post-RoPE (q, k, v) of every call
+
+    # -- cache plumbing --------------------------------------------------------
+    def _new_arena(self, B, dtype, device, tokens):
+        cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
+        return _Arena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits)
+
+    def _arena_of(self, past_key_value, dtype, device) -> _Arena:
+        arena = getattr(past_key_value, "arena", None)
+        if arena is not None and arena.kv_len == past_key_value[-1]:
+            return arena
+        # a plain tuple in the reference's format: copy it into a fresh arena
+        kf, ind, rs, rm, ts, tm, v, n = past_key_value
+        arena = self._new_arena(v.shape[0], dtype, device, n + 1)
+        if ind is not None:
+            g = ind.shape[2]
+            arena.codes[:, :, :g] = ind
+            for dst, src in zip(arena.meta, (rs, rm, ts, tm)):
+                dst[:, :, :g] = src
+            arena.n_groups = g
+        if kf is not None:
+            arena.kres[:, :, :kf.shape[2]] = kf
+            arena.n_resid = kf.shape[2]
+        arena.v[:, :, :n] = v
+        arena.kv_len = n
+        return arena
+
+    # -- forward (reference :39-133) ---------------------------------------------
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_value=None, position_embeddings: Tuple[torch.Tensor, torch.Tensor] = None, **kwargs):
+        bsz, q_len, _ = hidden_states.size()
+        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = position_embeddings
+        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        if self.capture is not None:
+            self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
+
+        if q_len == 1:   # decoding time (:61-101)
+            arena = self._arena_of(past_key_value, query_states.dtype, query_states.device)
+            arena.reserve(arena.kv_len + 1)
+            arena.kres[:, :, arena.n_resid] = key_states[:, :, 0]          # :77
+            arena.v[:, :, arena.kv_len] = value_states[:, :, 0]            # :98
+            arena.n_resid += 1
+            arena.kv_len += 1
+            attn_output = polar_decode_attention(
+                query_states, arena.codes if arena.n_groups else None, *(arena.meta if arena.n_groups else [None] * 4),
+                arena.kres, arena.v, arena.n_groups, arena.n_resid, attention_mask=_mask_u8(attention_mask),
+                rbits=self.rbits, tbits=self.tbits, sm_scale=1.0 / math.sqrt(self.head_dim))   # :66-99
+            if arena.n_resid % self.residual_length == 0:                  # :83-92
+                arena.quantize_into(arena.kres)
+                arena.n_resid = 0
+            past_key_value = arena.as_tuple()                              # :101
+        else:            # pre-filling (:102-128)
+            assert past_key_value is None
+            kv_seq_len = key_states.shape[2]
+            attn_output = _prefill_attention(query_states, key_states, value_states, attention_mask,
+                                             self.num_key_value_groups, self.is_causal)
+            arena = self._new_arena(bsz, key_states.dtype, key_states.device, kv_seq_len + 1)
+            residual_length = kv_seq_len % self.residual_length
+            n_quant = kv_seq_len - residual_length if kv_seq_len >= self.residual_length else 0
+            if n_quant:
+                arena.quantize_into(key_states[:, :, :n_quant])            # :124-126 (read in place, strided)
+            if kv_seq_len - n_quant:
+                arena.kres[:, :, :kv_seq_len - n_quant] = key_states[:, :, n_quant:]
+            arena.n_resid = kv_seq_len - n_quant
+            arena.v[:, :, :kv_seq_len] = value_states
+            arena.kv_len = kv_seq_len
+            past_key_value = arena.as_tuple()                              # :128
+
+        attn_output = attn_output.reshape(bsz, q_len, -1).contiguous()
+        attn_output = self.o_proj(attn_output)
+        return attn_output, past_key_value
+
+    def quantize_and_pack_nbit(self, key_states):
+        """(reference :135-157) -> (indices, rscale, rmn, tscale, tmn)."""
+        return quantize_and_pack_nbit(key_states, self.rbits, self.tbits, self.group_size)
+
+
+def _prefill_attention(q, k, v, attention_mask, n_rep, is_causal):
+    """Causal prompt attention; returns [B, L, N, hd] like the reference's flash-attention call (:106-114).
+    `attention_mask` [B, L] of {0,1} marks left padding."""
+    B, N, L, hd = q.shape
+    if attention_mask is None or bool((attention_mask != 0).all()):
+        out = F.scaled_dot_product_attention(q, k, v, is_causal=is_causal and L > 1, enable_gqa=n_rep > 1)
+    else:
+        keep = (attention_mask != 0)[:, None, None, :]
+        causal = torch.ones(L, L, dtype=torch.bool, device=q.device).tril()[None, None]
+        m = keep & causal
+        m = m | torch.eye(L, dtype=torch.bool, device=q.device)[None, None]   # padded query rows: attend to self
+        out = F.scaled_dot_product_attention(q, k, v, attn_mask=m, enable_gqa=n_rep > 1)
+    return out.transpose(1, 2)
+
+
+# ----------------------------------------------------------------------------- model shell
+@dataclass
+class CausalLMOutputWithPast:
+    logits: torch.Tensor = None
+    past_key_values: tuple = None
+
+
+class PolarDecoderLayer(nn.Module):
+    attention_class = PolarGroupAttention
+
+    def __init__(self, config, layer_idx):
+        super().__init__()
+        self.config, self.layer_idx = config, layer_idx
+        self.hidden_size = config.hidden_size
+        self.self_attn = self.attention_class(config, layer_idx)
+        self.mlp = MLP(config)
+        self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, hidden_states, attention_mask=None, past_key_value=None, position_embeddings=None, **kwargs):
+        residual = hidden_states
+        hidden_states = self.input_layernorm(hidden_states)
+        hidden_states, present_key_value = self.self_attn(
+            hidden_states=hidden_states, attention_mask=attention_mask, past_key_value=past_key_value,
+            position_embeddings=position_embeddings, **kwargs)
+        hidden_states = residual + hidden_states
+        residual = hidden_states
+        hidden_states = self.post_attention_layernorm(hidden_states)
+        hidden_states = self.mlp(hidden_states)
+        hidden_states = residual + hidden_states
+        return (hidden_states, present_key_value)
+
+
+class PolarModel(nn.Module):
+    layer_class = PolarDecoderLayer
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList([self.layer_class(config, i) for i in range(config.num_hidden_layers)])
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        head_dim = _cfg(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
+        self.rotary_emb = RotaryEmbedding(head_dim, _cfg(config, "rope_theta", 10000.0))
+
+    def forward(self, input_ids=None, attention_mask=None, past_key_values=None):
+        bsz, q_len = input_ids.shape
+        next_decoder_cache = ()
+        inputs_embeds = self.embed_tokens(input_ids)
+        past_seen_tokens = 0 if past_key_values is None else past_key_values[0][-1]          # reference :501
+        cache_position = torch.arange(past_seen_tokens, past_seen_tokens + q_len, device=inputs_embeds.device)
+        hidden_states = inputs_embeds
+        position_embeddings = self.rotary_emb(hidden_states, cache_position.unsqueeze(0))
+        for layer_idx, decoder_layer in enumerate(self.layers):
+            hidden_states, past_key_value = decoder_layer(
+                hidden_states, attention_mask=attention_mask,
+                past_key_value=past_key_values[layer_idx] if past_key_values is not None else None,
+                position_embeddings=position_embeddings)
+            next_decoder_cache += (past_key_value,)
+        hidden_states = self.norm(hidden_states)
+        return hidden_states, next_decoder_cache
+
+
+class PolarForCausalLM(nn.Module):
+    model_class = PolarModel
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.model = self.model_class(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        if _cfg(config, "tie_word_embeddings", False):
+            self.lm_head.weight = self.model.embed_tokens.weight
+
+    @property
+    def device(self):
+        return next(self.parameters()).device
+
+    def forward(self, input_ids=None, attention_mask=None, past_key_values=None, num_logits_to_keep=0,
+                return_dict=True):
+        hidden_states, past_key_values = self.model(input_ids=input_ids, attention_mask=attention_mask,
+                                                    past_key_values=past_key_values)
+        logits = self.lm_head(hidden_states[:, -num_logits_to_keep:, :])
+        return CausalLMOutputWithPast(logits=logits, past_key_values=past_key_values)
+
+    def kv_cache_bytes_per_token(self) -> int:
+        """Bytes one cached token costs across all layers: 1 code byte per pair, 4 metadata
+        halves per (group, pair) amortised over 128 tokens, fp16 V."""
+        c = self.config
+        nk = _cfg(c, "num_key_value_heads", c.num_attention_heads)
+        return c.num_hidden_layers * nk * (64 + 4 * 64 * 2 // 128 + 128 * 2)
+
+
+# ----------------------------------------------------------------------------- generation (reference :565-666)
+def top_k_top_p_filtering(logits, top_k: int = 0, top_p: float = 1.0, filter_value: float = -float("Inf"),
+                          min_tokens_to_keep: int = 1):
+    if top_k > 0:
+        top_k = min(max(top_k, min_tokens_to_keep), logits.size(-1))
+        indices_to_remove = logits < torch.topk(logits, top_k)[0][..., -1, None]
+        logits[indices_to_remove] = filter_value
+    if top_p < 1.0:
+        sorted_logits, sorted_indices = torch.sort(logits, descending=True)
+        cumulative_probs = torch.cumsum(F.softmax(sorted_logits, dim=-1), dim=-1)
+        sorted_indices_to_remove = cumulative_probs > top_p
+        if min_tokens_to_keep > 1:
+            sorted_indices_to_remove[..., :min_tokens_to_keep] = 0
+        sorted_indices_to_remove[..., 1:] = sorted_indices_to_remove[..., :-1].clone()
+        sorted_indices_to_remove[..., 0] = 0
+        indices_to_remove = sorted_indices_to_remove.scatter(1, sorted_indices, sorted_indices_to_remove)
+        logits[indices_to_remove] = filter_value
+    return logits
+
+
+def sample(logits, generation_config, do_sample=False):
+    if do_sample:
+        logits_ = top_k_top_p_filtering(logits.view(-1, logits.size(-1)) / generation_config.temperature,
+                                        top_k=generation_config.top_k, top_p=generation_config.top_p)
+        return torch.multinomial(logits_.softmax(-1), num_samples=1)
+    return torch.argmax(logits, dim=-1)
+
+
+@dataclass
+class GenerationConfig:
+    eos_token_id: List[int] = field(default_factory=lambda: [2])
+    top_k: int = 50
+    top_p: float = 1.0
+    temperature: float = 1.0
+
+
+def generate(model, input_ids, attention_mask, generation_config, do_sample=False, max_new_tokens=8):
+    current_input_ids = input_ids
+    batch_size = input_ids.size(0)
+    device = model.device
+    generate_ids = torch.zeros([batch_size, max_new_tokens], dtype=torch.long, device=device)
+    eos_sequence = torch.zeros([batch_size, 1], dtype=torch.bool, device=device)
+    eos = generation_config.eos_token_id
+    stop_tensor = torch.tensor(eos if isinstance(eos, (list, tuple)) else [eos], dtype=torch.long, device=device)
+    next_decoder_cache = None
+    with torch.no_grad():
+        step = 0
+        while True:
+            if step >= max_new_tokens:
+                break
+            outputs = model(input_ids=current_input_ids, attention_mask=attention_mask,
+                            past_key_values=next_decoder_cache, num_logits_to_keep=1)
+            output_ids = sample(outputs.logits, generation_config, do_sample=do_sample)
+            next_decoder_cache = outputs.past_key_values
+            generate_ids[:, step:step + 1] = output_ids
+            current_input_ids = output_ids
+            if attention_mask is not None:
+                attention_mask = torch.cat([attention_mask, torch.ones_like(output_ids)], dim=-1)
+            eos_sequence = eos_sequence | torch.isin(current_input_ids, stop_tensor)
+            if eos_sequence.sum().item() == batch_size:
+                break
+            step += 1
+    step = min(step + 1, max_new_tokens)
+    return generate_ids[:, :step]

@@ -1,0 +1,24 @@
+"""Llama polar-key attention and model shell under the reference's class names
+(models/modeling_llama_polar.py): LlamaPolarGroupAttention, LlamaPolarDecoderLayer,
+LlamaPolarModel, LlamaPolarForCausalLM, generate, sample, top_k_top_p_filtering."""
+from .kernel4group import attention_decode_forward_triton_impl  # noqa: F401  (re-exported, as the reference imports it here)
+from .modeling_common import (  # noqa: F401
+    CausalLMOutputWithPast, GenerationConfig, PolarCache, PolarConfig, PolarDecoderLayer, PolarForCausalLM,
+    PolarGroupAttention, PolarModel, apply_rotary_pos_emb, generate, repeat_kv, repeat_kv_quant, sample,
+    top_k_top_p_filtering)
+
+
+class LlamaPolarGroupAttention(PolarGroupAttention):
+    """q/k/v projections without bias unless config.attention_bias says otherwise (Llama)."""
+
+
+class LlamaPolarDecoderLayer(PolarDecoderLayer):
+    attention_class = LlamaPolarGroupAttention
+
+
+class LlamaPolarModel(PolarModel):
+    layer_class = LlamaPolarDecoderLayer
+
+
+class LlamaPolarForCausalLM(PolarForCausalLM):
+    model_class = LlamaPolarModel

@@ -1,0 +1,130 @@
+"""The drop-in attention classes and model shell on the GPU, checked against the CPU
+oracle's restatement of the reference forward (prefill split, decode step, flush)."""
+import math
+
+import pytest
+import torch
+
+from oracle import polar_oracle as po
+from polarquant_amd.modeling_common import PolarConfig
+from polarquant_amd.modeling_llama_polar import (GenerationConfig, LlamaPolarForCausalLM, LlamaPolarGroupAttention,
+                                                 PolarCache, generate)
+from polarquant_amd.modeling_qwen_polar import Qwen2PolarForCausalLM, Qwen2PolarGroupAttention
+
+pytestmark = pytest.mark.gpu
+
+
+def _tiny(n_heads=4, n_kv=2, layers=2, **kw):
+    return PolarConfig(hidden_size=n_heads * 128, num_attention_heads=n_heads, num_key_value_heads=n_kv,
+                       num_hidden_layers=layers, intermediate_size=512, vocab_size=1000, rope_theta=1e4,
+                       eos_token_id=[999999], **kw)
+
+
+def _rope(cfg, start, n, dtype, dev):
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    ang = torch.arange(start, start + n, dtype=torch.float32)[:, None] * inv[None]
+    emb = torch.cat([ang, ang], -1)[None]
+    return emb.cos().to(dtype).to(dev), emb.sin().to(dtype).to(dev)
+
+
+@pytest.mark.parametrize("cls,n_heads,n_kv,rb,tb", [(LlamaPolarGroupAttention, 4, 2, 4, 4), (Qwen2PolarGroupAttention, 7, 1, 3, 3)])
+@pytest.mark.parametrize("L", [5, 200, 256])
+def test_attention_forward_matches_reference_restatement(gpu, cls, n_heads, n_kv, rb, tb, L):
+    """Prefill then decode across a residual flush.  The post-RoPE q/k/v of every call are captured
+    on the GPU and replayed through the oracle's forward: cache contents must be bit-identical
+    (codes, metadata, residual keys, values, kv_seq_len) and outputs within the fp16 tolerance."""
+    torch.manual_seed(0)
+    cfg = _tiny(n_heads, n_kv, rbits=rb, tbits=tb)
+    att = cls(cfg, 0).half().to(gpu)
+    assert (att.q_proj.bias is not None) == (cls is Qwen2PolarGroupAttention)
+    att.capture = []
+    B, steps = 2, 140
+    mask = torch.ones(B, L, dtype=torch.int64)
+    mask[1, :min(3, L - 1)] = 0                              # left padding on sequence 1
+    x = (torch.randn(B, L + steps, cfg.hidden_size) * 0.5).half().to(gpu)
+    with torch.no_grad():
+        out, cache = att(x[:, :L], attention_mask=mask.to(gpu), past_key_value=None, position_embeddings=_rope(cfg, 0, L, torch.float16, gpu))
+    assert isinstance(cache, tuple) and len(cache) == 8 and cache[-1] == L
+    q, k, v = [t.cpu() for t in att.capture[-1]]
+    ref_cache = po.prefill_cache(k, v, rb, tb)
+    _check_cache(cache, ref_cache)
+    o_proj = att.o_proj.weight.detach().float().cpu()
+    for i in range(steps):
+        mask = torch.cat([mask, torch.ones(B, 1, dtype=torch.int64)], -1)
+        with torch.no_grad():
+            out, cache = att(x[:, L + i:L + i + 1], attention_mask=mask.to(gpu), past_key_value=cache,
+                             position_embeddings=_rope(cfg, L + i, 1, torch.float16, gpu))
+        q, k, v = [t.cpu() for t in att.capture[-1]]
+        ref_attn, ref_cache = po.decode_step(q, k, v, ref_cache, mask, rb, tb)
+        ref_out = ref_attn.reshape(B, 1, -1).float() @ o_proj.T
+        assert out.shape == (B, 1, cfg.hidden_size)
+        err = (out.float().cpu() - ref_out).abs().max().item()
+        assert err < 2e-2 * max(1.0, ref_out.abs().max().item()), (i, err)
+        if i in (0, 1, steps // 2, steps - 1) or (L + i + 1) % 128 in (0, 1):
+            _check_cache(cache, ref_cache)
+
+
+def _check_cache(got, ref):
+    assert got[-1] == ref[-1]
+    for j, (g, r) in enumerate(zip(got[:-1], ref[:-1])):
+        assert (g is None) == (r is None), "tuple element %d" % j
+        if g is not None:
+            g = g.cpu()
+            assert g.shape == r.shape and g.dtype == r.dtype, "tuple element %d" % j
+            if g.dtype == torch.uint8:
+                assert torch.equal(g, r), "codes differ"
+            else:
+                assert bool((g.float() == r.float()).all()), "tuple element %d differs" % j
+
+
+def test_plain_reference_tuple_is_accepted(gpu):
+    """A cache tuple built elsewhere in the reference's format (plain tuple, no arena) can be passed in."""
+    torch.manual_seed(1)
+    cfg = _tiny()
+    att = LlamaPolarGroupAttention(cfg, 0).half().to(gpu)
+    att.capture = []
+    x = torch.randn(1, 301, cfg.hidden_size).half().to(gpu)
+    with torch.no_grad():
+        _, cache = att(x[:, :300], None, None, _rope(cfg, 0, 300, torch.float16, gpu))
+        plain = tuple(t.clone() if torch.is_tensor(t) else t for t in cache)
+        assert not isinstance(plain, PolarCache)
+        o1, c1 = att(x[:, 300:], None, cache, _rope(cfg, 300, 1, torch.float16, gpu))
+        o2, c2 = att(x[:, 300:], None, plain, _rope(cfg, 300, 1, torch.float16, gpu))
+    assert torch.equal(o1, o2) and c1[-1] == c2[-1] == 301
+
+
+@pytest.mark.parametrize("cls,cfg", [(LlamaPolarForCausalLM, _tiny()), (Qwen2PolarForCausalLM, _tiny(7, 1, rbits=3, tbits=3, attention_bias=True))])
+def test_generate_greedy_matches_cpu_replay(gpu, cls, cfg):
+    """Greedy generation across a flush; every decode step's logits are replayed on the CPU with
+    the oracle attention (fp32 weights) and must agree."""
+    torch.manual_seed(2)
+    model = cls(cfg).half().to(gpu).eval()
+    B, L, new = 2, 250, 12
+    ids = torch.randint(0, cfg.vocab_size, (B, L))
+    gen = GenerationConfig(eos_token_id=[999999])
+    out = generate(model, ids.to(gpu), torch.ones(B, L, dtype=torch.int64, device=gpu), gen, max_new_tokens=new)
+    assert out.shape == (B, new) and out.dtype == torch.long
+    assert model.kv_cache_bytes_per_token() == cfg.num_hidden_layers * cfg.num_key_value_heads * (64 + 4 + 256)
+    # replay: same model, step by step, capturing q/k/v per layer and checking the layer outputs
+    for layer in model.model.layers:
+        layer.self_attn.capture = []
+    with torch.no_grad():
+        o = model(ids.to(gpu), None, None, num_logits_to_keep=1)
+        caches = o.past_key_values
+        assert caches[0][-1] == L and len(caches) == cfg.num_hidden_layers
+        ref_caches = []
+        for layer in model.model.layers:
+            q, k, v = [t.cpu() for t in layer.self_attn.capture[-1]]
+            ref_caches.append(po.prefill_cache(k, v, cfg.rbits, cfg.tbits))
+        tok = o.logits.argmax(-1)
+        assert torch.equal(tok.cpu(), out[:, :1].cpu())
+        for s in range(1, new):
+            o = model(tok, None, caches, num_logits_to_keep=1)
+            caches = o.past_key_values
+            for li, layer in enumerate(model.model.layers):
+                q, k, v = [t.cpu() for t in layer.self_attn.capture[-1]]
+                _, ref_caches[li] = po.decode_step(q, k, v, ref_caches[li], None, cfg.rbits, cfg.tbits)
+                _check_cache(caches[li], ref_caches[li])
+            tok = o.logits.argmax(-1)
+            assert torch.equal(tok.cpu(), out[:, s:s + 1].cpu())
+        assert caches[0][-1] == L + new - 1
