@@ -112,6 +112,15 @@ int pq_validate_quantize_groups(const void *k, const int64_t *k_strides, int dty
                                 const void *tscale, const void *tmn,
                                 int out_group_capacity, int out_group_offset);
 
+/* Device self-test of the quantizer's arithmetic (no reference counterpart).
+ * The kernel takes a cheap arctangent / square root first and the exact,
+ * eager-torch-identical routines only near a rounding boundary; this runs both on
+ * ALL 2^32 (y, x) operand pairs of the dtype (NaNs skipped) and adds to
+ * counters[0] the number of pairs whose rounded angle or radius differ (must stay
+ * 0) and to counters[1] the number of pairs that needed the exact routine.
+ * `counters`: device uint64[2], zeroed by the caller. Takes ~0.1 s. */
+int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
+
 /* ---------------------------------------------------------------------------
  * R+M+X+V — fused decode attention over the polar key cache.
  * Replaces the decode branch of LlamaPolarGroupAttention.forward between the

@@ -32,6 +32,7 @@ SIGNATURES = {
                            + [c_void_p] * 5 + [c_int, c_int, c_void_p]),
     "pq_validate_quantize_groups": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_uint]
                                     + [c_void_p] * 5 + [c_int, c_int]),
+    "pq_selftest_quantizer_math": (c_int, [c_int, c_void_p, c_void_p]),
     "pq_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_int64, c_void_p, c_int64, c_float]
                        + [c_int] * 7 + [c_void_p, c_size_t, c_void_p, c_void_p]),

@@ -111,6 +111,15 @@ int pq_quantize_groups(const void* k, const int64_t* k_strides, int dtype,
 
 extern "C" {
 
+int pq_selftest_quantizer_math(int dtype, uint64_t* counters, void* stream) {
+    if (!counters) return PQ_ERR_NULL_POINTER;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (!aligned(counters, 8)) return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_selftest(dtype, reinterpret_cast<unsigned long long*>(counters),
+                                        static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || max_groups <= 0) return 1;
     if (n_cus <= 0) n_cus = 256;

@@ -14,6 +14,8 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
                     unsigned flags, uint8_t* codes, void* rscale, void* rmn, void* tscale, void* tmn,
                     int cap, int off, hipStream_t st);
 
+int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;

@@ -21,6 +21,76 @@ namespace pq {
 template <typename T>
 __device__ __forceinline__ float rnd(float f) { return lo2f<T>(f2lo<T>(f)); }
 
+// ---- angle and radius of one pair, rounded to the key dtype -------------------
+// Eager torch gives round_dtype(atan2f_sleef(y, x)) and round_dtype(sqrt_rn(x*x + y*y)).
+// The exact routines cost ~100 instructions per pair, so a cheap estimate is tried
+// first: a 3.5-ulp arctangent (reciprocal, degree-8 polynomial in r^2, quadrant
+// fix-up; it stays within 4 ulp of the exact routine) and the hardware square
+// root (1 ulp).  Rounding the estimate to the key dtype gives the same word as
+// rounding the exact value unless the estimate lies within its error bound of a
+// rounding boundary of the dtype (a midpoint between two neighbouring dtype
+// values, i.e. low fp32 mantissa bits == 100..0).  Only those lanes, plus the
+// special operands (zeros, infinities, NaNs, results below the dtype's normal
+// range), take the exact path.  That the two paths agree on EVERY pair of half /
+// bfloat16 operands is checked exhaustively on the device by pq_selftest_quantizer_math.
+template <typename T> struct DT;
+template <> struct DT<F16> { static constexpr uint32_t kLowMask = 0x1fffu, kMid = 0x1000u; static constexpr float kMinNormal = 6.103515625e-05f; };
+template <> struct DT<BF16> { static constexpr uint32_t kLowMask = 0xffffu, kMid = 0x8000u; static constexpr float kMinNormal = 1.17549435e-38f; };
+
+constexpr uint32_t kAtanGuardUlps = 5;   // the fast arctangent stays within 4 ulp of the exact routine (exhaustive self-test)
+constexpr uint32_t kSqrtGuardUlps = 2;   // v_sqrt_f32 is within 1 ulp
+
+template <typename T>
+__device__ __forceinline__ bool near_rounding_boundary(float a, uint32_t guard) {
+    // |low mantissa bits - midpoint pattern| <= guard, computed without a branch
+    const uint32_t low = (__float_as_uint(a) + (guard - DT<T>::kMid)) & DT<T>::kLowMask;
+    return low <= 2u * guard;
+}
+
+__device__ __forceinline__ float atan2_fast(float y, float x) {
+    const float ax = fabsf(x), ay = fabsf(y);
+    const float mx = fmaxf(ax, ay), mn = fminf(ax, ay);
+    const float r = mn * __builtin_amdgcn_rcpf(mx);
+    const float s = r * r;
+    float u = 0.00282363896258175373077393f;
+    u = __builtin_fmaf(u, s, -0.0159569028764963150024414f);
+    u = __builtin_fmaf(u, s, 0.0425049886107444763183594f);
+    u = __builtin_fmaf(u, s, -0.0748900920152664184570312f);
+    u = __builtin_fmaf(u, s, 0.106347933411598205566406f);
+    u = __builtin_fmaf(u, s, -0.142027363181114196777344f);
+    u = __builtin_fmaf(u, s, 0.199926957488059997558594f);
+    u = __builtin_fmaf(u, s, -0.333331018686294555664062f);
+    float a = __builtin_fmaf(u * s, r, r);
+    a = ay > ax ? 1.57079637050628662109f - a : a;
+    a = x < 0.0f ? 3.14159274101257324219f - a : a;
+    return __builtin_copysignf(a, y);
+}
+
+// -> (angle in [-pi, pi], radius), both already rounded to the key dtype
+template <typename T>
+__device__ __forceinline__ void angle_radius(float x, float y, float* phi, float* rad) {
+    const float ss = __builtin_fmaf(x, x, y * y);          // x*x, y*y are exact for half/bf16 operands
+    float a = atan2_fast(y, x);
+    float r = __builtin_amdgcn_sqrtf(ss);
+    // zeros, infinities, NaNs, and magnitudes (bfloat16 only) at which the reciprocal or the
+    // hardware square root leave their accurate range
+    const bool special = !(ss > 0x1p-80f && ss < 0x1p80f) || fminf(fabsf(x), fabsf(y)) == 0.0f;
+    const bool risky = special || fabsf(a) < DT<T>::kMinNormal || r < DT<T>::kMinNormal ||
+                       near_rounding_boundary<T>(a, kAtanGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
+    if (__builtin_expect(risky, 0)) {
+        a = math::atan2f_sleef_u10(y, x);
+        r = __fsqrt_rn(ss);
+    }
+    *phi = rnd<T>(a);
+    *rad = rnd<T>(r);
+}
+
+template <typename T>
+__device__ __forceinline__ void angle_radius_exact(float x, float y, float* phi, float* rad) {
+    *phi = rnd<T>(math::atan2f_sleef_u10(y, x));
+    *rad = rnd<T>(__fsqrt_rn(__builtin_fmaf(x, x, y * y)));
+}
+
 template <typename T>
 __device__ __forceinline__ uint32_t code_of(float v, float mn, float scale, int top) {
     const float d = rnd<T>(v - mn);
@@ -67,9 +137,9 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float x = lo2f<T>(xs[i]), y = lo2f<T>(ys[i]);
-            float phi = rnd<T>(math::atan2f_sleef_u10(y, x));          // :143
+            float phi, r;
+            angle_radius<T>(x, y, &phi, &r);                           // :143, :150
             if (phi < 0.0f) phi = rnd<T>(phi + two_pi);                // :144
-            const float r = rnd<T>(__fsqrt_rn(__builtin_fmaf(x, x, y * y)));   // :150 (x*x, y*y are exact)
             pmx[i] = fmaxf(pmx[i], phi); pmn[i] = fminf(pmn[i], phi);
             rmx[i] = fmaxf(rmx[i], r);   rmn_[i] = fminf(rmn_[i], r);
             pr[it][i] = static_cast<uint32_t>(f2lo<T>(phi)) | (static_cast<uint32_t>(f2lo<T>(r)) << 16);
@@ -127,6 +197,33 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         }
         *reinterpret_cast<uint32_t*>(cb + tok * kPairs + 4 * pq4) = w;
     }
+}
+
+// Exhaustive check of angle_radius against angle_radius_exact: block == bit pattern of y,
+// thread t covers x patterns t, t+256, ...; NaN operands are skipped.
+template <typename T>
+__global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* mismatches, unsigned long long* slow_lanes) {
+    const uint16_t yb = static_cast<uint16_t>(blockIdx.x);
+    const float y = lo2f<T>(yb);
+    unsigned int bad = 0, slow = 0;
+    for (uint32_t xb = threadIdx.x; xb < 65536u; xb += 256u) {
+        const float x = lo2f<T>(static_cast<uint16_t>(xb));
+        if (x != x || y != y) continue;
+        float p0, r0, p1, r1;
+        angle_radius<T>(x, y, &p0, &r0);
+        angle_radius_exact<T>(x, y, &p1, &r1);
+        bad += (f2lo<T>(p0) != f2lo<T>(p1)) || (f2lo<T>(r0) != f2lo<T>(r1));
+        const float a = atan2_fast(y, x), r = __builtin_amdgcn_sqrtf(__builtin_fmaf(x, x, y * y));
+        slow += near_rounding_boundary<T>(a, kAtanGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
+    }
+    if (bad) atomicAdd(mismatches, static_cast<unsigned long long>(bad));
+    if (slow) atomicAdd(slow_lanes, static_cast<unsigned long long>(slow));
+}
+
+int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st) {
+    if (dtype == 0) hipLaunchKernelGGL(selftest_kernel<F16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+    else hipLaunchKernelGGL(selftest_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+    return static_cast<int>(hipGetLastError());
 }
 
 int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int Nk, int Nb, int rbits, int tbits,

@@ -114,3 +114,16 @@ def test_quantize_wrap_fp32_flag(gpu):
     # libm atan2f (C oracle) vs the SLEEF restatement may differ in the last ulp: allow a handful, report them
     print("wrap_fp32 flips vs C oracle", flips, flush=True)
     assert flips["codes"] <= 4 and flips["rscale"] == 0 and flips["rmn"] == 0
+
+
+@pytest.mark.parametrize("dtype_code,name", [(0, "float16"), (1, "bfloat16")])
+def test_quantizer_math_selftest_exhaustive(gpu, dtype_code, name):
+    """The cheap-estimate-with-guard path against the exact path on all 2^32 operand pairs of the dtype."""
+    from polarquant_amd import _ffi
+    counters = torch.zeros(2, dtype=torch.int64, device=gpu)
+    rc = _ffi.lib().pq_selftest_quantizer_math(dtype_code, counters.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    bad, slow = counters.tolist()
+    print("%s: %d mismatching pairs, %.3f%% of pairs take the exact path" % (name, bad, 100.0 * slow / 2 ** 32), flush=True)
+    assert bad == 0
