@@ -1,0 +1,149 @@
+"""Parity at BASELINE.json's full sizes (configs[1], [2], [3]).
+
+The CPU oracle cannot chew through a gigabyte of cache in seconds, so each
+full-size case combines (a) the oracle on whole (sequence, KV head) planes picked
+from the full problem, and (b) size-independent properties of the full result:
+invariance to the context split, to the batch order, chunked == one-shot
+quantization, per-sequence == batched for ragged batches.
+"""
+import math
+
+import pytest
+import torch
+
+import bench
+from oracle import polar_oracle as po
+from polarquant_amd.attention import polar_decode_attention
+from polarquant_amd.quantize import quantize_and_pack_nbit
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def _ok(got, ref):
+    err = (got.double() - ref.double()).abs()
+    return bool((err <= ATOL + RTOL * ref.double().abs()).all()), float(err.max())
+
+
+def _attn(w, **kw):
+    sh = w["shape"]
+    args = dict(rbits=sh.rbits, tbits=sh.tbits, n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"])
+    args.update(kw)
+    return polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], **args)
+
+
+def _oracle_plane(w, b, kvh, n_groups, n_resid):
+    """fp64 oracle attention for the `rep` query heads of one (sequence, KV head) plane."""
+    sh = w["shape"]
+    rep = sh.n_heads // sh.n_kv_heads
+    q = w["q"][b:b + 1, kvh * rep:(kvh + 1) * rep].cpu()
+    quant = (None,) * 5
+    if n_groups:
+        quant = [w["codes"][b:b + 1, kvh:kvh + 1, :n_groups].cpu()] + [m[b:b + 1, kvh:kvh + 1, :n_groups].cpu() for m in w["meta"]]
+    kres = w["kres"][b:b + 1, kvh:kvh + 1, :n_resid].cpu() if n_resid else None
+    v = w["v"][b:b + 1, kvh:kvh + 1, :n_groups * 128 + n_resid].cpu()
+    return po.decode_attention_exact(q, kres, *quant, v, None, sh.rbits, sh.tbits)
+
+
+def test_cfg1_full_size(gpu):
+    """configs[1]: batch 16, 32 q / 8 KV heads, context 32768, 4/4 bits."""
+    print("building configs[1]", flush=True)
+    w = bench.build_workload(1, gpu)
+    sh = w["shape"]
+    rep = sh.n_heads // sh.n_kv_heads
+    out = _attn(w).clone()
+    torch.cuda.synchronize()
+    assert out.shape == (16, 32, 1, 128) and torch.isfinite(out.float()).all()
+    # (a) oracle on three whole planes
+    for b, kvh in [(0, 0), (7, 3), (15, 7)]:
+        ref = _oracle_plane(w, b, kvh, w["n_groups"], w["n_resid"])
+        ok, err = _ok(out[b:b + 1, kvh * rep:(kvh + 1) * rep].cpu(), ref)
+        print("plane", b, kvh, "max abs err %.2e" % err, flush=True)
+        assert ok
+    # (b) the context split must not matter
+    for ns in (5, 16, 64):
+        other = _attn(w, n_splits=ns)
+        ok, err = _ok(other.cpu(), out.cpu())
+        assert ok, (ns, err)
+    # (c) reversing the batch reverses the output, bit for bit
+    flip = lambda t: t.flip(0).contiguous()
+    w2 = dict(w, q=flip(w["q"]), codes=flip(w["codes"]), meta=[flip(m) for m in w["meta"]], kres=flip(w["kres"]), v=flip(w["v"]))
+    assert torch.equal(_attn(w2).flip(0), out)
+    # (d) masking all but the last 1000 tokens == attention over that suffix alone (oracle on one plane)
+    L = w["n_groups"] * 128 + w["n_resid"]
+    mask = torch.zeros(16, L, dtype=torch.uint8, device=gpu)
+    mask[:, -1000:] = 1
+    om = _attn(w, attention_mask=mask)
+    b, kvh = 3, 5
+    qq = w["q"][b:b + 1, kvh * rep:(kvh + 1) * rep].cpu()
+    quant = [w["codes"][b:b + 1, kvh:kvh + 1].cpu()] + [m[b:b + 1, kvh:kvh + 1].cpu() for m in w["meta"]]
+    ref = po.decode_attention_exact(qq, w["kres"][b:b + 1, kvh:kvh + 1, :1].cpu(), *quant, w["v"][b:b + 1, kvh:kvh + 1].cpu(),
+                                    mask[b:b + 1].cpu(), sh.rbits, sh.tbits)
+    ok, err = _ok(om[b:b + 1, kvh * rep:(kvh + 1) * rep].cpu(), ref)
+    assert ok, err
+
+
+def test_cfg2_full_size_ragged(gpu):
+    """configs[2]: batch 64, 28 q / 4 KV heads (GQA 7), 3/3 bits, per-sequence lengths in [512, 8192]."""
+    print("building configs[2]", flush=True)
+    w = bench.build_workload(2, gpu)
+    sh = w["shape"]
+    lens = w["lengths"]
+    assert int(lens.min()) >= 512 and int(lens.max()) <= 8192
+    out = _attn(w).clone()
+    torch.cuda.synchronize()
+    assert out.shape == (64, 28, 1, 128) and torch.isfinite(out.float()).all()
+    # (a) oracle on whole planes of the shortest, the longest and two other sequences
+    order = torch.argsort(lens)
+    for b in [int(order[0]), int(order[-1]), int(order[20]), int(order[41])]:
+        ng, nr = int(lens[b]) // 128, int(lens[b]) % 128
+        for kvh in (0, 3):
+            ref = _oracle_plane(w, b, kvh, ng, nr)
+            ok, err = _ok(out[b:b + 1, kvh * 7:(kvh + 1) * 7].cpu(), ref)
+            print("seq", b, "len", int(lens[b]), "kvh", kvh, "max abs err %.2e" % err, flush=True)
+            assert ok
+    # (b) every sequence alone (batch of one, uniform counts) == its row in the ragged batch
+    for b in [int(order[1]), int(order[33]), int(order[-2])]:
+        ng, nr = int(lens[b]) // 128, int(lens[b]) % 128
+        alone = polar_decode_attention(w["q"][b:b + 1], w["codes"][b:b + 1], *[m[b:b + 1] for m in w["meta"]],
+                                       w["kres"][b:b + 1], w["v"][b:b + 1], ng, nr, rbits=3, tbits=3)
+        ok, err = _ok(alone.cpu(), out[b:b + 1].cpu())
+        assert ok, err
+    # (c) split invariance
+    ok, err = _ok(_attn(w, n_splits=7).cpu(), out.cpu())
+    assert ok, err
+
+
+def test_cfg3_full_size_append_and_decode(gpu):
+    """configs[3]: batch 1, context 131072: quantize all prompt keys, then one decode step."""
+    print("building configs[3]", flush=True)
+    w = bench.build_workload(3, gpu, keep_keys=True)
+    sh = w["shape"]
+    k = w["keys"]                                            # [1,8,131072,128] fp16 on the GPU
+    assert k.shape == (1, 8, 131072, 128)
+    codes, meta = w["codes"], w["meta"]
+    assert int(codes.max()) <= 255
+    # (a) append: oracle, bit for bit, on group ranges spread over heads and positions
+    for kvh, g0, n in [(0, 0, 8), (3, 500, 8), (7, 1016, 8), (5, 257, 3)]:
+        ref = po.quantize_and_pack_nbit(k[:, kvh:kvh + 1, g0 * 128:(g0 + n) * 128].cpu(), 4, 4)
+        assert torch.equal(codes[:, kvh:kvh + 1, g0:g0 + n].cpu(), ref[0])
+        for m, r in zip(meta, ref[1:]):
+            assert bool((m[:, kvh:kvh + 1, g0:g0 + n].cpu().float() == r.float()).all())
+    # (b) chunked append (one group at a time into a cache slot, as decode does) == one-shot, via checksums
+    kvh = 2
+    one = quantize_and_pack_nbit(k[:, kvh:kvh + 1], 4, 4)
+    slot = (torch.zeros_like(one[0]), *[torch.zeros_like(m) for m in one[1:]])
+    for g in range(0, 1024, 97):
+        quantize_and_pack_nbit(k[:, kvh:kvh + 1, g * 128:(g + 1) * 128], 4, 4, out=slot, group_offset=g)
+        assert torch.equal(slot[0][:, :, g], one[0][:, :, g])
+    assert int(one[0].long().sum()) == int(codes[:, kvh].long().sum())
+    # (c) decode over the whole cache: oracle on two planes, and split invariance
+    out = _attn(w).clone()
+    for kvh in (1, 6):
+        ref = _oracle_plane(w, 0, kvh, w["n_groups"], w["n_resid"])
+        ok, err = _ok(out[:, kvh * 4:(kvh + 1) * 4].cpu(), ref)
+        print("cfg3 plane", kvh, "max abs err %.2e" % err, flush=True)
+        assert ok
+    for ns in (64, 333):
+        ok, err = _ok(_attn(w, n_splits=ns).cpu(), out.cpu())
+        assert ok, (ns, err)
