@@ -66,20 +66,32 @@ __device__ __forceinline__ float atan2_fast(float y, float x) {
     return __builtin_copysignf(a, y);
 }
 
-// -> (angle in [-pi, pi], radius), both already rounded to the key dtype
+// Cheap estimates of the angle (in [-pi, pi]) and radius, NOT yet rounded; returns true when
+// the exact routines must be used instead (see above).
 template <typename T>
-__device__ __forceinline__ void angle_radius(float x, float y, float* phi, float* rad) {
+__device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out, float* r_out) {
     const float ss = __builtin_fmaf(x, x, y * y);          // x*x, y*y are exact for half/bf16 operands
-    float a = atan2_fast(y, x);
-    float r = __builtin_amdgcn_sqrtf(ss);
+    const float a = atan2_fast(y, x);
+    const float r = __builtin_amdgcn_sqrtf(ss);
     // zeros, infinities, NaNs, and magnitudes (bfloat16 only) at which the reciprocal or the
     // hardware square root leave their accurate range
-    const bool special = !(ss > 0x1p-80f && ss < 0x1p80f) || fminf(fabsf(x), fabsf(y)) == 0.0f;
-    const bool risky = special || fabsf(a) < DT<T>::kMinNormal || r < DT<T>::kMinNormal ||
-                       near_rounding_boundary<T>(a, kAtanGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
-    if (__builtin_expect(risky, 0)) {
+    // (bitwise | on purpose: one straight-line predicate instead of a chain of exec-mask branches)
+    const int in_range = static_cast<int>(ss > 0x1p-80f) & static_cast<int>(ss < 0x1p80f);
+    const int special = (in_range ^ 1) | static_cast<int>(fminf(fabsf(x), fabsf(y)) == 0.0f);
+    *a_out = a;
+    *r_out = r;
+    return (special | static_cast<int>(fminf(fabsf(a), r) < DT<T>::kMinNormal) |
+            static_cast<int>(near_rounding_boundary<T>(a, kAtanGuardUlps)) |
+            static_cast<int>(near_rounding_boundary<T>(r, kSqrtGuardUlps))) != 0;
+}
+
+// -> (angle in [-pi, pi], radius), both rounded to the key dtype
+template <typename T>
+__device__ __forceinline__ void angle_radius(float x, float y, float* phi, float* rad) {
+    float a, r;
+    if (__builtin_expect(angle_radius_fast<T>(x, y, &a, &r), 0)) {
         a = math::atan2f_sleef_u10(y, x);
-        r = __fsqrt_rn(ss);
+        r = __fsqrt_rn(__builtin_fmaf(x, x, y * y));
     }
     *phi = rnd<T>(a);
     *rad = rnd<T>(r);
@@ -104,14 +116,49 @@ __device__ __forceinline__ uint32_t code_of(float v, float mn, float scale, int 
 
 constexpr int kQThreads = 256;
 constexpr int kTokPerThread = kGroup / 16;   // 8
+constexpr int kEntries = kTokPerThread * 4;  // (token, pair) entries per thread
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef unsigned short ushort2v __attribute__((ext_vector_type(2)));
+
+// Packed min / max of two (angle word | radius word << 16) registers.  Both values are
+// non-negative (the angle after the 2*pi wrap, the radius always) and their sign bits are
+// cleared, so bfloat16 words order like unsigned integers; half words use v_pk_max/min_f16.
+template <typename T> __device__ __forceinline__ uint32_t pk_max(uint32_t a, uint32_t b);
+template <typename T> __device__ __forceinline__ uint32_t pk_min(uint32_t a, uint32_t b);
+template <> __device__ __forceinline__ uint32_t pk_max<F16>(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b)));
+}
+template <> __device__ __forceinline__ uint32_t pk_min<F16>(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(half2v, a), __builtin_bit_cast(half2v, b)));
+}
+template <> __device__ __forceinline__ uint32_t pk_max<BF16>(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(ushort2v, a), __builtin_bit_cast(ushort2v, b)));
+}
+template <> __device__ __forceinline__ uint32_t pk_min<BF16>(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(ushort2v, a), __builtin_bit_cast(ushort2v, b)));
+}
+template <typename T> struct PkInit;   // identity elements of pk_max / pk_min
+template <> struct PkInit<F16> { static constexpr uint32_t kMax = 0x00000000u, kMin = 0x7c007c00u; };   // 0 / +inf
+template <> struct PkInit<BF16> { static constexpr uint32_t kMax = 0x00000000u, kMin = 0xffffffffu; };
+
+// (angle word | radius word << 16) of one pair: wrap applied, sign bits cleared
+template <typename T>
+__device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, float two_pi) {
+    float phi = rnd<T>(a);
+    if (phi < 0.0f) phi = rnd<T>(phi + two_pi);                    // :144
+    return (static_cast<uint32_t>(f2lo<T>(phi)) | (static_cast<uint32_t>(f2lo<T>(r)) << 16)) & 0x7fff7fffu;
+}
 
 template <typename T>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t st, int Nk, int rbits, int tbits, float two_pi,
     uint8_t* __restrict__ codes, uint16_t* __restrict__ rscale, uint16_t* __restrict__ rmn,
     uint16_t* __restrict__ tscale, uint16_t* __restrict__ tmn, int cap, int off) {
-    __shared__ float red[4][16][kPairs];      // stat, token lane, pair
-    __shared__ float fin[4][kPairs];
+    // angle/radius words of the tile, entry-major so that a wavefront's accesses are contiguous
+    __shared__ uint32_t pr[kEntries][kQThreads];
+    __shared__ uint32_t red[2][4][kPairs];      // max / min, wavefront, pair
+    __shared__ uint32_t fin[2][kPairs];
 
     const int tid = threadIdx.x;
     const int pq4 = tid & 15, tl = tid >> 4;
@@ -119,15 +166,11 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     const int b = bh / Nk, h = bh - b * Nk;
     const uint16_t* kb = k + b * sb + h * sh + static_cast<int64_t>(grp) * kGroup * st;
 
-    uint32_t pr[kTokPerThread][4];   // (phi word) | (radius word << 16)
-    float pmx[4], pmn[4], rmx[4], rmn_[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) { pmx[i] = -INFINITY; pmn[i] = INFINITY; rmx[i] = -INFINITY; rmn_[i] = INFINITY; }
-
+    // ---- pass 1: cheap estimates for every entry; remember which entries need the exact routines
+    uint32_t risky_mask = 0;
 #pragma unroll
     for (int it = 0; it < kTokPerThread; it++) {
-        const int tok = it * 16 + tl;
-        const uint16_t* row = kb + tok * st;
+        const uint16_t* row = kb + (it * 16 + tl) * st;
         const uint2 xw = *reinterpret_cast<const uint2*>(row + 4 * pq4);
         const uint2 yw = *reinterpret_cast<const uint2*>(row + kPairs + 4 * pq4);
         const uint16_t xs[4] = {static_cast<uint16_t>(xw.x), static_cast<uint16_t>(xw.x >> 16),
@@ -136,26 +179,52 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
                                 static_cast<uint16_t>(yw.y), static_cast<uint16_t>(yw.y >> 16)};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float x = lo2f<T>(xs[i]), y = lo2f<T>(ys[i]);
-            float phi, r;
-            angle_radius<T>(x, y, &phi, &r);                           // :143, :150
-            if (phi < 0.0f) phi = rnd<T>(phi + two_pi);                // :144
-            pmx[i] = fmaxf(pmx[i], phi); pmn[i] = fminf(pmn[i], phi);
-            rmx[i] = fmaxf(rmx[i], r);   rmn_[i] = fminf(rmn_[i], r);
-            pr[it][i] = static_cast<uint32_t>(f2lo<T>(phi)) | (static_cast<uint32_t>(f2lo<T>(r)) << 16);
+            float a, r;
+            const bool risky = angle_radius_fast<T>(lo2f<T>(xs[i]), lo2f<T>(ys[i]), &a, &r);   // :143, :150
+            risky_mask |= static_cast<uint32_t>(risky) << (it * 4 + i);
+            pr[it * 4 + i][tid] = pack_angle_radius<T>(a, rnd<T>(r), two_pi);
         }
     }
+    // ---- fix-up: each lane redoes ITS risky entries with the exact routines (a lane has ~0.1 of
+    // them, so the wavefront makes one or two trips instead of branching at all 32 entries)
+    while (risky_mask) {
+        const int e = __builtin_ctz(risky_mask);
+        risky_mask &= risky_mask - 1;
+        const uint16_t* row = kb + ((e >> 2) * 16 + tl) * st;
+        const float x = lo2f<T>(row[4 * pq4 + (e & 3)]), y = lo2f<T>(row[kPairs + 4 * pq4 + (e & 3)]);
+        float a, r;
+        angle_radius_exact<T>(x, y, &a, &r);
+        pr[e][tid] = pack_angle_radius<T>(a, r, two_pi);
+    }
+    // ---- per-pair max / min of angle and radius over the 128 tokens (packed: both at once)
+    uint32_t vmax[4], vmin[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) { vmax[i] = PkInit<T>::kMax; vmin[i] = PkInit<T>::kMin; }
+#pragma unroll
+    for (int e = 0; e < kEntries; e++) {
+        const uint32_t w = pr[e][tid];
+        vmax[e & 3] = pk_max<T>(vmax[e & 3], w);
+        vmin[e & 3] = pk_min<T>(vmin[e & 3], w);
+    }
+    // the 16 token lanes of a pair: 4 inside the wavefront (lane bits 4,5), 4 wavefronts
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        red[0][tl][4 * pq4 + i] = pmx[i]; red[1][tl][4 * pq4 + i] = pmn[i];
-        red[2][tl][4 * pq4 + i] = rmx[i]; red[3][tl][4 * pq4 + i] = rmn_[i];
+#pragma unroll
+        for (int o = 16; o <= 32; o <<= 1) {
+            vmax[i] = pk_max<T>(vmax[i], static_cast<uint32_t>(__shfl_xor(static_cast<int>(vmax[i]), o)));
+            vmin[i] = pk_min<T>(vmin[i], static_cast<uint32_t>(__shfl_xor(static_cast<int>(vmin[i]), o)));
+        }
+    }
+    if ((tid & 48) == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) { red[0][tid >> 6][4 * pq4 + i] = vmax[i]; red[1][tid >> 6][4 * pq4 + i] = vmin[i]; }
     }
     __syncthreads();
-    {
+    if (tid < 2 * kPairs) {
         const int s = tid >> 6, p = tid & 63;
-        float v = red[s][0][p];
+        uint32_t v = red[s][0][p];
 #pragma unroll
-        for (int j = 1; j < 16; j++) v = (s & 1) ? fminf(v, red[s][j][p]) : fmaxf(v, red[s][j][p]);
+        for (int j = 1; j < 4; j++) v = s ? pk_min<T>(v, red[s][j][p]) : pk_max<T>(v, red[s][j][p]);
         fin[s][p] = v;
     }
     __syncthreads();
@@ -164,10 +233,11 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     float ts[4], tm[4], rs[4], rm[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int p = 4 * pq4 + i;
-        tm[i] = fin[1][p]; rm[i] = fin[3][p];
-        ts[i] = rnd<T>(rnd<T>(fin[0][p] - tm[i]) / inv_t);              // :147
-        rs[i] = rnd<T>(rnd<T>(fin[2][p] - rm[i]) / inv_r);              // :152
+        const uint32_t wmax = fin[0][4 * pq4 + i], wmin = fin[1][4 * pq4 + i];
+        tm[i] = lo2f<T>(static_cast<uint16_t>(wmin & 0xffffu));
+        rm[i] = lo2f<T>(static_cast<uint16_t>(wmin >> 16));
+        ts[i] = rnd<T>(rnd<T>(lo2f<T>(static_cast<uint16_t>(wmax & 0xffffu)) - tm[i]) / inv_t);   // :147
+        rs[i] = rnd<T>(rnd<T>(lo2f<T>(static_cast<uint16_t>(wmax >> 16)) - rm[i]) / inv_r);       // :152
     }
     const size_t plane = static_cast<size_t>(bh) * cap + off + grp;
     if (tl == 0) {
@@ -181,21 +251,22 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         *reinterpret_cast<uint2*>(rscale + mi) = pack4(rs);
         *reinterpret_cast<uint2*>(rmn + mi) = pack4(rm);
     }
+    // ---- pass 2: codes
     const int ttop = (1 << tbits) - 1, rtop = (1 << rbits) - 1;
     uint8_t* cb = codes + plane * (kGroup * kPairs);
 #pragma unroll
     for (int it = 0; it < kTokPerThread; it++) {
-        const int tok = it * 16 + tl;
         uint32_t w = 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float phi = lo2f<T>(static_cast<uint16_t>(pr[it][i] & 0xffffu));
-            const float r = lo2f<T>(static_cast<uint16_t>(pr[it][i] >> 16));
+            const uint32_t v = pr[it * 4 + i][tid];
+            const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
+            const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
             const uint32_t th = code_of<T>(phi, tm[i], ts[i], ttop);    // :148
             const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop);      // :153
             w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
         }
-        *reinterpret_cast<uint32_t*>(cb + tok * kPairs + 4 * pq4) = w;
+        *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPairs + 4 * pq4) = w;
     }
 }
 
