@@ -1,0 +1,88 @@
+"""End-to-end greedy decode with the polar-key attention (BASELINE configs[4]):
+random-init Llama-3-8B architecture (32 layers, hidden 4096, 32 q / 8 KV heads, FFN 14336,
+vocab 128256), bf16 weights ~N(0, 0.02), batch 8, prompt 16384 random ids, 256 new tokens.
+Reports prefill seconds, decode tokens/s and KV-cache bytes per token.  Mirrors the
+reference's throughput script (benchmark/benchmark_throughput.py:15-113): one timed prefill,
+then the timed greedy loop with EOS made unreachable.
+
+    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import time
+
+import torch
+
+from .modeling_common import PolarConfig
+from .modeling_llama_polar import LlamaPolarForCausalLM
+
+
+def build_model(cfg: PolarConfig, device, dtype=torch.bfloat16):
+    torch.manual_seed(0)
+    with torch.device(device):
+        prev = torch.get_default_dtype()
+        torch.set_default_dtype(dtype)
+        try:
+            model = LlamaPolarForCausalLM(cfg)
+        finally:
+            torch.set_default_dtype(prev)
+    g = torch.Generator(device=device).manual_seed(1234)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() >= 2:
+                p.normal_(0.0, 0.02, generator=g)
+    return model.eval()
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=16384)
+    ap.add_argument("--new", type=int, default=256)
+    ap.add_argument("--layers", type=int, default=32)
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    cfg = PolarConfig.llama3_8b(num_hidden_layers=args.layers, cache_capacity=args.prompt + args.new + 128,
+                                eos_token_id=[128256 + 10])
+    model = build_model(cfg, dev)
+    g = torch.Generator(device=dev).manual_seed(1004)
+    ids = torch.randint(0, cfg.vocab_size, (args.batch, args.prompt), generator=g, device=dev)
+    mask = torch.ones_like(ids)
+    with torch.no_grad():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = model(input_ids=ids, attention_mask=mask, past_key_values=None, num_logits_to_keep=1)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        cache = out.past_key_values
+        tok = out.logits.argmax(-1)
+        n_out = 1
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.new - 1):
+            mask = torch.cat([mask, torch.ones_like(tok)], dim=-1)
+            out = model(input_ids=tok, attention_mask=mask, past_key_values=cache, num_logits_to_keep=1)
+            cache = out.past_key_values
+            tok = out.logits.argmax(-1)
+            n_out += 1
+        torch.cuda.synchronize()
+        t_decode = time.perf_counter() - t0
+    steps = args.new - 1
+    kv = model.kv_cache_bytes_per_token()
+    fp16_kv = cfg.num_hidden_layers * cfg.num_key_value_heads * 2 * 128 * 2
+    print(json.dumps({
+        "workload": "configs[4]: greedy decode, random-init Llama-3-8B architecture, bf16, batch %d, prompt %d, %d new tokens"
+                    % (args.batch, args.prompt, args.new),
+        "layers": args.layers, "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
+        "decode_ms_per_step": round(1e3 * t_decode / steps, 3),
+        "decode_tokens_per_s": round(args.batch * steps / t_decode, 1),
+        "kv_cache_bytes_per_token": kv, "fp16_kv_cache_bytes_per_token": fp16_kv,
+        "kv_seq_len": cache[0][-1], "quantized_groups": cache[0][1].shape[2],
+        "peak_memory_GiB": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+    }))
+
+
+if __name__ == "__main__":
+    main()
