@@ -224,8 +224,10 @@ __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes
         static_for<BW>([&](auto CC) {
             constexpr int cc = decltype(CC)::value, c = bi * BW + cc;
             const uint32_t r4 = r4s[buf][cc];
+            // consume the batch's reads youngest first: the first use then waits for the whole
+            // batch at once (LDS returns in order) and the other three need no wait instruction
             static_for<4>([&](auto II) {
-                constexpr int i = decltype(II)::value;
+                constexpr int i = 3 - decltype(II)::value;
                 const float t = static_cast<float>((r4 >> (8 * i)) & 0xFFu) + cds[4 * c + i];
                 static_for<REPP>([&](auto JJ) {
                     constexpr int j = decltype(JJ)::value;
