@@ -128,3 +128,45 @@ def test_generate_greedy_matches_cpu_replay(gpu, cls, cfg):
             tok = o.logits.argmax(-1)
             assert torch.equal(tok.cpu(), out[:, s:s + 1].cpu())
         assert caches[0][-1] == L + new - 1
+
+
+def test_cache_arena_grows_past_its_initial_capacity(gpu):
+    """cache_capacity is only a hint: decoding past it reallocates (doubling) and keeps every cached token."""
+    torch.manual_seed(3)
+    cfg = _tiny(cache_capacity=128)
+    att = LlamaPolarGroupAttention(cfg, 0).half().to(gpu)
+    att.capture = []
+    L, steps = 100, 400                      # ends at 500 tokens: 3 groups + 116 residual, capacity grown twice
+    x = (torch.randn(1, L + steps, cfg.hidden_size) * 0.5).half().to(gpu)
+    with torch.no_grad():
+        _, cache = att(x[:, :L], None, None, _rope(cfg, 0, L, torch.float16, gpu))
+        q, k, v = [t.cpu() for t in att.capture[-1]]
+        ref_cache = po.prefill_cache(k, v)
+        cap0 = cache.arena.vcap
+        for i in range(steps):
+            out, cache = att(x[:, L + i:L + i + 1], None, cache, _rope(cfg, L + i, 1, torch.float16, gpu))
+            q, k, v = [t.cpu() for t in att.capture[-1]]
+            _, ref_cache = po.decode_step(q, k, v, ref_cache)
+    assert cache.arena.vcap > cap0 and cache[-1] == L + steps
+    _check_cache(cache, ref_cache)
+
+
+def test_decode_with_bf16_model(gpu):
+    torch.manual_seed(4)
+    cfg = _tiny()
+    att = LlamaPolarGroupAttention(cfg, 0).bfloat16().to(gpu)
+    att.capture = []
+    L = 130
+    x = (torch.randn(2, L + 3, cfg.hidden_size) * 0.5).bfloat16().to(gpu)
+    with torch.no_grad():
+        _, cache = att(x[:, :L], None, None, _rope(cfg, 0, L, torch.bfloat16, gpu))
+        q, k, v = [t.cpu() for t in att.capture[-1]]
+        ref_cache = po.prefill_cache(k, v)
+        _check_cache(cache, ref_cache)
+        for i in range(3):
+            out, cache = att(x[:, L + i:L + i + 1], None, cache, _rope(cfg, L + i, 1, torch.bfloat16, gpu))
+            q, k, v = [t.cpu() for t in att.capture[-1]]
+            ref_attn, ref_cache = po.decode_step(q, k, v, ref_cache)
+            ref_out = ref_attn.reshape(2, 1, -1).float() @ att.o_proj.weight.detach().float().cpu().T
+            assert (out.float().cpu() - ref_out).abs().max().item() < 5e-2 * max(1.0, ref_out.abs().max().item())
+    assert cache[1].dtype == torch.uint8 and cache[2].dtype == torch.bfloat16
