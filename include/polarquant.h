@@ -146,8 +146,14 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *   mask     optional device u8 [B, mask_stride]: 1 = attend, 0 = masked; column t
  *            is token t (reference attention_mask, :94-95); NULL = no mask
  *   sm_scale multiplier applied to every score (1/sqrt(128) in the reference)
- *   n_splits context splits per (batch, KV head) for the quantized part, >= 1;
+ *   n_splits context slices (blocks) per (batch, KV head) for the quantized part, >= 1;
  *            use pq_decode_attn_plan to choose
+ *   min_groups_per_split  0, or a lower bound on the groups one slice takes.  For ragged
+ *            batches pass ceil(total groups of all (batch, KV head) planes / (4 * CUs)) and
+ *            n_splits = ceil(group_capacity / that): every wavefront then gets about the same
+ *            number of groups whatever its sequence's length, and a short sequence uses only
+ *            its first few slices (the others return at once).  n_splits * max(this,
+ *            ceil(groups / n_splits)) always covers the sequence.
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
  * ------------------------------------------------------------------------- */
@@ -159,7 +165,7 @@ int pq_decode_attn(const void *q,
                    const void *v, int64_t v_capacity,
                    const uint8_t *mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                   int n_splits, void *workspace, size_t workspace_bytes,
+                   int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
                    void *out, void *stream);
 
 int pq_validate_decode_attn(const void *q,
@@ -170,7 +176,7 @@ int pq_validate_decode_attn(const void *q,
                             const void *v, int64_t v_capacity,
                             const uint8_t *mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, const void *workspace, size_t workspace_bytes,
+                            int n_splits, int min_groups_per_split, const void *workspace, size_t workspace_bytes,
                             const void *out);
 
 /* The two launches of pq_decode_attn as separate calls, same arguments and
@@ -188,7 +194,7 @@ int pq_decode_attn_partials(const void *q,
                             const void *v, int64_t v_capacity,
                             const uint8_t *mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, void *workspace, size_t workspace_bytes, void *stream);
+                            int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes, void *stream);
 
 int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
                          void *out, void *stream);

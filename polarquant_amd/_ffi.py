@@ -35,13 +35,13 @@ SIGNATURES = {
     "pq_selftest_quantizer_math": (c_int, [c_int, c_void_p, c_void_p]),
     "pq_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_int64, c_void_p, c_int64, c_float]
-                       + [c_int] * 7 + [c_void_p, c_size_t, c_void_p, c_void_p]),
+                       + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_void_p]),
     "pq_validate_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
-                                + [c_int] * 7 + [c_void_p, c_size_t, c_void_p]),
+                                + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "pq_decode_attn_partials": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
-                                + [c_int] * 7 + [c_void_p, c_size_t, c_void_p]),
+                                + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "pq_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),
     "pq_decode_attn_workspace_bytes": (c_size_t, [c_int] * 3),

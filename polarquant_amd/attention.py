@@ -49,8 +49,14 @@ def polar_decode_attention(
     rbits: int = 4, tbits: int = 4, sm_scale: Optional[float] = None,
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
+    total_groups: Optional[int] = None, min_groups_per_split: Optional[int] = None,
 ) -> torch.Tensor:
-    """-> attention output [B,N,1,128] in the query dtype."""
+    """-> attention output [B,N,1,128] in the query dtype.
+
+    Ragged batches (`n_groups_per_seq` given): `total_groups`, the sum of the per-sequence group
+    counts if the caller knows it on the host (no device sync is made here), lets the context be
+    cut into slices of equal size across sequences, so that short sequences do not leave
+    wavefronts idle; without it the average sequence is assumed to be half the capacity."""
     if not query_states.is_cuda:
         raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
     dev = query_states.device
@@ -83,6 +89,16 @@ def polar_decode_attention(
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(hd)
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
+    min_gps = 0
+    if n_groups_per_seq is not None and n_splits is None and max_groups > 0:
+        tot = total_groups if total_groups is not None else (B * max_groups + 1) // 2
+        # one wavefront per SIMD; every (sequence, KV head) rounds its slice count up, so leave one
+        # slot per plane for that and the whole batch still runs in a single round
+        slots = max(4 * _num_cus(dev) - B * Nk, B * Nk)
+        min_gps = max(1, -(-tot * Nk // slots))
+        n_splits = max(1, -(-max_groups // min_gps))
+    if min_groups_per_split is not None:
+        min_gps = min_groups_per_split
     if n_splits is None:
         n_splits = plan_splits(B, Nk, max_groups, dev)
     ws = workspace_for(B, N, n_splits, dev)
@@ -94,6 +110,6 @@ def polar_decode_attention(
         rc = _ffi.lib().pq_decode_attn(
             q.data_ptr(), *cptr, g_cap, n_groups, gps, kptr, r_cap, n_resid, rps,
             value_states.data_ptr(), v_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
-            n_splits, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
+            n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn")
     return out

@@ -3,8 +3,8 @@
 // (reference decode branch: models/modeling_llama_polar.py:66-99), split over
 // the context, followed by a small merge kernel.
 //
-// attn_kernel: grid (n_splits, B*Nk), one wavefront per block: block x works
-// through the x-th slice of the sequence's quantized groups; the last block of
+// attn_kernel: grid n_splits * B*Nk (plane index fastest), one wavefront per block: a block works
+// through one slice of its sequence's quantized groups; the last block of
 // a (batch, KV head) then also takes the fp16 residual keys (0..128 tokens).
 // The kernel is built for ONE resident wavefront per SIMD (4 per CU) with deep
 // software prefetch instead of many wavefronts: V operands are double-buffered
@@ -162,7 +162,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                  const int32_t* __restrict__ n_resid_per_seq,
                  const uint16_t* __restrict__ v, int64_t v_capacity,
                  const uint8_t* __restrict__ mask, int64_t mask_stride,
-                 float scale_log2, int N, int Nk, int rep, int n_splits, float* __restrict__ ws) {
+                 float scale_log2, int N, int Nk, int rep, int n_splits, int min_gps, float* __restrict__ ws) {
     using L = Lut<TB, REPP>;
     // the table region doubles as the fp32 query buffer of the residual block
     constexpr int kLutBytes = L::BYTES > REPP * kHeadDim * 4 ? L::BYTES : REPP * kHeadDim * 4;
@@ -171,8 +171,13 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
 
     const int lane = threadIdx.x;
-    const int split = blockIdx.x;
-    const int bh = blockIdx.y;
+    // 1-D grid, (batch, KV head) index fastest.  Consecutive workgroup ids go to different XCDs, so
+    // every XCD receives whole (batch, KV head) planes with all their slices; with the slice index
+    // fastest an XCD would receive one slice index of every plane, and in a ragged batch the XCDs
+    // that own the high slice indices would sit idle (measured: 165 us instead of 120 us).
+    const int units = gridDim.x / n_splits;
+    const int bh = blockIdx.x % units;
+    const int split = blockIdx.x / units;
     const int b = bh / Nk, kvh = bh - b * Nk;
 
     int nb = n_groups_per_seq ? n_groups_per_seq[b] : n_groups;
@@ -181,6 +186,17 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
     nres = nres < 0 ? 0 : (nres > resid_capacity ? resid_capacity : nres);
     int64_t n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
     n_tokens = n_tokens > v_capacity ? v_capacity : n_tokens;   // never read past the (batch, head) plane of V
+
+    // slices past the end of a short sequence have nothing to do: mark their partials empty and leave
+    {
+        int gps = (nb + n_splits - 1) / n_splits;
+        gps = gps < min_gps ? min_gps : gps;
+        if (split > 0 && split * gps >= nb) {
+            if (lane < rep)
+                ws[((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats] = -INFINITY;
+            return;
+        }
+    }
 
     const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
@@ -198,7 +214,10 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 
     {
         // ---------------- quantized groups [g0, g1) ----------------
-        const int gps = (nb + n_splits - 1) / n_splits;
+        // groups per slice: an even split of this sequence, but never fewer than min_gps (ragged
+        // batches: short sequences then use fewer slices, and the unused blocks return at once)
+        int gps = (nb + n_splits - 1) / n_splits;
+        gps = gps < min_gps ? min_gps : gps;
         const int g0 = split * gps;
         const int g1 = (g0 + gps) < nb ? (g0 + gps) : nb;
         if (g0 < g1) {
@@ -263,7 +282,14 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             }
         }
     }
-    if (split == n_splits - 1 && nres > 0) {
+    // the residual keys go to the block that holds the last quantized group of the sequence
+    int last_split = 0;
+    {
+        int gps = (nb + n_splits - 1) / n_splits;
+        gps = gps < min_gps ? min_gps : gps;
+        last_split = nb > 0 ? (nb - 1) / gps : 0;
+    }
+    if (split == last_split && nres > 0) {
         // ---------------- fp16 residual keys ----------------
         asm volatile("" ::: "memory");
         // q as fp32 in LDS: [REPP][128]
@@ -389,7 +415,7 @@ __global__ __launch_bounds__(kHeadDim) void merge_kernel(const float* __restrict
 template <typename T, int TB>
 static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     const int rep = a.N / a.Nk;
-    dim3 grid(a.n_splits, a.B * a.Nk), block(kWave);
+    dim3 grid(static_cast<unsigned>(a.n_splits) * static_cast<unsigned>(a.B * a.Nk)), block(kWave);
     const float scale_log2 = a.sm_scale * kLog2e;
 #define PQ_LAUNCH(REPP)                                                                                              \
     hipLaunchKernelGGL((attn_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,                \
@@ -397,7 +423,7 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.N, a.Nk, rep,        \
-                       a.n_splits, a.workspace)
+                       a.n_splits, a.min_groups_per_split, a.workspace)
     switch (rep_pad(rep)) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;

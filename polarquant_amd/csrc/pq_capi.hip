@@ -147,7 +147,7 @@ int pq_validate_decode_attn(const void* q,
                             const void* v, int64_t v_capacity,
                             const uint8_t* mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, const void* workspace, size_t workspace_bytes,
+                            int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
                             const void* out) {
     if (!q || !v || !workspace || !out) return PQ_ERR_NULL_POINTER;
     if (int rc = check_heads(B, N, Nk)) return rc;
@@ -169,7 +169,7 @@ int pq_validate_decode_attn(const void* q,
     if (mask && !n_groups_per_seq && !n_resid_per_seq &&
         mask_stride < static_cast<int64_t>(n_groups) * PQ_GROUP + n_resid) return PQ_ERR_BAD_STRIDE;
     if (!(sm_scale == sm_scale)) return PQ_ERR_BAD_SHAPE;
-    if (n_splits < 1 || n_splits > 65534) return PQ_ERR_WORKSPACE;
+    if (n_splits < 1 || n_splits > 65534 || min_groups_per_split < 0) return PQ_ERR_WORKSPACE;
     if (workspace_bytes < pq_decode_attn_workspace_bytes(B, N, n_splits)) return PQ_ERR_WORKSPACE;
     if (!aligned(q, 2) || !aligned(v, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return PQ_ERR_MISALIGNED;
     if (codes && !aligned(codes, 16)) return PQ_ERR_MISALIGNED;
@@ -185,12 +185,12 @@ int pq_decode_attn_partials(const void* q,
                             const void* v, int64_t v_capacity,
                             const uint8_t* mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, void* workspace, size_t workspace_bytes, void* stream) {
+                            int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes, void* stream) {
     // `out` is not touched by this half: validate with a stand-in non-null, aligned pointer
     if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
-                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, workspace,
-                                         workspace_bytes, workspace))
+                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
+                                         workspace, workspace_bytes, workspace))
         return rc;
     pq::AttnArgs a;
     a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
@@ -198,6 +198,7 @@ int pq_decode_attn_partials(const void* q,
     a.k_resid = k_resid; a.resid_capacity = resid_capacity; a.n_resid = n_resid; a.n_resid_per_seq = n_resid_per_seq;
     a.v = v; a.v_capacity = v_capacity; a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
     a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
+    a.min_groups_per_split = min_groups_per_split;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
@@ -224,13 +225,13 @@ int pq_decode_attn(const void* q,
                    const void* v, int64_t v_capacity,
                    const uint8_t* mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                   int n_splits, void* workspace, size_t workspace_bytes,
+                   int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
                    void* out, void* stream) {
     if (!out) return PQ_ERR_NULL_POINTER;
     if (int rc = pq_decode_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
-                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, workspace,
-                                         workspace_bytes, stream))
+                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
+                                         workspace, workspace_bytes, stream))
         return rc;
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }

@@ -30,7 +30,7 @@ struct AttnArgs {
     const uint8_t* mask;
     int64_t mask_stride;
     float sm_scale;
-    int B, N, Nk, tbits, dtype, n_splits;
+    int B, N, Nk, tbits, dtype, n_splits, min_groups_per_split;
     float* workspace;
     void* out;
 };

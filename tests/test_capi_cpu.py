@@ -89,19 +89,19 @@ def test_validate_decode_attn_and_plan(lib):
     B, N, Nk, ns = 2, 32, 8, 4
     wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
     assert wsb == B * N * ns * 132 * 4
-    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, 1024, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, P, wsb, P]
+    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, 1024, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P]
     assert lib.pq_validate_decode_attn(*ok) == 0
 
     def bad(i, v):
         a = list(ok); a[i] = v
         return lib.pq_validate_decode_attn(*a)
-    assert bad(0, None) == -1 and bad(13, None) == -1 and bad(25, None) == -1 and bad(27, None) == -1
+    assert bad(0, None) == -1 and bad(13, None) == -1 and bad(26, None) == -1 and bad(28, None) == -1
     assert bad(1, None) == -1            # groups > 0 but no codes
     assert bad(9, None) == -1            # residual > 0 but no residual keys
     assert bad(7, 5) == -6               # n_groups > capacity
     assert bad(11, 129) == -6            # n_resid > capacity
     assert bad(14, 3 * 128 + 4) == -6    # V capacity below tokens
-    assert bad(24, 0) == -7 and bad(26, wsb - 1) == -7
+    assert bad(24, 0) == -7 and bad(27, wsb - 1) == -7 and bad(25, -1) == -7
     assert bad(20, 5) == -2 and bad(22, 5) == -3 and bad(23, 3) == -4
     assert bad(13, P + 8) == -5
     a = list(ok); a[15] = P; a[16] = 100          # mask row shorter than the context
