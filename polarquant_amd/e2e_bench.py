@@ -5,7 +5,10 @@ Reports prefill seconds, decode tokens/s and KV-cache bytes per token.  Mirrors 
 reference's throughput script (benchmark/benchmark_throughput.py:15-113): one timed prefill,
 then the timed greedy loop with EOS made unreachable.
 
-    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32]
+    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32] [--graph]
+
+--graph replays the decode step from a captured HIP graph (polarquant_amd/graph_decode.py)
+instead of driving ~40 launches per layer from Python.
 """
 from __future__ import annotations
 
@@ -42,6 +45,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=16384)
     ap.add_argument("--new", type=int, default=256)
     ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--graph", action="store_true")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = PolarConfig.llama3_8b(num_hidden_layers=args.layers, cache_capacity=args.prompt + args.new + 128,
@@ -51,31 +55,48 @@ def main():
     ids = torch.randint(0, cfg.vocab_size, (args.batch, args.prompt), generator=g, device=dev)
     mask = torch.ones_like(ids)
     with torch.no_grad():
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        out = model(input_ids=ids, attention_mask=mask, past_key_values=None, num_logits_to_keep=1)
-        torch.cuda.synchronize()
-        t_prefill = time.perf_counter() - t0
-        cache = out.past_key_values
-        tok = out.logits.argmax(-1)
-        n_out = 1
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.new - 1):
-            mask = torch.cat([mask, torch.ones_like(tok)], dim=-1)
-            out = model(input_ids=tok, attention_mask=mask, past_key_values=cache, num_logits_to_keep=1)
+        if args.graph:
+            from .graph_decode import PolarGraphDecoder
+            dec = PolarGraphDecoder(model, max_len=args.prompt + args.new + 128)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            logits = dec.prefill(ids)
+            torch.cuda.synchronize()
+            t_prefill = time.perf_counter() - t0
+            tok = logits.argmax(-1)
+            tok = dec.step(tok).argmax(-1)          # capture happens on the first step: not timed
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.new - 2):
+                tok = dec.step(tok).argmax(-1)
+            torch.cuda.synchronize()
+            t_decode = time.perf_counter() - t0
+            steps = args.new - 2
+            cache = dec.cache()
+        else:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = model(input_ids=ids, attention_mask=mask, past_key_values=None, num_logits_to_keep=1)
+            torch.cuda.synchronize()
+            t_prefill = time.perf_counter() - t0
             cache = out.past_key_values
             tok = out.logits.argmax(-1)
-            n_out += 1
-        torch.cuda.synchronize()
-        t_decode = time.perf_counter() - t0
-    steps = args.new - 1
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.new - 1):
+                mask = torch.cat([mask, torch.ones_like(tok)], dim=-1)
+                out = model(input_ids=tok, attention_mask=mask, past_key_values=cache, num_logits_to_keep=1)
+                cache = out.past_key_values
+                tok = out.logits.argmax(-1)
+            torch.cuda.synchronize()
+            t_decode = time.perf_counter() - t0
+            steps = args.new - 1
     kv = model.kv_cache_bytes_per_token()
     fp16_kv = cfg.num_hidden_layers * cfg.num_key_value_heads * 2 * 128 * 2
     print(json.dumps({
         "workload": "configs[4]: greedy decode, random-init Llama-3-8B architecture, bf16, batch %d, prompt %d, %d new tokens"
                     % (args.batch, args.prompt, args.new),
-        "layers": args.layers, "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
+        "layers": args.layers, "graph": bool(args.graph), "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
         "decode_ms_per_step": round(1e3 * t_decode / steps, 3),
         "decode_tokens_per_s": round(args.batch * steps / t_decode, 1),
         "kv_cache_bytes_per_token": kv, "fp16_kv_cache_bytes_per_token": fp16_kv,
