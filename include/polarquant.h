@@ -53,6 +53,11 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
 /* flags for pq_quantize_groups */
 #define PQ_WRAP_FP32 1u /* add 2*pi in fp32 (eager CUDA semantics) instead of the
                            dtype-rounded 6.28125 that eager CPU torch adds */
+#define PQ_ANGLE_UNIFORM 2u /* fixed angle bins over [-pi, pi) instead of the group's own
+                               [min, max]: the reference formula (:148) with the constants
+                               tmn = -pi and tscale = 2*pi / 2^tbits, both rounded to the key
+                               dtype and written to the metadata tensors like any other, so
+                               the decode kernels need no switch.  No reference counterpart. */
 
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pq_version(void);

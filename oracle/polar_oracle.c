@@ -77,9 +77,12 @@ static uint8_t code_of(float v, float mn, float scale, int bits, int bf) {
 
 /* k: [B,Nk,L,2D] contiguous low-precision words.  Outputs contiguous:
  * codes [B,Nk,Nb,G,D] u8; rscale,rmn,tscale,tmn [B,Nk,Nb,D] low-precision words. */
-int po_quantize(const uint16_t *k, int bf, int wrap_fp32, int B, int Nk, int L, int D, int G, int rbits, int tbits,
+int po_quantize(const uint16_t *k, int bf, int flags, int B, int Nk, int L, int D, int G, int rbits, int tbits,
                 uint8_t *codes, uint16_t *rscale, uint16_t *rmn, uint16_t *tscale, uint16_t *tmn) {
     if (L % G || rbits + tbits > 8) return -1;
+    /* flags: bit 0 = wrap in fp32, bit 1 = uniform angle bins over [-pi, pi) (no reference
+     * counterpart: tmn = -pi, tscale = 2*pi / 2^tbits as key-dtype constants, no wrap) */
+    const int wrap_fp32 = flags & 1, uniform = (flags >> 1) & 1;
     /* torch-CPU casts the python scalar 2*pi to the tensor dtype before the add
      * (6.28125 in both half and bfloat16); wrap_fp32 != 0 keeps it in fp32, which
      * is what an eager CUDA add of a half tensor and a python scalar does. */
@@ -95,7 +98,7 @@ int po_quantize(const uint16_t *k, int bf, int wrap_fp32, int B, int Nk, int L, 
                 for (int g = 0; g < G; g++) {
                     float x = lo2f(base[(long)g * 2 * D + d], bf), y = lo2f(base[(long)g * 2 * D + D + d], bf);
                     float p = rnd(atan2f(y, x), bf);                       /* :143 */
-                    if (p < 0) p = rnd(p + TWO_PI, bf);                    /* :144 */
+                    if (p < 0 && !uniform) p = rnd(p + TWO_PI, bf);        /* :144 */
                     float r = rnd(sqrtf(x * x + y * y), bf);               /* :150 */
                     phi[g] = p; rad[g] = r;
                     if (p > pmx) pmx = p;
@@ -104,6 +107,10 @@ int po_quantize(const uint16_t *k, int bf, int wrap_fp32, int B, int Nk, int L, 
                     if (r < rmn_) rmn_ = r;
                 }
                 float ts = rnd(rnd(pmx - pmn, bf) / (float)(1 << tbits), bf);   /* :147 */
+                if (uniform) {
+                    pmn = rnd(-(float)3.14159265358979323846, bf);
+                    ts = rnd(rnd((float)(2.0 * 3.14159265358979323846), bf) / (float)(1 << tbits), bf);
+                }
                 float rs = rnd(rnd(rmx_ - rmn_, bf) / (float)(1 << rbits), bf); /* :152 */
                 long mi = (bh * Nb + nb) * D + d;
                 tscale[mi] = f2lo(ts, bf); tmn[mi] = f2lo(pmn, bf);

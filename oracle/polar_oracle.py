@@ -71,12 +71,16 @@ def _to_u8_defined(x: torch.Tensor) -> torch.Tensor:
 
 
 def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4,
-                           group_size: int = GROUP_SIZE):
+                           group_size: int = GROUP_SIZE, angle_mode: str = "group"):
     """key_states [B,Nk,L,2*D] half/bf16 (post-RoPE) ->
     (indices u8 [B,Nk,Nb,G,D], rscale, rmn, tscale, tmn [B,Nk,Nb,1,D] in key dtype).
 
     Every op runs eagerly in the key dtype, exactly as the reference does
     (modeling_llama_polar.py:141-155): x = dims [0,D), y = dims [D,2D).
+
+    angle_mode="uniform" (no reference counterpart; the fixed-grid special case of the same
+    formula): the angle is not wrapped, tmn = -pi and tscale = 2*pi / 2^tbits as key-dtype
+    constants, theta by line :148 unchanged.
     """
     B, N, L, D2 = key_states.shape
     assert D2 % 2 == 0 and L % group_size == 0 and rbits + tbits <= 8
@@ -84,9 +88,13 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     ks = key_states.reshape(B, N, L // G, G, 2, D)
 
     phi = torch.atan2(ks[:, :, :, :, 1, :], ks[:, :, :, :, 0, :])             # :143
-    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)                        # :144
-    tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]      # :146
-    tscale = (tmx - tmn) / (2 ** tbits)                                       # :147
+    if angle_mode == "uniform":
+        tmn = torch.full_like(phi[..., :1, :], -math.pi)
+        tscale = torch.full_like(tmn, 2 * math.pi) / (2 ** tbits)
+    else:
+        phi = torch.where(phi < 0, phi + 2 * math.pi, phi)                    # :144
+        tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]  # :146
+        tscale = (tmx - tmn) / (2 ** tbits)                                   # :147
     theta = torch.clamp(_to_u8_defined((phi - tmn) / tscale), 0, 2 ** tbits - 1)  # :148
 
     radii = torch.norm(ks, p=2, dim=-2)                                       # :150

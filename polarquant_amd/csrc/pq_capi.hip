@@ -82,7 +82,7 @@ int pq_validate_quantize_groups(const void* k, const int64_t* k_strides, int dty
         return PQ_ERR_BAD_SHAPE;
     if (rbits < 1 || tbits < 1 || rbits + tbits > 8) return PQ_ERR_BAD_BITS;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
-    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32)) return PQ_ERR_BAD_SHAPE;
+    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM)) return PQ_ERR_BAD_SHAPE;
     if (k_strides[3] != 1) return PQ_ERR_BAD_STRIDE;
     if (k_strides[0] < 0 || k_strides[1] < 0 || k_strides[2] < PQ_HEAD_DIM) return PQ_ERR_BAD_STRIDE;
     if (out_group_offset < 0 || out_group_capacity < out_group_offset + Nb) return PQ_ERR_BAD_STRIDE;

@@ -15,7 +15,7 @@ PAIRS = 64
 
 
 def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4, group_size: int = GROUP,
-                           wrap_fp32: bool = False,
+                           wrap_fp32: bool = False, angle_mode: str = "group",
                            out: Optional[Tuple[torch.Tensor, ...]] = None, group_offset: int = 0):
     """key_states [B,Nk,L,128] half/bf16 on the GPU (any batch/head/token strides, unit dim stride)
     -> (indices u8 [B,Nk,Nb,128,64], rscale, rmn, tscale, tmn [B,Nk,Nb,1,64]).
@@ -23,7 +23,12 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     `out`, if given, is a 5-tuple of pre-allocated cache tensors
     ([B,Nk,cap,128,64] u8 and four [B,Nk,cap,1,64]) that receive the Nb new groups
     at group index `group_offset`; nothing is allocated then.
+
+    `angle_mode="group"` is the reference's binning (2^tbits bins over each group's own angle
+    range); `"uniform"` uses fixed bins over [-pi, pi) and writes the constants
+    tmn = -pi, tscale = 2*pi/2^tbits into the metadata, so decode is unchanged.
     """
+    assert angle_mode in ("group", "uniform")
     if not key_states.is_cuda:
         raise RuntimeError("polarquant_amd: the quantizer needs tensors on the GPU (no CPU fallback)")
     B, Nk, L, D2 = key_states.shape
@@ -45,7 +50,7 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     strides = (ctypes.c_int64 * 4)(*key_states.stride())
     with torch.cuda.device(dev):
         rc = _ffi.lib().pq_quantize_groups(key_states.data_ptr(), ctypes.cast(strides, ctypes.c_void_p), dt, B, Nk, Nb,
-                                           rbits, tbits, _ffi.PQ_WRAP_FP32 if wrap_fp32 else 0,
+                                           rbits, tbits, (_ffi.PQ_WRAP_FP32 if wrap_fp32 else 0) | (_ffi.PQ_ANGLE_UNIFORM if angle_mode == "uniform" else 0),
                                            codes.data_ptr(), *[m.data_ptr() for m in meta], cap, off,
                                            _stream_ptr(dev))
     _ffi.check(rc, "pq_quantize_groups")

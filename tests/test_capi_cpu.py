@@ -71,7 +71,8 @@ def test_validate_quantize_groups(lib):
     assert bad(3, 0) == -2 and bad(5, 0) == -2
     assert bad(6, 5) == -3 and bad(7, 0) == -3
     assert bad(2, 7) == -4
-    assert bad(8, 2) == -2                           # unknown flag bit
+    assert bad(8, 1) == 0 and bad(8, 2) == 0 and bad(8, 3) == 0   # PQ_WRAP_FP32, PQ_ANGLE_UNIFORM
+    assert bad(8, 4) == -2                           # unknown flag bit
     assert bad(14, 1) == -6 and bad(15, 1) == -6     # capacity < offset + Nb
     assert bad(0, P + 2) == -5                       # key pointer not 8-byte aligned
     for i, s in enumerate([(8 * 256 * 128, 256 * 128, 128, 2), (8 * 256 * 128, 256 * 128, 64, 1),

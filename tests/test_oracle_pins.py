@@ -106,6 +106,41 @@ def test_quantizer_vs_fp64_brute_force_counts_edge_flips():
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("tb", [4, 3])
+def test_uniform_angle_mode_known_answers(dtype, tb):
+    """Fixed angle bins over [-pi, pi): keys placed on the bin centres -pi + (j + 0.5) * 2*pi/2^t
+    must get theta == j, the metadata must hold the constants -pi and 2*pi/2^t (rounded to the
+    dtype), the radius side must be untouched by the mode, and the two restatements must agree."""
+    G, D, rb = 128, 64, 4
+    w = 2 * math.pi / 2 ** tb
+    g = torch.Generator().manual_seed(5)
+    jj = torch.randint(0, 2 ** tb, (G, D), generator=g)
+    ang = -math.pi + (jj.double() + 0.5) * w
+    rad = 0.5 + 3 * torch.rand(G, D, generator=g, dtype=torch.float64)
+    keys = torch.cat([rad * torch.cos(ang), rad * torch.sin(ang)], dim=-1).to(dtype).reshape(1, 1, G, 2 * D)
+    ref_group = po.quantize_and_pack_nbit(keys, rb, tb)
+    for quant in (po.quantize_and_pack_nbit, co.quantize):
+        codes, rscale, rmn, tscale, tmn = quant(keys, rb, tb, angle_mode="uniform")
+        assert torch.equal(codes[0, 0, 0] & (2 ** tb - 1), jj.to(torch.uint8))
+        assert torch.equal(codes >> tb, ref_group[0] >> tb)                     # radius codes: same as reference mode
+        assert torch.equal(rscale, ref_group[1]) and torch.equal(rmn, ref_group[2])
+        assert torch.equal(tmn, torch.full_like(tmn, -math.pi))
+        assert torch.equal(tscale, torch.full_like(tscale, 2 * math.pi) / 2 ** tb)
+        assert abs(float(tmn.flatten()[0]) + math.pi) < 2e-2 and abs(float(tscale.flatten()[0]) - w) < 2e-3
+    # random keys: both restatements, every angle within half a bin of its bin centre
+    k, _ = _keys(1, 2, 512, 6, dtype)
+    a = po.quantize_and_pack_nbit(k, rb, tb, angle_mode="uniform")
+    b = co.quantize(k, rb, tb, angle_mode="uniform")
+    assert int((a[0] != b[0]).sum()) <= 1e-4 * a[0].numel()
+    assert all(torch.equal(x, y) for x, y in zip(a[1:], b[1:]))
+    ks = k.double().reshape(1, 2, 4, 128, 2, 64)
+    phi = torch.atan2(ks[..., 1, :], ks[..., 0, :])
+    centre = a[4].double() + ((a[0] & (2 ** tb - 1)).double() + 0.5) * a[3].double()
+    tol = 1e-2 if dtype == torch.float16 else 5e-2
+    assert float((phi - centre).abs().max()) <= w / 2 + tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (5, 3)])
 def test_c_and_torch_restatements_agree(dtype, rbits, tbits):
     """Two independent restatements (torch eager ops with SLEEF atan2 / scalar C with libm atan2f)."""

@@ -102,6 +102,30 @@ def test_quantize_special_values(gpu):
     assert all(v == 0 for v in flips.values()), flips
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3)])
+def test_quantize_uniform_angle_mode(gpu, dtype, rbits, tbits):
+    """Fixed angle bins over [-pi, pi): bit-exact against the oracle's same mode, and the cache
+    it writes is decoded by the unchanged score kernel."""
+    from polarquant_amd.kernel4group import attention_decode_forward_triton_impl
+    print("case uniform", dtype, rbits, tbits, flush=True)
+    g = torch.Generator().manual_seed(23)
+    k = wl.make_keys(2, 4, 1024, 5e5, g, dtype)
+    ref = po.quantize_and_pack_nbit(k, rbits, tbits, angle_mode="uniform")
+    got = quantize_and_pack_nbit(k.to(gpu), rbits, tbits, angle_mode="uniform")
+    flips = count_flips(got, ref)
+    print("flips", flips, flush=True)
+    assert all(v == 0 for v in flips.values()), flips
+    q = wl.make_half((2, 8, 1, 128), g, dtype)
+    want = po.decode_scores(q, *ref, rbits, tbits)
+    have = attention_decode_forward_triton_impl(q.to(gpu), *got, rbits=rbits, tbits=tbits).cpu()
+    assert (have - want).abs().max().item() <= 1e-3 * want.abs().max().item()
+    # and they approximate the scores of the unquantized keys
+    exact = torch.matmul(q.float(), po.repeat_kv(k, 2).float().transpose(2, 3))
+    rel = (have - exact).norm() / exact.norm()
+    assert rel < (0.15 if tbits == 4 else 0.3), rel    # quantization noise of a fixed 2*pi/2^t grid
+
+
 def test_quantize_wrap_fp32_flag(gpu):
     """PQ_WRAP_FP32 adds 2*pi in fp32 (what an eager GPU add of a half tensor and a
     python float does); checked against the plain-C oracle's same switch."""
