@@ -204,6 +204,61 @@ int pq_decode_attn_partials(const void *q,
 int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
                          void *out, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * 4-bit values: the reference's Mixed variant (LlamaPolarMixedGroupAttention,
+ * models/modeling_llama_polar.py:158-292).
+ *
+ * pq_quantize_values replaces triton_quantize_and_pack_along_last_dim(values, 128, 4)
+ * at :236 and :275 (a routine of the kivi_quant package, which is not in the
+ * reference tree; its published form is followed): per token and head, over the
+ * 128 dims, scale = (max - min) / 15, code = round_half_even(clamp((x - min) / scale, 0, 15)),
+ * each op rounded to the value dtype; 8 codes per int32, dim 8w+i in bits [4i, 4i+4)
+ * of word w.  A constant row (0/0) yields code 0.
+ *   v        [B,Nk,T,128] half words, element strides v_strides[4] (dim stride 1,
+ *            the others multiples of 8), 16-byte aligned
+ *   codes    int32 [B,Nk,out_token_capacity,16]; scale, zero [B,Nk,out_token_capacity]
+ *            (the reference's [..., 1] tensors); rows out_token_offset .. +T are written
+ *
+ * pq_decode_attn_v4 replaces the decode branch :185-241 between RoPE and o_proj:
+ * as pq_decode_attn, but the values of the quantized groups are 4-bit
+ * (v_codes / v_scale / v_zero, token t of a sequence is row t, rows
+ * [0, n_groups*128) are read; :229-236 cuda_bmm_fA_qB_outer) and `v_resid`
+ * [B,Nk,resid_capacity,128] holds the half-precision values of the residual
+ * window only, row r belonging to residual key r (:238).  Keys and values
+ * share the window's fill (n_resid) and are flushed together (:207,:243).
+ * ------------------------------------------------------------------------- */
+int pq_quantize_values(const void *v, const int64_t *v_strides, int dtype, int B, int Nk, int T,
+                       int32_t *codes, void *scale, void *zero,
+                       int64_t out_token_capacity, int64_t out_token_offset, void *stream);
+
+int pq_validate_quantize_values(const void *v, const int64_t *v_strides, int dtype, int B, int Nk, int T,
+                                const int32_t *codes, const void *scale, const void *zero,
+                                int64_t out_token_capacity, int64_t out_token_offset);
+
+int pq_decode_attn_v4(const void *q,
+                      const uint8_t *codes, const void *rscale, const void *rmn,
+                      const void *tscale, const void *tmn, int group_capacity,
+                      int n_groups, const int32_t *n_groups_per_seq,
+                      const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                      const void *v_resid,
+                      const int32_t *v_codes, const void *v_scale, const void *v_zero, int64_t v4_capacity,
+                      const uint8_t *mask, int64_t mask_stride,
+                      float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                      int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
+                      void *out, void *stream);
+
+int pq_validate_decode_attn_v4(const void *q,
+                               const uint8_t *codes, const void *rscale, const void *rmn,
+                               const void *tscale, const void *tmn, int group_capacity,
+                               int n_groups, const int32_t *n_groups_per_seq,
+                               const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                               const void *v_resid,
+                               const int32_t *v_codes, const void *v_scale, const void *v_zero, int64_t v4_capacity,
+                               const uint8_t *mask, int64_t mask_stride,
+                               float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                               int n_splits, int min_groups_per_split, const void *workspace, size_t workspace_bytes,
+                               const void *out);
+
 /* Suggested n_splits for a shape (host-only; `max_groups` = largest group count
  * of any sequence, `n_cus` = compute units of the device or 0 for 256). */
 int pq_decode_attn_plan(int B, int Nk, int max_groups, int n_cus);

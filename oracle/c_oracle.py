@@ -49,6 +49,19 @@ def quantize(key_states: torch.Tensor, rbits=4, tbits=4, group_size=128, wrap_fp
     return (torch.from_numpy(codes),) + tuple(back(m) for m in meta)
 
 
+def quantize_values(v: torch.Tensor, bits=4):
+    """[B,Nk,T,128] -> (int32 [B,Nk,T,16], scale [B,Nk,T,1], mn [B,Nk,T,1])"""
+    B, Nk, T, D = v.shape
+    bf = int(v.dtype == torch.bfloat16)
+    per = 32 // bits
+    codes = np.empty((B, Nk, T, D // per), np.int32)
+    scale, mn = np.empty((B, Nk, T, 1), np.uint16), np.empty((B, Nk, T, 1), np.uint16)
+    rc = lib().po_quantize_values(_p(_words(v)), bf, ctypes.c_long(B * Nk * T), D, bits, _p(codes), _p(scale), _p(mn))
+    assert rc == 0
+    back = lambda m: torch.from_numpy(m.view(np.int16)).view(v.dtype)
+    return torch.from_numpy(codes), back(scale), back(mn)
+
+
 def scores(q, codes, rscale, rmn, tscale, tmn, rbits=4, tbits=4):
     B, N = q.shape[:2]
     _, Nk, Nb, G, D = codes.shape

@@ -125,6 +125,42 @@ int po_quantize(const uint16_t *k, int bf, int flags, int B, int Nk, int L, int 
     return 0;
 }
 
+/* 4-bit values of the Mixed variant (models/modeling_llama_polar.py:236,275 call
+ * triton_quantize_and_pack_along_last_dim(values, 128, 4) of a kivi_quant package that is not in
+ * the reference tree; restated from KIVI's published quant/new_pack.py).
+ * v: [rows, D] contiguous low-precision words, one quantization group per row (D == group size).
+ * codes: [rows, D*bits/32] int32, element i of each run of 32/bits in bits [i*bits, (i+1)*bits);
+ * scale, mn: [rows] low-precision words. */
+int po_quantize_values(const uint16_t *v, int bf, long rows, int D, int bits, int32_t *codes, uint16_t *scale,
+                       uint16_t *mn) {
+    if (bits <= 0 || 32 % bits || D % (32 / bits)) return -1;
+    const int per = 32 / bits, top = (1 << bits) - 1;
+    for (long r = 0; r < rows; r++) {
+        const uint16_t *row = v + r * D;
+        float lo = INFINITY, hi = -INFINITY;
+        for (int d = 0; d < D; d++) {
+            float x = lo2f(row[d], bf);
+            if (x < lo) lo = x;
+            if (x > hi) hi = x;
+        }
+        float sc = rnd(rnd(hi - lo, bf) / (float)top, bf);
+        scale[r] = f2lo(sc, bf); mn[r] = f2lo(lo, bf);
+        for (int w = 0; w < D / per; w++) {
+            uint32_t word = 0;
+            for (int i = 0; i < per; i++) {
+                float q = rnd(rnd(lo2f(row[w * per + i], bf) - lo, bf) / sc, bf);
+                if (q < 0) q = 0;
+                if (q > top) q = (float)top;
+                q = nearbyintf(q);                        /* round half to even (default rounding mode) */
+                uint32_t c = (q == q) ? (uint32_t)q : 0u; /* 0/0 on a constant row -> 0 (defined here) */
+                word |= c << (i * bits);
+            }
+            codes[r * (D / per) + w] = (int32_t)word;
+        }
+    }
+    return 0;
+}
+
 /* scores[b,h,l] = sum_d (q[d] cos phi^ + q[d+D] sin phi^) * r^ ; out [B,N,Nb*G] fp32 */
 int po_scores(const uint16_t *q, int bf, const uint8_t *codes, const uint16_t *rscale, const uint16_t *rmn,
               const uint16_t *tscale, const uint16_t *tmn, float *out,

@@ -24,6 +24,19 @@ the checks live in tests/test_oracle_pins.py):
                            over the concatenated dequantized+residual keys.
   prefill_cache/decode_step pinned: shape/bookkeeping property tests (quantized
                            token count, residual length, kv_seq_len).
+  quantize_values_along_last_dim / dequantize_values / decode_attention_mixed
+                           (4-bit values of the reference's Mixed variant):
+                           the routines the reference calls live in a kivi_quant
+                           package that is NOT in its tree and carries no version
+                           pin; they are restated from KIVI's published source.
+                           Pinned by what the mathematics fixes: closed-form row
+                           (codes and packed words known), min->0 / max->2^b-1,
+                           |v - v^| <= scale/2, round-half-even, independent C
+                           restatement, fp64 one-shot attention over dequantized
+                           values.  PARITY UNPINNED: the nibble order inside a
+                           packed int32 and the rounding mode are taken from the
+                           published KIVI source, which nothing in the reference
+                           tree confirms.
   Degenerate groups (tscale==0 or rscale==0 -> 0/0) are undefined behaviour in
   the reference (NaN -> uint8); this oracle defines the code as 0 there, which
   is what torch-CPU's cast yields.  That choice is "parity unpinned".
@@ -274,6 +287,126 @@ def decode_step(query_states, key_states, value_states, past_key_value, attentio
         ind, rs, rm, ts, tm = cat(ind, i2), cat(rs, rs2), cat(rm, rm2), cat(ts, ts2), cat(tm, tm2)
         k_full = None
     return out, (k_full, ind, rs, rm, ts, tm, v_full, kv_len + 1)
+
+
+# --------------------------------------------------------------------------
+# 4-bit values of the Mixed variant (models/modeling_llama_polar.py:158-292).
+# The reference imports triton_quantize_and_pack_along_last_dim and
+# cuda_bmm_fA_qB_outer from `.kivi_quant` (modeling_llama_polar.py:18-19), a
+# directory that is absent from its tree and has no pinned version.  What
+# follows restates the published KIVI routines (github.com/jy-yuan/KIVI,
+# quant/new_pack.py: triton_quantize_and_pack_along_last_dim, _pack_along_last_dim;
+# quant/matmul.py + csrc: cuda_bmm_fA_qB_outer), anchored on the reference's call
+# sites: values [B,Nk,T,128] are quantized per token along the 128 dims with
+# group size 128 (:236,:275: one group per token and head), 4 bits (:161).
+# --------------------------------------------------------------------------
+def quantize_values_along_last_dim(data: torch.Tensor, group_size: int = GROUP_SIZE, bits: int = 4):
+    """data [B,Nk,T,D] half/bf16 -> (code int32 [B,Nk,T,D*bits/32], scale [B,Nk,T,D/group], mn [B,Nk,T,D/group]).
+
+    Eager ops in the data dtype, as KIVI does them: scale = (mx - mn) / (2^bits - 1);
+    q = round(clamp((x - mn) / scale, 0, 2^bits - 1)) (torch.round: half to even);
+    32/bits consecutive codes share an int32, element i in bits [i*bits, (i+1)*bits)."""
+    B, nh, T, D = data.shape
+    assert D % group_size == 0 and 32 % bits == 0
+    ng = D // group_size
+    x = data.reshape(B * nh * T, ng, group_size)
+    mn, mx = x.min(dim=-1)[0], x.max(dim=-1)[0]
+    scale = (mx - mn) / (2 ** bits - 1)
+    x = x - mn.unsqueeze(-1)
+    x = x / scale.unsqueeze(-1)
+    x = x.clamp(0, 2 ** bits - 1).round()
+    x = torch.where(torch.isfinite(x), x, torch.zeros_like(x)).to(torch.int32)      # constant row: 0/0 -> code 0 (defined here)
+    per = 32 // bits
+    x = x.reshape(B * nh * T, D // per, per).to(torch.int64)
+    shifts = torch.arange(per, dtype=torch.int64) * bits
+    word = (x << shifts).sum(-1)                                                     # disjoint bit fields: sum == or
+    word = torch.where(word >= 2 ** 31, word - 2 ** 32, word).to(torch.int32)        # two's complement int32
+    return word.view(B, nh, T, D // per), scale.reshape(B, nh, T, ng), mn.reshape(B, nh, T, ng)
+
+
+def unpack_values(code: torch.Tensor, bits: int = 4) -> torch.Tensor:
+    """int32 [..., W] -> integer codes [..., W*32/bits] (int64)."""
+    per = 32 // bits
+    w = code.to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(per, dtype=torch.int64) * bits
+    return ((w.unsqueeze(-1) >> shifts) & (2 ** bits - 1)).reshape(*code.shape[:-1], code.shape[-1] * per)
+
+
+def dequantize_values(code, scale, mn, bits: int = 4, dtype=torch.float32) -> torch.Tensor:
+    """-> [B,Nk,T,128]: q * scale + zero, as cuda_bmm_fA_qB_outer forms each weight (group size 128:
+    one scale / zero per token and head)."""
+    return unpack_values(code, bits).to(dtype) * scale.to(dtype) + mn.to(dtype)
+
+
+def decode_attention_mixed(query_states, key_resid, indices, rscale, rmn, tscale, tmn,
+                           value_resid, value_codes, value_scale, value_mn,
+                           attention_mask: Optional[torch.Tensor] = None, rbits: int = 4, tbits: int = 4,
+                           vbits: int = 4) -> torch.Tensor:
+    """One decode step of LlamaPolarMixedGroupAttention (:185-241), AFTER the new key / value were
+    appended to key_resid / value_resid.  value_resid [B,Nk,res,128] (res >= 1), value_codes /
+    value_scale / value_mn for the tokens before it, or None."""
+    B, N, _, hd = query_states.shape
+    Nk = value_resid.shape[1]
+    rep = N // Nk
+    parts = []
+    if indices is not None:
+        parts.append(decode_scores(query_states, indices, rscale, rmn, tscale, tmn, rbits, tbits).to(torch.float32))  # :189-199
+    w = torch.matmul(query_states.float(), repeat_kv(key_resid, rep).float().transpose(2, 3))                           # :203
+    parts.append(w.to(query_states.dtype).to(torch.float32))
+    attn = torch.cat(parts, dim=-1) / math.sqrt(hd)                                                                     # :204
+    if attention_mask is not None:
+        attn = attn + (1.0 - attention_mask[:, None, None, :].to(torch.float32)) * torch.finfo(torch.float32).min       # :219-220
+    p = torch.softmax(attn, dim=-1).to(query_states.dtype)                                                               # :222
+    vfl = value_resid.shape[2]
+    if value_codes is None:
+        return torch.matmul(p.float(), repeat_kv(value_resid, rep).float()).to(query_states.dtype)                      # :227
+    vhat = dequantize_values(value_codes, value_scale, value_mn, vbits)
+    out = torch.matmul(p[..., :-vfl].float(), repeat_kv(vhat, rep)).to(value_scale.dtype)                                # :229-236
+    return out + torch.matmul(p[..., -vfl:].float(), repeat_kv(value_resid, rep).float()).to(query_states.dtype)        # :238
+
+
+def decode_attention_mixed_exact(query_states, key_resid, indices, rscale, rmn, tscale, tmn,
+                                 value_resid, value_codes, value_scale, value_mn, attention_mask=None,
+                                 rbits=4, tbits=4, vbits=4) -> torch.Tensor:
+    """Same step as one fp64 softmax attention over [dequantized ; residual] keys and values."""
+    v = value_resid.to(torch.float64)
+    if value_codes is not None:
+        v = torch.cat([dequantize_values(value_codes, value_scale, value_mn, vbits, torch.float64), v], dim=2)
+    return decode_attention_exact(query_states, key_resid, indices, rscale, rmn, tscale, tmn, v, attention_mask, rbits, tbits)
+
+
+def prefill_cache_mixed(key_states, value_states, rbits=4, tbits=4, vbits=4, residual_length=GROUP_SIZE):
+    """Prompt keys/values -> the Mixed variant's 11-tuple (:259-281)."""
+    k_full, ind, rs, rm, ts, tm, _, L = prefill_cache(key_states, value_states, rbits, tbits, residual_length)
+    r = L % residual_length
+    if r == 0:
+        v_full, v_quant = None, value_states
+    else:
+        v_full = value_states if L < residual_length else value_states[:, :, -r:, :]
+        v_quant = None if L < residual_length else value_states[:, :, :-r, :]
+    vc = vs = vm = None
+    if v_quant is not None:
+        vc, vs, vm = quantize_values_along_last_dim(v_quant.contiguous(), residual_length, vbits)
+    return (k_full, ind, rs, rm, ts, tm, v_full, vc, vs, vm, L)
+
+
+def decode_step_mixed(query_states, key_states, value_states, past_key_value, attention_mask=None,
+                      rbits=4, tbits=4, vbits=4, residual_length=GROUP_SIZE):
+    """One Mixed decode step on post-RoPE q/k/v [B,H,1,128] (:185-257) -> (attn_output, new 11-tuple)."""
+    k_full, ind, rs, rm, ts, tm, v_full, vc, vs, vm, kv_len = past_key_value
+    cat = lambda a, b: b if a is None else torch.cat([a, b], dim=2)
+    k_full, v_full = cat(k_full, key_states), cat(v_full, value_states)                     # :201, :223
+    out = decode_attention_mixed(query_states, k_full, ind, rs, rm, ts, tm, v_full, vc, vs, vm, attention_mask,
+                                 rbits, tbits, vbits)
+    if k_full.shape[2] % residual_length == 0:                                              # :207
+        q5 = quantize_and_pack_nbit(k_full.contiguous(), rbits, tbits, residual_length)
+        ind, rs, rm, ts, tm = [cat(a, b) for a, b in zip((ind, rs, rm, ts, tm), q5)]
+        k_full = None
+    if v_full.shape[2] % residual_length == 0:                                              # :243
+        c2, s2, m2 = quantize_values_along_last_dim(v_full.contiguous(), residual_length, vbits)
+        vc, vs, vm = cat(vc, c2), cat(vs, s2), cat(vm, m2)
+        v_full = None
+    return out, (k_full, ind, rs, rm, ts, tm, v_full, vc, vs, vm, kv_len + 1)
 
 
 # --------------------------------------------------------------------------

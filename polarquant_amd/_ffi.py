@@ -44,6 +44,18 @@ SIGNATURES = {
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
                                 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "pq_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "pq_quantize_values": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                   c_int64, c_int64, c_void_p]),
+    "pq_validate_quantize_values": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                            c_int64, c_int64]),
+    "pq_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                                   c_void_p, c_int64, c_float]
+                          + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_void_p]),
+    "pq_validate_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                                            c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                                            c_void_p, c_int64, c_float]
+                                   + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),
     "pq_decode_attn_workspace_bytes": (c_size_t, [c_int] * 3),
 }

@@ -113,3 +113,66 @@ def polar_decode_attention(
             n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn")
     return out
+
+
+def polar_decode_attention_v4(
+    query_states: torch.Tensor,               # [B,N,1,128] or [B,N,128]
+    indices: Optional[torch.Tensor], rscale: Optional[torch.Tensor], rmn: Optional[torch.Tensor],
+    tscale: Optional[torch.Tensor], tmn: Optional[torch.Tensor],
+    key_resid: torch.Tensor,                  # [B,Nk,res_cap,128] keys of the residual window (new key included)
+    value_resid: torch.Tensor,                # [B,Nk,res_cap,128] values of the same window
+    value_codes: Optional[torch.Tensor],      # int32 [B,Nk,cap_tokens,16]; rows [0, n_groups*128) are used
+    value_scale: Optional[torch.Tensor], value_mn: Optional[torch.Tensor],   # [B,Nk,cap_tokens,1]
+    n_groups: int, n_resid: int,
+    attention_mask: Optional[torch.Tensor] = None,
+    rbits: int = 4, tbits: int = 4, sm_scale: Optional[float] = None,
+    n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
+    n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None, min_groups_per_split: int = 0,
+) -> torch.Tensor:
+    """Decode attention of the reference's Mixed variant (polar keys + 4-bit values,
+    models/modeling_llama_polar.py:185-241) -> [B,N,1,128] in the query dtype."""
+    if not query_states.is_cuda:
+        raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
+    dev = query_states.device
+    B, N = query_states.shape[:2]
+    hd = query_states.shape[-1]
+    Nk = key_resid.shape[1]
+    assert hd == 128
+    dt = _dtype_code(query_states)
+    q = query_states.reshape(B, N, hd)
+    if not q.is_contiguous():
+        q = q.contiguous()
+    assert key_resid.is_contiguous() and value_resid.is_contiguous() and key_resid.shape == value_resid.shape
+    assert key_resid.dtype == query_states.dtype == value_resid.dtype
+    r_cap = key_resid.shape[2]
+    if indices is not None:
+        assert indices.is_contiguous() and all(m.is_contiguous() for m in (rscale, rmn, tscale, tmn))
+        assert value_codes is not None and value_codes.is_contiguous() and value_codes.dtype == torch.int32
+        assert value_scale.is_contiguous() and value_mn.is_contiguous() and value_scale.dtype == query_states.dtype
+        g_cap, v4_cap = indices.shape[2], value_codes.shape[2]
+        cptr = [indices.data_ptr(), rscale.data_ptr(), rmn.data_ptr(), tscale.data_ptr(), tmn.data_ptr()]
+        vptr = [value_codes.data_ptr(), value_scale.data_ptr(), value_mn.data_ptr()]
+    else:
+        g_cap, v4_cap, cptr, vptr = 0, 0, [None] * 5, [None] * 3
+    mptr, mstride = None, 0
+    if attention_mask is not None:
+        m8 = attention_mask if attention_mask.dtype == torch.uint8 else (attention_mask != 0).to(torch.uint8)
+        m8 = m8.contiguous()
+        mptr, mstride = m8.data_ptr(), m8.stride(0)
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(hd)
+    max_groups = g_cap if n_groups_per_seq is not None else n_groups
+    if n_splits is None:
+        n_splits = plan_splits(B, Nk, max_groups, dev)
+    ws = workspace_for(B, N, n_splits, dev)
+    if out is None:
+        out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
+    gps = n_groups_per_seq.data_ptr() if n_groups_per_seq is not None else None
+    rps = n_resid_per_seq.data_ptr() if n_resid_per_seq is not None else None
+    with torch.cuda.device(dev):
+        rc = _ffi.lib().pq_decode_attn_v4(
+            q.data_ptr(), *cptr, g_cap, n_groups, gps, key_resid.data_ptr(), r_cap, n_resid, rps,
+            value_resid.data_ptr(), *vptr, v4_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
+            n_splits, min_groups_per_split, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
+    _ffi.check(rc, "pq_decode_attn_v4")
+    return out

@@ -62,6 +62,7 @@ struct AttnState {
     float m[REPP];        // running maximum (log2 units), wave-uniform
     float l[REPP];        // per-lane partial sum of probabilities
     floatx4 acc[8];       // lane (g,n): acc[e][i] = out_head_n[dim 8*(4g+i)+e]
+    float zp[REPP];       // 4-bit values only: per-lane partial sum of p * zero-point of the token
 };
 
 #pragma clang diagnostic push
@@ -123,6 +124,107 @@ __device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// ---- 4-bit values (the Mixed variant, models/modeling_llama_polar.py:158-292) ----
+// A cached value row is 16 int32 words; word n holds dims 8n..8n+7, dim 8n+e in bits [4e, 4e+4),
+// with one (scale, zero-point) pair per token and head: v^ = code * scale + zero.  Then
+//     sum_t p_t v^_t[dim] = sum_t (p_t scale_t) code_t[dim]  +  sum_t p_t zero_t
+// and only the first term needs the matrix cores.  Lane (g,n) owns exactly word n of its tokens,
+// so the MFMA row for dim 8n+e is nibble e of that word.  A nibble isolated in a byte and
+// zero-extended to 16 bits IS the half-precision subnormal code * 2^-24 (odd nibbles are left in
+// the high half of their byte: 16 * code * 2^-24), which v_mfma_f32_16x16x16_f16 multiplies
+// exactly; so the A operand costs two v_and per word and one v_perm per register, like the
+// half-precision rows it replaces, and the accumulators are brought back to real units once,
+// after the last quantized tile (finish_v4).  The probabilities go through half precision for
+// this product whatever the model dtype; kV4Pre keeps p * scale inside its range.
+constexpr float kV4Pre = 0x1p-6f;
+constexpr float kV4PostEven = 0x1p30f;   // 2^24 / kV4Pre
+constexpr float kV4PostOdd = 0x1p26f;    // nibble left at 16 * code
+
+// Tokens of a 16-token block are handed to the MFMA k-index transposed (k = 4g+i <-> token 4i+g),
+// so that one load instruction of a wavefront covers 4 whole consecutive rows (256 contiguous
+// bytes).  v4_slot is where lane == token puts its probability so that the B operand agrees.
+__device__ __forceinline__ int v4_slot(int lane) { return (lane & 48) | ((lane & 3) << 2) | ((lane >> 2) & 3); }
+
+//   vq[tb][i]  word n of token 16*tb + 4*i + g
+//   sc, zp     this lane's token's scale and zero-point (lane == token)
+template <int REPP>
+__device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&t)[REPP], const uint32_t (&vq)[4][4],
+                                                   float sc, float zp, uint32_t pbuf, int lane) {
+    bool raise = false;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) raise |= t[j] > st.m[j] + kLazyThreshold;
+    if (__any(raise)) {
+        float alpha[REPP];
+#pragma unroll
+        for (int j = 0; j < REPP; j++) {
+            const float mn = fmaxf(st.m[j], wave_max(t[j]));
+            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2f(st.m[j] - mn);
+            st.m[j] = mn;
+            st.l[j] *= alpha[j];
+            st.zp[j] *= alpha[j];
+        }
+        float a = alpha[0];
+#pragma unroll
+        for (int j = 1; j < REPP; j++) a = ((lane & 15) == j) ? alpha[j] : a;
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.acc[e] *= a;
+    }
+    const int slot = v4_slot(lane);
+    const float scp = sc * kV4Pre;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) {
+        const float ms = (st.m[j] == -INFINITY) ? 0.0f : st.m[j];
+        const float p = exp2f(t[j] - ms);
+        st.l[j] += p;
+        st.zp[j] = __builtin_fmaf(p, zp, st.zp[j]);
+        *lds_ptr<__attribute__((address_space(3))) uint16_t>(pbuf + (j * kWave + slot) * 2) = f2lo<F16>(p * scp);
+    }
+    asm volatile("" ::: "memory");
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t prow = pbuf + ((n & (REPP - 1)) * kWave + 4 * g) * 2;
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) {
+        const __attribute__((address_space(3))) uint2* pp = lds_ptr<__attribute__((address_space(3))) uint2>(prow + tb * 32);
+        uint2 pb;
+        pb.x = pp->x; pb.y = pp->y;
+        uint32_t ev[4], od[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) { ev[i] = vq[tb][i] & 0x0f0f0f0fu; od[i] = vq[tb][i] & 0xf0f0f0f0u; }
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            // byte e/2 of the even / odd words of two tokens -> two zero-extended 16-bit fields
+            const uint32_t by = static_cast<uint32_t>(e >> 1);
+            const uint32_t sel = 0x0c000c00u | ((4u + by) << 16) | by;
+            const uint32_t (&src)[4] = (e & 1) ? od : ev;
+            uint2 va;
+            va.x = __builtin_amdgcn_perm(src[1], src[0], sel);
+            va.y = __builtin_amdgcn_perm(src[3], src[2], sel);
+            st.acc[e] = mfma16<F16>(va, pb, st.acc[e]);
+        }
+    }
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// After the last 4-bit tile: accumulators back to real units, plus the zero-point term (the same
+// for all 128 dims of a head).
+template <int REPP>
+__device__ __forceinline__ void finish_v4(AttnState<REPP>& st, int lane) {
+    float z = 0.0f;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) {
+        const float zj = wave_sum(st.zp[j]);
+        z = ((lane & 15) == j) ? zj : z;
+        st.zp[j] = 0.0f;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const float k = (e & 1) ? kV4PostOdd : kV4PostEven;
+#pragma unroll
+        for (int i = 0; i < 4; i++) st.acc[e][i] = __builtin_fmaf(st.acc[e][i], k, z);
+    }
+}
+
 // Hot-loop loads go through buffer resources: the address is a wave-uniform
 // base held in scalar registers plus one fixed 32-bit lane offset plus a scalar
 // offset that carries the loop position, so no per-lane 64-bit pointer has to
@@ -152,7 +254,28 @@ __device__ __forceinline__ void load_v_tile(uint4 (&vv)[4][4], __amdgpu_buffer_r
             vv[tb][i] = buf_load16(rv, voff, tile_off + static_cast<uint32_t>((16 * tb + i) * kHeadDim * 2));
 }
 
-template <typename T, int TB, int REPP>
+// 4-bit value words of the 64-token tile at byte offset `tile_off` of the (batch, KV head) plane
+// of value codes (64 bytes per token): voff = g*64 + n*4.
+__device__ __forceinline__ void load_v4_tile(uint32_t (&vq)[4][4], __amdgpu_buffer_rsrc_t rv, uint32_t voff, uint32_t tile_off) {
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            vq[tb][i] = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b32(
+                rv, static_cast<int>(voff), static_cast<int>(tile_off + static_cast<uint32_t>((16 * tb + 4 * i) * 64)), kAuxStream));
+}
+
+template <bool V4> struct VTile { uint4 r[4][4]; };         // one 64-token tile of V operands, per lane
+template <> struct VTile<true> { uint32_t r[4][4]; };
+
+struct V4Args {
+    const uint32_t* codes;     // [B,Nk,capacity,16]
+    const uint16_t* scale;     // [B,Nk,capacity]
+    const uint16_t* zero;      // [B,Nk,capacity]
+    int64_t capacity;          // tokens per (batch, KV head) plane
+};
+
+template <typename T, int TB, int REPP, bool V4>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(1, 2)))
 void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                  const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
@@ -162,7 +285,10 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                  const int32_t* __restrict__ n_resid_per_seq,
                  const uint16_t* __restrict__ v, int64_t v_capacity,
                  const uint8_t* __restrict__ mask, int64_t mask_stride,
-                 float scale_log2, int N, int Nk, int rep, int n_splits, int min_gps, float* __restrict__ ws) {
+                 float scale_log2, int N, int Nk, int rep, int n_splits, int min_gps, float* __restrict__ ws,
+                 V4Args v4) {
+    // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
+    // residual window, row 0 = first residual token; otherwise `v` holds every row.
     using L = Lut<TB, REPP>;
     // the table region doubles as the fp32 query buffer of the residual block
     constexpr int kLutBytes = L::BYTES > REPP * kHeadDim * 4 ? L::BYTES : REPP * kHeadDim * 4;
@@ -185,7 +311,13 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
     int nres = n_resid_per_seq ? n_resid_per_seq[b] : n_resid;
     nres = nres < 0 ? 0 : (nres > resid_capacity ? resid_capacity : nres);
     int64_t n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
-    n_tokens = n_tokens > v_capacity ? v_capacity : n_tokens;   // never read past the (batch, head) plane of V
+    if (V4) {
+        nb = static_cast<int64_t>(nb) * kGroup > v4.capacity ? static_cast<int>(v4.capacity / kGroup) : nb;
+        nres = nres > v_capacity ? static_cast<int>(v_capacity) : nres;
+        n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
+    } else {
+        n_tokens = n_tokens > v_capacity ? v_capacity : n_tokens;   // never read past the (batch, head) plane of V
+    }
 
     // slices past the end of a short sequence have nothing to do: mark their partials empty and leave
     {
@@ -200,7 +332,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 
     const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
-                                                static_cast<uint32_t>(n_tokens * (kHeadDim * 2)));
+                                                static_cast<uint32_t>((V4 ? nres : n_tokens) * (kHeadDim * 2)));
     const uint32_t voff_v = static_cast<uint32_t>(lane >> 4) * (4 * kHeadDim * 2) + static_cast<uint32_t>(lane & 15) * 16;
     const bool has_mask = mask != nullptr;
     const __amdgpu_buffer_rsrc_t rm = make_rsrc(has_mask ? mask + static_cast<size_t>(b) * mask_stride : nullptr,
@@ -208,7 +340,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 
     AttnState<REPP> st;
 #pragma unroll
-    for (int j = 0; j < REPP; j++) { st.m[j] = -INFINITY; st.l[j] = 0.0f; }
+    for (int j = 0; j < REPP; j++) { st.m[j] = -INFINITY; st.l[j] = 0.0f; st.zp[j] = 0.0f; }
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -242,8 +374,25 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             const uint16_t* ptm = tmn + plane * kPairs + lane;
             uint16_t mrs = prs[g0 * kPairs], mrm = prm[g0 * kPairs], mts = pts[g0 * kPairs], mtm = ptm[g0 * kPairs];
             // V operands are double-buffered by tile parity: tile t+1 is requested before tile t is scored
-            uint4 vv[2][4][4];
-            load_v_tile(vv[0], rv, voff_v, static_cast<uint32_t>(2 * g0) * kWave * (kHeadDim * 2));
+            VTile<V4> vv[2];
+            const size_t vplane = static_cast<size_t>(bh) * static_cast<size_t>(V4 ? v4.capacity : 0);
+            const __amdgpu_buffer_rsrc_t rq = make_rsrc(V4 ? v4.codes + vplane * 16 : nullptr,
+                                                        V4 ? static_cast<uint32_t>(nb) * (kGroup * 64) : 0u);
+            const __amdgpu_buffer_rsrc_t rvs = make_rsrc(V4 ? v4.scale + vplane : nullptr, V4 ? static_cast<uint32_t>(nb) * (kGroup * 2) : 0u);
+            const __amdgpu_buffer_rsrc_t rvz = make_rsrc(V4 ? v4.zero + vplane : nullptr, V4 ? static_cast<uint32_t>(nb) * (kGroup * 2) : 0u);
+            const uint32_t voff_q = static_cast<uint32_t>(lane >> 4) * 64 + static_cast<uint32_t>(lane & 15) * 4;
+            uint16_t vsz[2][2] = {{0, 0}, {0, 0}};             // (scale, zero-point) words of this lane's token, by tile parity
+            auto load_values = [&](int buf, uint32_t tile_tok, bool in_range) {
+                if constexpr (V4) {
+                    load_v4_tile(vv[buf].r, rq, voff_q, in_range ? tile_tok * 64u : 0xFFFFFF00u);
+                    const int so = in_range ? static_cast<int>(tile_tok * 2u) : static_cast<int>(0x7FFFFF00);
+                    vsz[buf][0] = __builtin_amdgcn_raw_buffer_load_b16(rvs, lane * 2, so, 0);
+                    vsz[buf][1] = __builtin_amdgcn_raw_buffer_load_b16(rvz, lane * 2, so, 0);
+                } else {
+                    load_v_tile(vv[buf].r, rv, voff_v, in_range ? tile_tok * (kHeadDim * 2) : 0xFFFFFF00u);
+                }
+            };
+            load_values(0, static_cast<uint32_t>(2 * g0) * kWave, true);
             for (int grp = g0; grp < g1; grp++) {
                 asm volatile("" ::: "memory");
                 const float cdv = build_lut<T, TB, REPP>(lut, lane, qx, qy, mrs, mrm, mts, mtm);
@@ -259,7 +408,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     const int tt = 2 * grp + half;
                     const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
                     // past the last tile of this slice the loads run off the buffer's end and return zeros
-                    load_v_tile(vv[half ^ 1], rv, voff_v, (half == 0 || grp + 1 < g1) ? (tok0 + kWave) * (kHeadDim * 2) : 0xFFFFFF00u);
+                    load_values(half ^ 1, tok0 + kWave, half == 0 || grp + 1 < g1);
                     uint32_t cw[16];
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
@@ -277,9 +426,14 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     const bool keep = has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(tok0), 0) != 0) : true;
 #pragma unroll
                     for (int j = 0; j < REPP; j++) s[j] = keep ? s[j] * scale_log2 : -INFINITY;
-                    softmax_pv_tile<T, REPP>(st, s, vv[half], pbuf, lane);
+                    if constexpr (V4) {
+                        softmax_pv_tile_v4<REPP>(st, s, vv[half].r, lo2f<T>(vsz[half][0]), lo2f<T>(vsz[half][1]), pbuf, lane);
+                    } else {
+                        softmax_pv_tile<T, REPP>(st, s, vv[half].r, pbuf, lane);
+                    }
                 }
             }
+            if constexpr (V4) finish_v4<REPP>(st, lane);
         }
     }
     // the residual keys go to the block that holds the last quantized group of the sequence
@@ -308,7 +462,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             const bool valid = tok < nres;
             const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
             uint4 vv[4][4];
-            load_v_tile(vv, rv, voff_v, arow * (kHeadDim * 2));
+            load_v_tile(vv, rv, voff_v, (V4 ? static_cast<uint32_t>(tt * kWave) : arow) * (kHeadDim * 2));
             float s[REPP];
 #pragma unroll
             for (int j = 0; j < REPP; j++) s[j] = 0.0f;
@@ -417,13 +571,20 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     const int rep = a.N / a.Nk;
     dim3 grid(static_cast<unsigned>(a.n_splits) * static_cast<unsigned>(a.B * a.Nk)), block(kWave);
     const float scale_log2 = a.sm_scale * kLog2e;
-#define PQ_LAUNCH(REPP)                                                                                              \
-    hipLaunchKernelGGL((attn_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,                \
+    V4Args v4{static_cast<const uint32_t*>(a.v4_codes), static_cast<const uint16_t*>(a.v4_scale),
+              static_cast<const uint16_t*>(a.v4_zero), a.v4_capacity};
+#define PQ_LAUNCH_V(REPP, V4)                                                                                        \
+    hipLaunchKernelGGL((attn_kernel<T, TB, REPP, V4>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,            \
                        (const uint16_t*)a.rscale, (const uint16_t*)a.rmn, (const uint16_t*)a.tscale,                 \
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.N, a.Nk, rep,        \
-                       a.n_splits, a.min_groups_per_split, a.workspace)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4)
+#define PQ_LAUNCH(REPP)                                                                                              \
+    do {                                                                                                             \
+        if (a.v4_codes) PQ_LAUNCH_V(REPP, true);                                                                     \
+        else PQ_LAUNCH_V(REPP, false);                                                                               \
+    } while (0)
     switch (rep_pad(rep)) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;
@@ -431,6 +592,7 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
         default: PQ_LAUNCH(8); break;
     }
 #undef PQ_LAUNCH
+#undef PQ_LAUNCH_V
     return static_cast<int>(hipGetLastError());
 }
 

@@ -236,4 +236,98 @@ int pq_decode_attn(const void* q,
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
 
+// ---- 4-bit values (Mixed variant) ------------------------------------------------------------
+int pq_validate_quantize_values(const void* v, const int64_t* v_strides, int dtype, int B, int Nk, int T,
+                                const int32_t* codes, const void* scale, const void* zero,
+                                int64_t out_token_capacity, int64_t out_token_offset) {
+    if (!v || !v_strides || !codes || !scale || !zero) return PQ_ERR_NULL_POINTER;
+    if (B <= 0 || Nk <= 0 || T <= 0 || static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (v_strides[3] != 1) return PQ_ERR_BAD_STRIDE;
+    for (int i = 0; i < 3; i++)
+        if (v_strides[i] < 0) return PQ_ERR_BAD_STRIDE;
+    if (v_strides[2] < PQ_HEAD_DIM) return PQ_ERR_BAD_STRIDE;
+    if (out_token_offset < 0 || out_token_capacity < out_token_offset + T) return PQ_ERR_BAD_STRIDE;
+    // rows are read as 16-byte pieces
+    if (!aligned(v, 16) || v_strides[0] % 8 || v_strides[1] % 8 || v_strides[2] % 8) return PQ_ERR_MISALIGNED;
+    if (!aligned(codes, 4) || !aligned(scale, 2) || !aligned(zero, 2)) return PQ_ERR_MISALIGNED;
+    return PQ_OK;
+}
+
+int pq_quantize_values(const void* v, const int64_t* v_strides, int dtype, int B, int Nk, int T,
+                       int32_t* codes, void* scale, void* zero,
+                       int64_t out_token_capacity, int64_t out_token_offset, void* stream) {
+    if (int rc = pq_validate_quantize_values(v, v_strides, dtype, B, Nk, T, codes, scale, zero, out_token_capacity,
+                                             out_token_offset))
+        return rc;
+    const int err = pq::launch_quantize_values(v, v_strides, dtype, B, Nk, T, codes, scale, zero, out_token_capacity,
+                                               out_token_offset, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+int pq_validate_decode_attn_v4(const void* q,
+                               const uint8_t* codes, const void* rscale, const void* rmn,
+                               const void* tscale, const void* tmn, int group_capacity,
+                               int n_groups, const int32_t* n_groups_per_seq,
+                               const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                               const void* v_resid,
+                               const int32_t* v_codes, const void* v_scale, const void* v_zero, int64_t v4_capacity,
+                               const uint8_t* mask, int64_t mask_stride,
+                               float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                               int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
+                               const void* out) {
+    // the residual window of values has the same capacity and fill as that of the keys
+    const bool any_resid = n_resid_per_seq ? resid_capacity > 0 : n_resid > 0;
+    if (any_resid && !v_resid) return PQ_ERR_NULL_POINTER;
+    const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
+    if (any_groups && (!v_codes || !v_scale || !v_zero)) return PQ_ERR_NULL_POINTER;
+    if (v4_capacity < 0) return PQ_ERR_BAD_STRIDE;
+    if (!n_groups_per_seq && static_cast<int64_t>(n_groups) * PQ_GROUP > v4_capacity) return PQ_ERR_BAD_STRIDE;
+    if ((v_codes && !aligned(v_codes, 4)) || (v_resid && !aligned(v_resid, 16))) return PQ_ERR_MISALIGNED;
+    // everything else as in the fp16-value entry point; its V-capacity rule is met by construction here
+    static const char dummy_v[16] __attribute__((aligned(16))) = {0};
+    const int64_t vcap = static_cast<int64_t>(group_capacity > n_groups ? group_capacity : n_groups) * PQ_GROUP + resid_capacity + 1;
+    return pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+                                   k_resid, resid_capacity, n_resid, n_resid_per_seq, dummy_v, vcap, mask, mask_stride,
+                                   sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
+                                   workspace_bytes, out);
+}
+
+int pq_decode_attn_v4(const void* q,
+                      const uint8_t* codes, const void* rscale, const void* rmn,
+                      const void* tscale, const void* tmn, int group_capacity,
+                      int n_groups, const int32_t* n_groups_per_seq,
+                      const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                      const void* v_resid,
+                      const int32_t* v_codes, const void* v_scale, const void* v_zero, int64_t v4_capacity,
+                      const uint8_t* mask, int64_t mask_stride,
+                      float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                      int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
+                      void* out, void* stream) {
+    if (int rc = pq_validate_decode_attn_v4(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups,
+                                            n_groups_per_seq, k_resid, resid_capacity, n_resid, n_resid_per_seq,
+                                            v_resid, v_codes, v_scale, v_zero, v4_capacity, mask, mask_stride, sm_scale,
+                                            B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
+                                            workspace_bytes, out))
+        return rc;
+    const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
+    pq::AttnArgs a;
+    a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
+    a.group_capacity = group_capacity; a.n_groups = n_groups; a.n_groups_per_seq = n_groups_per_seq;
+    a.k_resid = k_resid; a.resid_capacity = resid_capacity; a.n_resid = n_resid; a.n_resid_per_seq = n_resid_per_seq;
+    a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
+    a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
+    a.min_groups_per_split = min_groups_per_split;
+    a.workspace = static_cast<float*>(workspace); a.out = nullptr;
+    if (any_groups) {
+        a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token
+        a.v4_codes = v_codes; a.v4_scale = v_scale; a.v4_zero = v_zero; a.v4_capacity = v4_capacity;
+    } else {
+        a.v = v_resid; a.v_capacity = resid_capacity;      // nothing quantized yet: the plain kernel over the window
+    }
+    const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
+    if (err != 0) return PQ_ERR_LAUNCH;
+    return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
+}
+
 }  // extern "C"

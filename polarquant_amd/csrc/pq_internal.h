@@ -16,6 +16,9 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
 
 int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st);
 
+int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int B, int Nk, int T,
+                           int32_t* codes, void* scale, void* mn, int64_t cap, int64_t off, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;
@@ -27,6 +30,9 @@ struct AttnArgs {
     const int32_t* n_resid_per_seq;
     const void* v;
     int64_t v_capacity;
+    // 4-bit values (Mixed variant): when v4_codes is set, `v` holds only the residual window's rows
+    const void *v4_codes = nullptr, *v4_scale = nullptr, *v4_zero = nullptr;
+    int64_t v4_capacity = 0;
     const uint8_t* mask;
     int64_t mask_stride;
     float sm_scale;

@@ -1,0 +1,78 @@
+// 4-bit value quantizer of the Mixed variant: values [B,Nk,T,128] are quantized
+// per token and head along the 128 dims (one min/max group per row), 8 codes to
+// an int32, element i in bits [4i, 4i+4).  HIP counterpart of the
+// triton_quantize_and_pack_along_last_dim(values, 128, 4) calls at
+// models/modeling_llama_polar.py:236 and :275 (the routine itself belongs to a
+// kivi_quant package that is not in the reference tree; its published form is
+// followed: scale = (max - min) / 15, q = round_half_even(clamp((x - min) / scale, 0, 15)),
+// every op rounded to the value dtype as eager torch does).
+//
+// 16 lanes own one row: each loads 16 bytes (dims 8n..8n+7) and writes the row's
+// n-th code word, so a wavefront reads four whole 256-byte rows and writes 256
+// contiguous bytes of codes.
+#include "pq_device.h"
+#include "pq_internal.h"
+
+namespace pq {
+
+template <typename T>
+__device__ __forceinline__ float rnd_v(float f) { return lo2f<T>(f2lo<T>(f)); }
+
+constexpr int kVThreads = 256;
+constexpr int kRowsPerBlock = kVThreads / 16;
+
+template <typename T>
+__global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t st, int Nk, int n_tok,
+    int32_t* __restrict__ codes, uint16_t* __restrict__ scale, uint16_t* __restrict__ mn, int64_t cap, int64_t off) {
+    const int n = threadIdx.x & 15;
+    const int t = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 4);
+    const int bh = blockIdx.y;
+    const bool live = t < n_tok;                       // whole 16-lane row groups are live or not
+    const int b = bh / Nk, h = bh - b * Nk;
+    float x[8];
+    float lo = INFINITY, hi = -INFINITY;
+    if (live) {
+        const uint4 w = *reinterpret_cast<const uint4*>(v + b * sb + h * sh + static_cast<int64_t>(t) * st + 8 * n);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[2 * i] = lo2f<T>(static_cast<uint16_t>(ww[i] & 0xffffu));
+            x[2 * i + 1] = lo2f<T>(static_cast<uint16_t>(ww[i] >> 16));
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
+    }
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+        lo = fminf(lo, __shfl_xor(lo, o));
+        hi = fmaxf(hi, __shfl_xor(hi, o));
+    }
+    if (!live) return;
+    const float sc = rnd_v<T>(rnd_v<T>(hi - lo) / 15.0f);
+    uint32_t word = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        float q = rnd_v<T>(rnd_v<T>(x[i] - lo) / sc);
+        q = fminf(fmaxf(q, 0.0f), 15.0f);          // NaN (0/0 on a constant row) comes out of fmaxf as 0
+        q = __builtin_rintf(q);                    // round half to even
+        word |= static_cast<uint32_t>(q) << (4 * i);
+    }
+    const int64_t row = static_cast<int64_t>(bh) * cap + off + t;
+    codes[row * 16 + n] = static_cast<int32_t>(word);
+    if (n == 0) { scale[row] = f2lo<T>(sc); mn[row] = f2lo<T>(lo); }
+}
+
+int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int B, int Nk, int T,
+                           int32_t* codes, void* scale, void* mn, int64_t cap, int64_t off, hipStream_t st) {
+    dim3 grid((T + kRowsPerBlock - 1) / kRowsPerBlock, B * Nk), block(kVThreads);
+    if (dtype == 0)
+        hipLaunchKernelGGL(quantize_values_kernel<F16>, grid, block, 0, st, (const uint16_t*)v, strides[0], strides[1],
+                           strides[2], Nk, T, codes, (uint16_t*)scale, (uint16_t*)mn, cap, off);
+    else
+        hipLaunchKernelGGL(quantize_values_kernel<BF16>, grid, block, 0, st, (const uint16_t*)v, strides[0], strides[1],
+                           strides[2], Nk, T, codes, (uint16_t*)scale, (uint16_t*)mn, cap, off);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace pq

@@ -1,0 +1,132 @@
+"""4-bit values of the Mixed variant on the GPU against the CPU oracle: the value quantizer is
+bit-exact (codes, scale, zero-point), the fused decode attention over polar keys + 4-bit values
+meets the output bar against the literal restatement and the fp64 evaluation."""
+import pytest
+import torch
+
+from oracle import polar_oracle as po
+from polarquant_amd import workloads as wl
+from polarquant_amd.attention import polar_decode_attention_v4
+from polarquant_amd.values import quantize_values
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 1e-3
+
+
+def _same_bits(a, b):
+    a, b = a.cpu(), b.cpu()
+    if a.dtype != torch.int32:
+        a, b = a.view(torch.int16), b.view(torch.int16)
+    return int((a != b).sum())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 17, 128, 1000])
+def test_value_quantizer_bit_exact(gpu, dtype, T):
+    print("case values", dtype, T, flush=True)
+    g = torch.Generator().manual_seed(31 + T)
+    v = wl.make_half((2, 3, T, 128), g, dtype)
+    v[0, 0, 0] = 0.75                               # constant row: 0/0 -> code 0
+    if T > 2:
+        v[1, 2, 2] *= 1e-3                          # tiny range
+        v[1, 1, 1, ::2] = 100.0                     # two-valued row
+    ref = po.quantize_values_along_last_dim(v)
+    got = quantize_values(v.to(gpu))
+    torch.cuda.synchronize()
+    assert [tuple(t.shape) for t in got] == [tuple(t.shape) for t in ref]
+    flips = [_same_bits(a, b) for a, b in zip(got, ref)]
+    print("value flips (codes words, scale, mn)", flips, flush=True)
+    assert flips == [0, 0, 0]
+
+
+def test_value_quantizer_strided_input_and_cache_slot(gpu):
+    g = torch.Generator().manual_seed(5)
+    v = wl.make_half((2, 256, 4, 128), g)            # [B, T, Nk, 128] as the projection leaves it
+    vt = v.to(gpu).transpose(1, 2)                   # [B, Nk, T, 128] view, token stride Nk*128
+    ref = po.quantize_values_along_last_dim(v.transpose(1, 2).contiguous())
+    cap = 512
+    out = (torch.full((2, 4, cap, 16), -1, dtype=torch.int32, device=gpu),
+           torch.zeros(2, 4, cap, 1, dtype=torch.float16, device=gpu), torch.zeros(2, 4, cap, 1, dtype=torch.float16, device=gpu))
+    got = quantize_values(vt, out=out, token_offset=128)
+    assert all(_same_bits(a, b) == 0 for a, b in zip(got, ref))
+    assert bool((out[0][:, :, :128] == -1).all()) and bool((out[0][:, :, 384:] == -1).all())
+
+
+def _close(got, ref, rtol=RTOL, atol=ATOL):
+    got, ref = got.double(), ref.double()
+    err = (got - ref).abs()
+    return int((err > atol + rtol * ref.abs()).sum()), float(err.max())
+
+
+def _case(gpu, B, N, Nk, n_groups, n_resid, rbits, tbits, dtype, mask_pad=0, seed=0, n_splits=None, caps=(0, 0), ragged=None):
+    g = torch.Generator().manual_seed(seed)
+    Lq = n_groups * 128
+    L = Lq + n_resid
+    k = wl.make_keys(B, Nk, L, 5e5, g, dtype)
+    q = wl.make_half((B, N, 1, 128), g, dtype)
+    v = wl.make_half((B, Nk, L, 128), g, dtype)
+    v[..., 5] += 2.0                                 # a channel with an offset: exercises the zero-point term
+    quant, vq = (None,) * 5, (None,) * 3
+    if n_groups:
+        quant = po.quantize_and_pack_nbit(k[:, :, :Lq].contiguous(), rbits, tbits)
+        vq = po.quantize_values_along_last_dim(v[:, :, :Lq].contiguous())
+    kres, vres = k[:, :, Lq:].contiguous(), v[:, :, Lq:].contiguous()
+    mask = None
+    if mask_pad:
+        mask = torch.ones(B, L, dtype=torch.int64)
+        for b in range(B):
+            mask[b, :(mask_pad * (b + 1)) % L] = 0
+    ref = po.decode_attention_mixed(q, kres, *quant, vres, *vq, mask, rbits, tbits)
+    ref64 = po.decode_attention_mixed_exact(q, kres, *quant, vres, *vq, mask, rbits, tbits)
+    gc, rc = caps
+    dq, dvq = [None] * 5, [None] * 3
+    if n_groups:
+        cap = n_groups + gc
+        dq = [torch.zeros((B, Nk, cap) + tuple(t.shape[3:]), dtype=t.dtype, device=gpu) for t in quant]
+        for d, t in zip(dq, quant):
+            d[:, :, :n_groups] = t.to(gpu)
+        dvq = [torch.full((B, Nk, cap * 128, t.shape[3]), -1 if t.dtype == torch.int32 else float("nan"), dtype=t.dtype, device=gpu)
+               for t in vq]
+        for d, t in zip(dvq, vq):
+            d[:, :, :Lq] = t.to(gpu)
+    dk = torch.zeros(B, Nk, 128 + rc, 128, dtype=dtype, device=gpu)
+    dv = torch.full((B, Nk, 128 + rc, 128), float("nan"), dtype=dtype, device=gpu)   # rows past the fill must not contribute
+    dk[:, :, :n_resid], dv[:, :, :n_resid] = kres.to(gpu), vres.to(gpu)
+    out = polar_decode_attention_v4(q.to(gpu), *dq, dk, dv, *dvq, n_groups, n_resid,
+                                    attention_mask=None if mask is None else mask.to(gpu),
+                                    rbits=rbits, tbits=tbits, n_splits=n_splits)
+    torch.cuda.synchronize()
+    out = out.cpu()
+    assert out.shape == (B, N, 1, 128) and out.dtype == dtype and torch.isfinite(out.float()).all()
+    return out, ref, ref64
+
+
+@pytest.mark.parametrize("N,Nk", [(8, 2), (4, 4), (7, 1), (2, 1)])
+@pytest.mark.parametrize("n_groups,n_resid", [(3, 1), (1, 128), (8, 77), (0, 5)])
+def test_attention_v4_matches_oracle(gpu, N, Nk, n_groups, n_resid):
+    print("case v4", N, Nk, n_groups, n_resid, flush=True)
+    out, ref, ref64 = _case(gpu, 2, N, Nk, n_groups, n_resid, 4, 4, torch.float16, seed=n_groups * 131 + n_resid)
+    for r in (ref, ref64):
+        nbad, emax = _close(out, r)
+        assert nbad == 0, (nbad, emax)
+
+
+@pytest.mark.parametrize("rbits,tbits", [(3, 3), (4, 2)])
+def test_attention_v4_other_bit_widths_mask_and_capacity(gpu, rbits, tbits):
+    out, ref, ref64 = _case(gpu, 3, 8, 2, 5, 33, rbits, tbits, torch.float16, mask_pad=150, seed=9, caps=(3, 7))
+    for r in (ref, ref64):
+        nbad, emax = _close(out, r)
+        assert nbad == 0, (nbad, emax)
+
+
+@pytest.mark.parametrize("n_splits", [1, 2, 5, 16])
+def test_attention_v4_split_counts_agree(gpu, n_splits):
+    out, ref, ref64 = _case(gpu, 1, 8, 2, 9, 2, 4, 4, torch.float16, seed=3, n_splits=n_splits)
+    nbad, emax = _close(out, ref64)
+    assert nbad == 0, (nbad, emax)
+
+
+def test_attention_v4_bf16(gpu):
+    out, ref, ref64 = _case(gpu, 2, 8, 2, 16, 3, 4, 4, torch.bfloat16, seed=4)
+    nbad, emax = _close(out, ref64, 2e-2, 4e-3)      # bf16 has 8 mantissa bits
+    assert nbad == 0, (nbad, emax)
