@@ -247,6 +247,10 @@ int pq_decode_attn_v4(const void *q,
                       int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
                       void *out, void *stream);
 
+/* Split count for pq_decode_attn_v4 (as pq_decode_attn_plan, which see; the 4-bit
+ * kernel runs two wavefronts per SIMD when N/Nk <= 4). No reference counterpart. */
+int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus);
+
 int pq_validate_decode_attn_v4(const void *q,
                                const uint8_t *codes, const void *rscale, const void *rmn,
                                const void *tscale, const void *tmn, int group_capacity,

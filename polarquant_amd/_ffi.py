@@ -57,6 +57,7 @@ SIGNATURES = {
                                                             c_void_p, c_int64, c_float]
                                    + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),
+    "pq_decode_attn_v4_plan": (c_int, [c_int] * 5),
     "pq_decode_attn_workspace_bytes": (c_size_t, [c_int] * 3),
 }
 

@@ -163,7 +163,7 @@ def polar_decode_attention_v4(
         sm_scale = 1.0 / math.sqrt(hd)
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
     if n_splits is None:
-        n_splits = plan_splits(B, Nk, max_groups, dev)
+        n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, N, Nk, max(max_groups, 1), _num_cus(dev))
     ws = workspace_for(B, N, n_splits, dev)
     if out is None:
         out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)

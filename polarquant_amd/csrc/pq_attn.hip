@@ -276,7 +276,7 @@ struct V4Args {
 };
 
 template <typename T, int TB, int REPP, bool V4>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(1, 2)))
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
 void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                  const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
                  const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,

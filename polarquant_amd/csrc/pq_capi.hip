@@ -237,6 +237,20 @@ int pq_decode_attn(const void* q,
 }
 
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
+int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
+    if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;
+    if (n_cus <= 0) n_cus = 256;
+    // with 4-bit values the kernel holds 32 instead of 128 registers of value operands and runs
+    // two wavefronts per SIMD (for up to 4 query heads per KV head): twice the slots
+    const int rep = N / Nk;
+    const long long slots = static_cast<long long>(n_cus) * (pq::rep_pad(rep) <= 4 ? 8 : 4);
+    long long n = slots / (static_cast<long long>(B) * Nk);
+    if (n < 1) n = 1;
+    if (n > max_groups) n = max_groups;
+    if (n > 65534) n = 65534;
+    return static_cast<int>(n);
+}
+
 int pq_validate_quantize_values(const void* v, const int64_t* v_strides, int dtype, int B, int Nk, int T,
                                 const int32_t* codes, const void* scale, const void* zero,
                                 int64_t out_token_capacity, int64_t out_token_offset) {

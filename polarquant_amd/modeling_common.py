@@ -30,8 +30,9 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .attention import polar_decode_attention
+from .attention import polar_decode_attention, polar_decode_attention_v4
 from .quantize import quantize_and_pack_nbit
+from .values import quantize_values
 
 GROUP = 128
 
@@ -311,6 +312,139 @@ class PolarGroupAttention(nn.Module):
     def quantize_and_pack_nbit(self, key_states):
         """(reference :135-157) -> (indices, rscale, rmn, tscale, tmn)."""
         return quantize_and_pack_nbit(key_states, self.rbits, self.tbits, self.group_size)
+
+
+# ----------------------------------------------------------------------------- Mixed variant: polar keys + 4-bit values
+class _MixedArena(_Arena):
+    """Per-layer cache of the Mixed variant: polar key groups, 4-bit value rows for the same tokens,
+    and a shared 128-token residual window of half-precision keys and values."""
+
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits):
+        self.vres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
+        super().__init__(B, Nk, dtype, device, capacity_tokens, rbits, tbits)
+
+    def _alloc(self, cap_tokens):
+        gcap = (cap_tokens + GROUP - 1) // GROUP
+        B, Nk, dev, dt = self.B, self.Nk, self.device, self.dtype
+        codes = torch.empty(B, Nk, gcap, GROUP, 64, dtype=torch.uint8, device=dev)
+        meta = [torch.empty(B, Nk, gcap, 1, 64, dtype=dt, device=dev) for _ in range(4)]
+        vcodes = torch.empty(B, Nk, gcap * GROUP, 16, dtype=torch.int32, device=dev)
+        vmeta = [torch.empty(B, Nk, gcap * GROUP, 1, dtype=dt, device=dev) for _ in range(2)]
+        if self.n_groups:
+            g, t = self.n_groups, self.n_groups * GROUP
+            codes[:, :, :g] = self.codes[:, :, :g]
+            for new, old in zip(meta, self.meta):
+                new[:, :, :g] = old[:, :, :g]
+            vcodes[:, :, :t] = self.vcodes[:, :, :t]
+            for new, old in zip(vmeta, self.vmeta):
+                new[:, :, :t] = old[:, :, :t]
+        self.codes, self.meta, self.vcodes, self.vmeta, self.gcap = codes, meta, vcodes, vmeta, gcap
+        self.v, self.vcap = None, gcap * GROUP + GROUP
+
+    def flush(self):
+        """The window holds 128 keys and values: both go to the quantized store together (reference :207-217, :243-250)."""
+        quantize_values(self.vres, out=(self.vcodes, *self.vmeta), token_offset=self.n_groups * GROUP)
+        self.quantize_into(self.kres)
+        self.n_resid = 0
+
+    def as_tuple(self) -> "PolarCache":
+        r, g = self.n_resid, self.n_groups
+        kf = self.kres[:, :, :r] if r else None
+        vf = self.vres[:, :, :r] if r else None
+        if g:
+            q5 = [self.codes[:, :, :g]] + [m[:, :, :g] for m in self.meta]
+            v3 = [self.vcodes[:, :, :g * GROUP]] + [m[:, :, :g * GROUP] for m in self.vmeta]
+        else:
+            q5, v3 = [None] * 5, [None] * 3
+        return PolarCache((kf, *q5, vf, *v3, self.kv_len), self)
+
+
+class PolarMixedGroupAttention(PolarGroupAttention):
+    """Polar keys + 4-bit values, the reference's LlamaPolarMixedGroupAttention
+    (models/modeling_llama_polar.py:160-292): same forward signature, 11-slot cache tuple
+    (key_states_full, indices, rscale, rmn, tscale, tmn, value_states_full, value_states_quant,
+    value_scale, value_mn, kv_seq_len)."""
+
+    def __init__(self, config, layer_idx: Optional[int] = None):
+        super().__init__(config, layer_idx)
+        self.vbits = 4                                                     # :163
+
+    def _new_arena(self, B, dtype, device, tokens):
+        cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
+        return _MixedArena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits)
+
+    def _arena_of(self, past_key_value, dtype, device) -> _MixedArena:
+        arena = getattr(past_key_value, "arena", None)
+        if arena is not None and arena.kv_len == past_key_value[-1]:
+            return arena
+        # a plain 11-tuple in the reference's format: copy it into a fresh arena
+        kf, ind, rs, rm, ts, tm, vf, vc, vs, vm, n = past_key_value
+        B = (kf if kf is not None else ind).shape[0]
+        arena = self._new_arena(B, dtype, device, n + 1)
+        if ind is not None:
+            g = ind.shape[2]
+            arena.codes[:, :, :g] = ind
+            for dst, src in zip(arena.meta, (rs, rm, ts, tm)):
+                dst[:, :, :g] = src
+            arena.vcodes[:, :, :g * GROUP] = vc
+            for dst, src in zip(arena.vmeta, (vs, vm)):
+                dst[:, :, :g * GROUP] = src
+            arena.n_groups = g
+        if kf is not None:
+            arena.kres[:, :, :kf.shape[2]] = kf
+            arena.vres[:, :, :kf.shape[2]] = vf
+            arena.n_resid = kf.shape[2]
+        arena.kv_len = n
+        return arena
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_value=None, position_embeddings: Tuple[torch.Tensor, torch.Tensor] = None, **kwargs):
+        bsz, q_len, _ = hidden_states.size()
+        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = position_embeddings
+        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        if self.capture is not None:
+            self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
+
+        if q_len == 1:   # decoding time (:185-257)
+            arena = self._arena_of(past_key_value, query_states.dtype, query_states.device)
+            arena.reserve(arena.kv_len + 1)
+            arena.kres[:, :, arena.n_resid] = key_states[:, :, 0]          # :201
+            arena.vres[:, :, arena.n_resid] = value_states[:, :, 0]        # :223
+            arena.n_resid += 1
+            arena.kv_len += 1
+            g = arena.n_groups
+            attn_output = polar_decode_attention_v4(
+                query_states, arena.codes if g else None, *(arena.meta if g else [None] * 4), arena.kres, arena.vres,
+                arena.vcodes if g else None, *(arena.vmeta if g else [None] * 2), g, arena.n_resid,
+                attention_mask=_mask_u8(attention_mask), rbits=self.rbits, tbits=self.tbits,
+                sm_scale=1.0 / math.sqrt(self.head_dim))                   # :189-241
+            if arena.n_resid % self.residual_length == 0:                  # :207, :243
+                arena.flush()
+            past_key_value = arena.as_tuple()                              # :257
+        else:            # pre-filling (:258-281)
+            assert past_key_value is None
+            kv_seq_len = key_states.shape[2]
+            attn_output = _prefill_attention(query_states, key_states, value_states, attention_mask,
+                                             self.num_key_value_groups, self.is_causal)
+            arena = self._new_arena(bsz, key_states.dtype, key_states.device, kv_seq_len + 1)
+            residual_length = kv_seq_len % self.residual_length
+            n_quant = kv_seq_len - residual_length if kv_seq_len >= self.residual_length else 0
+            if n_quant:
+                quantize_values(value_states[:, :, :n_quant], out=(arena.vcodes, *arena.vmeta), token_offset=0)   # :275
+                arena.quantize_into(key_states[:, :, :n_quant])            # :271
+            r = kv_seq_len - n_quant
+            if r:
+                arena.kres[:, :, :r] = key_states[:, :, n_quant:]
+                arena.vres[:, :, :r] = value_states[:, :, n_quant:]
+            arena.n_resid, arena.kv_len = r, kv_seq_len
+            past_key_value = arena.as_tuple()                              # :281
+
+        attn_output = attn_output.reshape(bsz, q_len, -1).contiguous()
+        attn_output = self.o_proj(attn_output)
+        return attn_output, past_key_value
 
 
 def _prefill_attention(q, k, v, attention_mask, n_rep, is_causal):

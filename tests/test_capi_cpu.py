@@ -119,6 +119,47 @@ def test_validate_decode_attn_and_plan(lib):
     assert lib.pq_decode_attn_merge(None, 0, 1, 1, 1, 0, None, None) == -1
 
 
+def test_validate_value_quantizer_and_v4_attention(lib):
+    strides = (ctypes.c_int64 * 4)(8 * 300 * 128, 300 * 128, 128, 1)
+    sp = ctypes.cast(strides, ctypes.c_void_p)
+    ok = [P, sp, 0, 2, 8, 300, P, P, P, 512, 100]
+    assert lib.pq_validate_quantize_values(*ok) == 0
+
+    def bad(i, v):
+        a = list(ok); a[i] = v
+        return lib.pq_validate_quantize_values(*a)
+    assert bad(0, None) == -1 and bad(1, None) == -1 and bad(6, None) == -1 and bad(7, None) == -1 and bad(8, None) == -1
+    assert bad(3, 0) == -2 and bad(5, 0) == -2 and bad(2, 3) == -4
+    assert bad(9, 399) == -6 and bad(10, -1) == -6          # capacity < offset + T
+    assert bad(0, P + 8) == -5                               # rows are read as 16-byte pieces
+    st = (ctypes.c_int64 * 4)(8 * 300 * 128, 300 * 128, 132, 1)
+    a = list(ok); a[1] = ctypes.cast(st, ctypes.c_void_p)
+    assert lib.pq_validate_quantize_values(*a) == -5
+    st = (ctypes.c_int64 * 4)(300 * 8 * 128, 128, 8 * 128, 1)   # transposed [B,T,Nk,128] view
+    a = list(ok); a[1] = ctypes.cast(st, ctypes.c_void_p)
+    assert lib.pq_validate_quantize_values(*a) == 0
+
+    B, N, Nk, ns = 2, 32, 8, 4
+    wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
+    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, P, P, P, 512, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P]
+    assert lib.pq_validate_decode_attn_v4(*ok) == 0
+
+    def bad4(i, v):
+        a = list(ok); a[i] = v
+        return lib.pq_validate_decode_attn_v4(*a)
+    assert bad4(13, None) == -1                               # residual window without values
+    assert bad4(14, None) == -1 and bad4(15, None) == -1 and bad4(16, None) == -1   # groups without 4-bit values
+    assert bad4(17, 3 * 128 - 1) == -6                        # value-code capacity below the quantized tokens
+    assert bad4(0, None) == -1 and bad4(1, None) == -1 and bad4(7, 5) == -6 and bad4(27, 0) == -7
+    assert bad4(13, P + 8) == -5
+    a = list(ok); a[1:6] = [None] * 5; a[6] = 0; a[7] = 0; a[14:17] = [None] * 3; a[17] = 0
+    assert lib.pq_validate_decode_attn_v4(*a) == 0            # nothing quantized yet
+    # two wavefronts per SIMD for up to 4 query heads per KV head, one beyond
+    assert lib.pq_decode_attn_v4_plan(16, 32, 8, 256, 256) == 16
+    assert lib.pq_decode_attn_v4_plan(64, 28, 4, 64, 256) == 4
+    assert lib.pq_decode_attn_v4_plan(1, 32, 8, 3, 256) == 3
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     import torch
     from polarquant_amd.attention import polar_decode_attention

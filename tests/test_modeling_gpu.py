@@ -71,8 +71,8 @@ def _check_cache(got, ref):
         if g is not None:
             g = g.cpu()
             assert g.shape == r.shape and g.dtype == r.dtype, "tuple element %d" % j
-            if g.dtype == torch.uint8:
-                assert torch.equal(g, r), "codes differ"
+            if g.dtype in (torch.uint8, torch.int32):
+                assert torch.equal(g, r), "codes differ (tuple element %d)" % j
             else:
                 assert bool((g.float() == r.float()).all()), "tuple element %d differs" % j
 
@@ -170,3 +170,46 @@ def test_decode_with_bf16_model(gpu):
             ref_out = ref_attn.reshape(2, 1, -1).float() @ att.o_proj.weight.detach().float().cpu().T
             assert (out.float().cpu() - ref_out).abs().max().item() < 5e-2 * max(1.0, ref_out.abs().max().item())
     assert cache[1].dtype == torch.uint8 and cache[2].dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("L", [5, 200, 256])
+def test_mixed_attention_forward_matches_reference_restatement(gpu, L):
+    """LlamaPolarMixedGroupAttention (polar keys + 4-bit values): prefill, then decode across a
+    flush of the shared residual window.  Captured post-RoPE q/k/v are replayed through the oracle's
+    Mixed forward: the 11-slot cache must be bit-identical (key codes and metadata, packed value
+    words, value scale and zero-point, residual keys and values, kv_seq_len), outputs within tolerance."""
+    from polarquant_amd.modeling_llama_polar import LlamaPolarMixedGroupAttention
+    torch.manual_seed(5)
+    cfg = _tiny(8, 2)
+    att = LlamaPolarMixedGroupAttention(cfg, 0).half().to(gpu)
+    assert att.vbits == 4
+    att.capture = []
+    B, steps = 2, 140
+    mask = torch.ones(B, L, dtype=torch.int64)
+    mask[1, :min(3, L - 1)] = 0
+    x = (torch.randn(B, L + steps, cfg.hidden_size) * 0.5).half().to(gpu)
+    with torch.no_grad():
+        out, cache = att(x[:, :L], attention_mask=mask.to(gpu), past_key_value=None, position_embeddings=_rope(cfg, 0, L, torch.float16, gpu))
+    assert isinstance(cache, tuple) and len(cache) == 11 and cache[-1] == L
+    q, k, v = [t.cpu() for t in att.capture[-1]]
+    ref_cache = po.prefill_cache_mixed(k, v)
+    _check_cache(cache, ref_cache)
+    o_proj = att.o_proj.weight.detach().float().cpu()
+    for i in range(steps):
+        mask = torch.cat([mask, torch.ones(B, 1, dtype=torch.int64)], -1)
+        with torch.no_grad():
+            out, cache = att(x[:, L + i:L + i + 1], attention_mask=mask.to(gpu), past_key_value=cache,
+                             position_embeddings=_rope(cfg, L + i, 1, torch.float16, gpu))
+        q, k, v = [t.cpu() for t in att.capture[-1]]
+        ref_attn, ref_cache = po.decode_step_mixed(q, k, v, ref_cache, mask)
+        ref_out = ref_attn.reshape(B, 1, -1).float() @ o_proj.T
+        err = (out.float().cpu() - ref_out).abs().max().item()
+        assert err < 2e-2 * max(1.0, ref_out.abs().max().item()), (i, err)
+        if i in (0, 1, steps // 2, steps - 1) or (L + i + 1) % 128 in (0, 1):
+            _check_cache(cache, ref_cache)
+    # a plain 11-tuple (no arena) is accepted too
+    plain = tuple(t.clone() if torch.is_tensor(t) else t for t in cache)
+    with torch.no_grad():
+        o1, c1 = att(x[:, -1:], None, cache, _rope(cfg, L + steps, 1, torch.float16, gpu))
+        o2, c2 = att(x[:, -1:], None, plain, _rope(cfg, L + steps, 1, torch.float16, gpu))
+    assert torch.equal(o1, o2) and c1[-1] == c2[-1] == L + steps + 1

@@ -304,3 +304,102 @@ def test_decode_steps_bookkeeping_and_equivalence():
             quant = po.quantize_and_pack_nbit(k[:, :, :nq_before].contiguous()) if nq_before else (None,) * 5
             ref = po.decode_attention_exact(qs[:, :, i:i + 1], k[:, :, nq_before:t + 1], *quant, v[:, :, :t + 1])
             assert float((out.double() - ref).abs().max()) < 2e-3
+
+
+# ------------------------------------------------------------------ 4-bit values (Mixed variant)
+def test_value_quantizer_known_answer_row_and_packing():
+    """A row mn + k*s with k = dim % 16 has scale exactly s and codes exactly k; with 8 codes per
+    int32, element i in bits [4i, 4i+4), the words alternate 0x76543210 / 0xFEDCBA98."""
+    row = (-1 + 0.25 * (torch.arange(128) % 16)).to(torch.float16).reshape(1, 1, 1, 128)
+    for quant in (po.quantize_values_along_last_dim, co.quantize_values):
+        code, scale, mn = quant(row)
+        assert code.dtype == torch.int32 and code.shape == (1, 1, 1, 16) and scale.shape == (1, 1, 1, 1)
+        words = [int(w) & 0xFFFFFFFF for w in code.flatten()]
+        assert words == [0x76543210, 0xFEDCBA98] * 8
+        assert float(scale) == 0.25 and float(mn) == -1.0
+    assert torch.equal(po.unpack_values(code).flatten(), torch.arange(128) % 16)
+    assert torch.equal(po.dequantize_values(code, scale, mn).flatten(), row.float().flatten())
+
+
+def test_value_quantizer_rounds_half_to_even_after_clamp():
+    """(x - mn)/scale landing exactly on k + 0.5 goes to the even neighbour (torch.round), and the
+    clamp comes first, so nothing above 15 survives."""
+    k = torch.tensor([0.0, 0.5, 1.5, 2.5, 3.5, 13.5, 14.5, 15.0])
+    row = torch.zeros(128)
+    row[:8] = k * 0.25                      # scale = 15*0.25/15 = 0.25 exactly, mn = 0
+    row[8:] = 3.75
+    for quant in (po.quantize_values_along_last_dim, co.quantize_values):
+        code, scale, mn = quant(row.to(torch.float16).reshape(1, 1, 1, 128))
+        assert float(scale) == 0.25 and float(mn) == 0.0
+        assert po.unpack_values(code).flatten()[:8].tolist() == [0, 0, 2, 2, 4, 14, 14, 15]
+
+
+@pytest.mark.parametrize("dtype,eps", [(torch.float16, 2e-3), (torch.bfloat16, 2e-2)])
+def test_value_quantizer_invariants_and_restatements(dtype, eps):
+    g = torch.Generator().manual_seed(12)
+    v = wl.make_half((2, 3, 200, 128), g, dtype)
+    v[0, 0, 0] = 0.5                        # constant row: 0/0, defined as code 0
+    a = po.quantize_values_along_last_dim(v)
+    b = co.quantize_values(v)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1].view(torch.int16), b[1].view(torch.int16))
+    assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
+    codes = po.unpack_values(a[0])
+    assert int(codes.min()) == 0 and int(codes.max()) == 15 and bool((codes[0, 0, 0] == 0).all())
+    vf = v.float()
+    # the row minimum gets code 0, the row maximum 15 (constant row aside)
+    lo, hi = vf.argmin(-1, keepdim=True), vf.argmax(-1, keepdim=True)
+    assert bool((codes.gather(-1, lo)[1:] == 0).all()) and bool((codes.gather(-1, hi)[1:] == 15).all())
+    assert torch.equal(a[2].float(), vf.min(-1, keepdim=True)[0])
+    # reconstruction within half a step (plus the dtype's own rounding of the intermediates)
+    err = (po.dequantize_values(*a) - vf).abs()
+    assert bool((err <= a[1].float() / 2 + eps * vf.abs().amax(-1, keepdim=True)).all())
+
+
+def test_mixed_attention_literal_vs_one_shot_fp64():
+    """The literal Mixed decode step (two matmuls, half-rounded probabilities) against one fp64
+    softmax attention over [dequantized ; residual] keys and values; and with no quantized part it
+    reduces to the plain fp16 attention."""
+    g = torch.Generator().manual_seed(13)
+    B, N, Nk, nb, res = 2, 8, 2, 3, 40
+    L = nb * 128 + res
+    k = wl.make_keys(B, Nk, L, 5e5, g)
+    q, v = wl.make_half((B, N, 1, 128), g), wl.make_half((B, Nk, L, 128), g)
+    quant = po.quantize_and_pack_nbit(k[:, :, :nb * 128].contiguous())
+    vq = po.quantize_values_along_last_dim(v[:, :, :nb * 128].contiguous())
+    kres, vres = k[:, :, nb * 128:], v[:, :, nb * 128:]
+    mask = torch.ones(B, L, dtype=torch.int64)
+    mask[1, :200] = 0
+    for m in (None, mask):
+        a = po.decode_attention_mixed(q, kres, *quant, vres, *vq, m)
+        e = po.decode_attention_mixed_exact(q, kres, *quant, vres, *vq, m)
+        assert (a.double() - e).abs().max().item() < 2e-3
+        # 4-bit values are a perturbation of the fp16-value attention, of the size the step predicts
+        plain = po.decode_attention_exact(q, kres, *quant, v, m)
+        assert (e - plain).abs().max().item() < 0.5 * float(vq[1].float().max())
+    a = po.decode_attention_mixed(q, kres, None, None, None, None, None, vres, None, None, None)
+    f = po.fp16_decode_attention(q, kres, vres)
+    assert (a.float() - f.float()).abs().max().item() < 2e-3
+
+
+@pytest.mark.parametrize("L", [1, 127, 128, 129, 300, 384])
+def test_mixed_cache_bookkeeping(L):
+    """Keys and values share the residual window: after any prompt length and any number of decode
+    steps, quantized tokens = 128 * floor(kv_len / 128) on both sides (0 when the prompt was
+    shorter than 128 and no flush happened yet), and the tuple has the reference's 11 slots."""
+    g = torch.Generator().manual_seed(L)
+    k, v = wl.make_keys(1, 2, L + 140, 1e4, g), wl.make_half((1, 2, L + 140, 128), g)
+    cache = po.prefill_cache_mixed(k[:, :, :L], v[:, :, :L])
+    assert len(cache) == 11 and cache[-1] == L
+    for i in range(140):
+        q = wl.make_half((1, 4, 1, 128), g)
+        out, cache = po.decode_step_mixed(q, k[:, :, L + i:L + i + 1], v[:, :, L + i:L + i + 1], cache)
+        n = L + i + 1
+        kf, ind, vf, vc, vs, vm = cache[0], cache[1], cache[6], cache[7], cache[8], cache[9]
+        nres = 0 if kf is None else kf.shape[2]
+        assert (vf is None) == (kf is None) and (vf is None or vf.shape[2] == nres)
+        nq = 0 if ind is None else ind.shape[2] * 128
+        assert nq + nres == n == cache[-1] and 0 <= nres < 128
+        assert (vc is None) == (ind is None)
+        if vc is not None:
+            assert vc.shape == (1, 2, nq, 16) and vs.shape == vm.shape == (1, 2, nq, 1)
+        assert out.shape == (1, 4, 1, 128)
