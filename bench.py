@@ -187,6 +187,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-baselines", action="store_true", help="skip the CPU and fp16 baselines")
     ap.add_argument("--splits", type=int, default=0, help="override the context split count")
+    ap.add_argument("--no-values4", action="store_true", help="skip the 4-bit-value (Mixed variant) measurement")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run 3 plain 1 GiB device copies (torch clone): under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` "
                          "their counter values give the scale factor for the attention kernel's")
@@ -263,6 +264,36 @@ def main():
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES},
     }
+    # the same step with the values of the quantized groups in 4 bits (the reference's Mixed variant)
+    if not args.no_values4:
+        from polarquant_amd.attention import polar_decode_attention_v4
+        from polarquant_amd.values import quantize_values
+        L = w["n_groups"] * 128
+        v4sets = []
+        for x in sets:
+            vq = quantize_values(x["v"][:, :, :L])
+            vres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=dev)
+            vres[:, :, :1] = x["v"][:, :, L:L + 1]
+            v4sets.append((vq, vres))
+        out4 = torch.empty_like(out)
+
+        def step4():
+            i = turn[0] & 1
+            x, (vq, vres) = sets[i], v4sets[i]
+            turn[0] += 1
+            polar_decode_attention_v4(x["q"], x["codes"], *x["meta"], x["kres"], vres, *vq, x["n_groups"], x["n_resid"],
+                                      rbits=sh.rbits, tbits=sh.tbits, out=out4)
+
+        ms4 = time_events(step4, args.steps, args.warmup)
+        bytes4 = wl.algorithmic_bytes(Nk, N, [L] * B, [w["n_resid"]] * B, sh.rbits, sh.tbits, value_bits=4)
+        result["values4"] = {
+            "workload": "same step, values of the quantized groups in 4 bits (Mixed variant): 136 B instead of 324 B per token and KV head",
+            "us_per_step": round(ms4 * 1e3, 2), "algorithmic_bytes": bytes4,
+            "hbm_gbps": round(bytes4 / (ms4 * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(bytes4 / (ms4 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "speedup_vs_fp16_values": round(ms / ms4, 3),
+            "max_abs_diff_vs_fp16_values": float((out4.float() - out.float()).abs().max()),
+        }
+        del v4sets
     turn[0] = 0
     step()                                   # leave set 0's result in `out` for the parity check
     torch.cuda.synchronize()

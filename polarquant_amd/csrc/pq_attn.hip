@@ -170,14 +170,21 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
         for (int e = 0; e < 8; e++) st.acc[e] *= a;
     }
     const int slot = v4_slot(lane);
-    const float scp = sc * kV4Pre;
+    // The weight the matrix cores see is w = half(p * scale * kV4Pre).  The zero-point term must use
+    // the SAME rounded weight (w * zero / (scale * kV4Pre)), not p: code * scale and zero are each a few
+    // units large and cancel to a value of order 1, so a weight that differs between the two terms by
+    // its rounding error (2^-11) would leave an error of that size times ~3 when one token dominates.
+    // A constant row has scale 0 and all codes 0: any scale serves, take 1.
+    const float scp = (sc == 0.0f ? 1.0f : sc) * kV4Pre;
+    const float zq = zp / scp;
 #pragma unroll
     for (int j = 0; j < REPP; j++) {
         const float ms = (st.m[j] == -INFINITY) ? 0.0f : st.m[j];
         const float p = exp2f(t[j] - ms);
         st.l[j] += p;
-        st.zp[j] = __builtin_fmaf(p, zp, st.zp[j]);
-        *lds_ptr<__attribute__((address_space(3))) uint16_t>(pbuf + (j * kWave + slot) * 2) = f2lo<F16>(p * scp);
+        const uint16_t wh = f2lo<F16>(p * scp);
+        st.zp[j] = __builtin_fmaf(lo2f<F16>(wh), zq, st.zp[j]);
+        *lds_ptr<__attribute__((address_space(3))) uint16_t>(pbuf + (j * kWave + slot) * 2) = wh;
     }
     asm volatile("" ::: "memory");
     const int g = lane >> 4, n = lane & 15;

@@ -108,13 +108,16 @@ def make_decode_inputs(shape: Shape, dtype=torch.float16, context: Optional[int]
 
 
 def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], resid_tokens: List[int],
-                      rbits: int = 4, tbits: int = 4, code_bytes_per_pair: float = 1.0) -> int:
+                      rbits: int = 4, tbits: int = 4, code_bytes_per_pair: float = 1.0, value_bits: int = 16) -> int:
     """HBM bytes one fused decode-attention step must move: one byte per pair
     code (the stored layout), 4 half metadata words per (group, pair), fp16 V
-    for every token, fp16 residual keys, plus q in / out."""
+    for every token, fp16 residual keys, plus q in / out.  With value_bits=4 (Mixed
+    variant) the values of the quantized tokens are 64 bytes of codes plus a half
+    scale and zero-point each; the residual window's values stay fp16."""
     total = 0
     for lq, res in zip(quant_tokens, resid_tokens):
+        v_bytes = lq * HEAD_DIM * 2 if value_bits == 16 else lq * (HEAD_DIM * value_bits // 8 + 4)
         total += n_kv_heads * (int(lq * 64 * code_bytes_per_pair) + (lq // GROUP) * 4 * 64 * 2
-                               + (lq + res) * HEAD_DIM * 2 + res * HEAD_DIM * 2)
+                               + v_bytes + res * HEAD_DIM * 2 + res * HEAD_DIM * 2)
     total += 2 * len(quant_tokens) * n_heads * HEAD_DIM * 2
     return total

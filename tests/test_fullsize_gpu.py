@@ -147,3 +147,47 @@ def test_cfg3_full_size_append_and_decode(gpu):
     for ns in (64, 333):
         ok, err = _ok(_attn(w, n_splits=ns).cpu(), out.cpu())
         assert ok, (ns, err)
+
+
+def test_cfg1_full_size_with_4bit_values(gpu):
+    """configs[1] with the values of the quantized groups in 4 bits (the Mixed variant): the value
+    quantizer over 4.2M rows against the oracle on whole planes (bit-exact), the attention against
+    the fp64 oracle on whole planes, split invariance, and chunked == one-shot value quantization."""
+    from polarquant_amd.attention import polar_decode_attention_v4
+    from polarquant_amd.values import quantize_values
+    print("building configs[1] + 4-bit values", flush=True)
+    w = bench.build_workload(1, gpu)
+    sh = w["shape"]
+    B, Nk, rep = sh.batch, sh.n_kv_heads, sh.n_heads // sh.n_kv_heads
+    L = w["n_groups"] * 128
+    vq = quantize_values(w["v"][:, :, :L])
+    vres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=gpu)
+    vres[:, :, :1] = w["v"][:, :, L:L + 1]
+    # chunked quantization into a pre-allocated store == one shot
+    store = (torch.empty_like(vq[0]), torch.empty_like(vq[1]), torch.empty_like(vq[2]))
+    for t0 in range(0, L, 8192):
+        quantize_values(w["v"][:, :, t0:t0 + 8192], out=store, token_offset=t0)
+    assert all(torch.equal(a, b) for a, b in zip(store, vq))
+
+    def attn(**kw):
+        return polar_decode_attention_v4(w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], 1,
+                                         rbits=sh.rbits, tbits=sh.tbits, **kw)
+    out = attn().clone()
+    torch.cuda.synchronize()
+    assert out.shape == (16, 32, 1, 128) and torch.isfinite(out.float()).all()
+    for b, kvh in [(0, 0), (9, 2), (15, 7)]:
+        v_plane = w["v"][b:b + 1, kvh:kvh + 1, :L].cpu()
+        ref_q = po.quantize_values_along_last_dim(v_plane)
+        for got, ref in zip(vq, ref_q):
+            g = got[b:b + 1, kvh:kvh + 1].cpu()
+            assert torch.equal(g if g.dtype == torch.int32 else g.view(torch.int16), ref if ref.dtype == torch.int32 else ref.view(torch.int16))
+        q = w["q"][b:b + 1, kvh * rep:(kvh + 1) * rep].cpu()
+        quant = [w["codes"][b:b + 1, kvh:kvh + 1].cpu()] + [m[b:b + 1, kvh:kvh + 1].cpu() for m in w["meta"]]
+        ref = po.decode_attention_mixed_exact(q, w["kres"][b:b + 1, kvh:kvh + 1, :1].cpu(), *quant,
+                                              vres[b:b + 1, kvh:kvh + 1, :1].cpu(), *ref_q)
+        ok, err = _ok(out[b:b + 1, kvh * rep:(kvh + 1) * rep].cpu(), ref)
+        print("plane", b, kvh, "max abs err %.2e" % err, flush=True)
+        assert ok
+    for ns in (3, 8, 64):
+        ok, err = _ok(attn(n_splits=ns).cpu(), out.cpu())
+        assert ok, (ns, err)

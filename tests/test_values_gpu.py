@@ -130,3 +130,30 @@ def test_attention_v4_bf16(gpu):
     out, ref, ref64 = _case(gpu, 2, 8, 2, 16, 3, 4, 4, torch.bfloat16, seed=4)
     nbad, emax = _close(out, ref64, 2e-2, 4e-3)      # bf16 has 8 mantissa bits
     assert nbad == 0, (nbad, emax)
+
+
+def test_attention_v4_peaked_softmax_keeps_code_and_zero_point_terms_consistent(gpu):
+    """When one token takes nearly all the probability, code*scale (~3) and the zero-point (~-3) of
+    that token must be weighted by the same rounded probability, or their cancellation leaves an
+    error of a probability's rounding error times 3.  Checked tightly against fp64, for 1 and many splits."""
+    g = torch.Generator().manual_seed(77)
+    B, N, Nk, nb = 1, 4, 1, 24
+    L = nb * 128
+    k = wl.make_keys(B, Nk, L + 1, 5e5, g)
+    q = wl.make_half((B, N, 1, 128), g)
+    for j in range(N):
+        q[0, j, 0] = (k[0, 0, 100 + 500 * j].float() * 0.9).half()      # each head locks onto one cached token
+    v = wl.make_half((B, Nk, L + 1, 128), g)
+    quant = po.quantize_and_pack_nbit(k[:, :, :L].contiguous())
+    vq = po.quantize_values_along_last_dim(v[:, :, :L].contiguous())
+    kres, vres = k[:, :, L:].contiguous(), v[:, :, L:].contiguous()
+    ref64 = po.decode_attention_mixed_exact(q, kres, *quant, vres, *vq)
+    dk = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=gpu)
+    dv = torch.zeros_like(dk)
+    dk[:, :, :1], dv[:, :, :1] = kres.to(gpu), vres.to(gpu)
+    for ns in (1, 4, 24):
+        out = polar_decode_attention_v4(q.to(gpu), *[t.to(gpu) for t in quant], dk, dv, *[t.to(gpu) for t in vq], nb, 1,
+                                        n_splits=ns).cpu()
+        err = (out.double() - ref64).abs().max().item()
+        print("peaked, n_splits", ns, "max abs err %.2e (|out| up to %.2f)" % (err, ref64.abs().max().item()), flush=True)
+        assert err < 1.5e-3 * max(1.0, ref64.abs().max().item()), (ns, err)
