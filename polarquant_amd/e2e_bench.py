@@ -5,7 +5,7 @@ Reports prefill seconds, decode tokens/s and KV-cache bytes per token.  Mirrors 
 reference's throughput script (benchmark/benchmark_throughput.py:15-113): one timed prefill,
 then the timed greedy loop with EOS made unreachable.
 
-    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32] [--graph]
+    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32] [--graph] [--values4]
 
 --graph replays the decode step from a captured HIP graph (polarquant_amd/graph_decode.py)
 instead of driving ~40 launches per layer from Python.
@@ -46,10 +46,11 @@ def main():
     ap.add_argument("--new", type=int, default=256)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--graph", action="store_true")
+    ap.add_argument("--values4", action="store_true", help="4-bit values as well (the reference's Mixed variant)")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = PolarConfig.llama3_8b(num_hidden_layers=args.layers, cache_capacity=args.prompt + args.new + 128,
-                                eos_token_id=[128256 + 10])
+                                eos_token_id=[128256 + 10], vbits=4 if args.values4 else 16)
     model = build_model(cfg, dev)
     g = torch.Generator(device=dev).manual_seed(1004)
     ids = torch.randint(0, cfg.vocab_size, (args.batch, args.prompt), generator=g, device=dev)
@@ -96,7 +97,7 @@ def main():
     print(json.dumps({
         "workload": "configs[4]: greedy decode, random-init Llama-3-8B architecture, bf16, batch %d, prompt %d, %d new tokens"
                     % (args.batch, args.prompt, args.new),
-        "layers": args.layers, "graph": bool(args.graph), "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
+        "layers": args.layers, "graph": bool(args.graph), "values": "4-bit" if args.values4 else "half", "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
         "decode_ms_per_step": round(1e3 * t_decode / steps, 3),
         "decode_tokens_per_s": round(args.batch * steps / t_decode, 1),
         "kv_cache_bytes_per_token": kv, "fp16_kv_cache_bytes_per_token": fp16_kv,

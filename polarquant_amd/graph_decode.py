@@ -22,7 +22,8 @@ from typing import List, Optional
 
 import torch
 
-from .attention import plan_splits, polar_decode_attention, workspace_for
+from . import _ffi
+from .attention import _num_cus, plan_splits, polar_decode_attention, polar_decode_attention_v4, workspace_for
 from .modeling_common import GROUP, apply_rotary_pos_emb
 
 
@@ -65,7 +66,11 @@ class PolarGraphDecoder:
         emb = torch.cat([ang, ang], dim=-1)
         self.cos_table, self.sin_table = emb.cos().to(dtype), emb.sin().to(dtype)
         nk = a0.Nk
-        self.n_splits = plan_splits(B, nk, max(self.max_len // GROUP, 1), dev)
+        self.mixed = hasattr(a0, "vcodes")          # Mixed variant: 4-bit values, shared residual window
+        if self.mixed:
+            self.n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, cfg.num_attention_heads, nk, max(self.max_len // GROUP, 1), _num_cus(dev))
+        else:
+            self.n_splits = plan_splits(B, nk, max(self.max_len // GROUP, 1), dev)
         workspace_for(B, cfg.num_attention_heads, self.n_splits, dev)                     # allocate before capture
         self.logits = None
         self.graph = None
@@ -87,10 +92,17 @@ class PolarGraphDecoder:
             v = att.v_proj(h).view(B, 1, att.num_key_value_heads, att.head_dim).transpose(1, 2)
             q, k = apply_rotary_pos_emb(q, k, cos, sin)
             ar.kres.index_copy_(2, self.resid_idx, k)
-            ar.v.index_copy_(2, self.pos, v)
-            o = polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, rbits=att.rbits, tbits=att.tbits,
-                                       sm_scale=1.0 / math.sqrt(att.head_dim), n_groups_per_seq=self.n_groups_dev,
-                                       n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits)
+            if self.mixed:
+                ar.vres.index_copy_(2, self.resid_idx, v)
+                o = polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0,
+                                              rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
+                                              n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev,
+                                              n_splits=self.n_splits)
+            else:
+                ar.v.index_copy_(2, self.pos, v)
+                o = polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, rbits=att.rbits, tbits=att.tbits,
+                                           sm_scale=1.0 / math.sqrt(att.head_dim), n_groups_per_seq=self.n_groups_dev,
+                                           n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits)
             x = x + att.o_proj(o.reshape(B, 1, -1))
             x = x + layer.mlp(layer.post_attention_layernorm(x))
         logits = model.lm_head(model.model.norm(x))
@@ -104,8 +116,11 @@ class PolarGraphDecoder:
         """Residual window full (128 keys): quantize it into the next group slot (reference :83-92)."""
         for ar in self.arenas:
             ar.n_resid, ar.kv_len = GROUP, self.kv_len
-            ar.quantize_into(ar.kres)
-            ar.n_resid = 0
+            if self.mixed:
+                ar.flush()
+            else:
+                ar.quantize_into(ar.kres)
+                ar.n_resid = 0
         self.n_resid = 0
         self.resid_idx.zero_()
         self.n_groups_dev.add_(1)

@@ -56,6 +56,7 @@ class PolarConfig:
     # polar cache
     rbits: int = 4
     tbits: int = 4
+    vbits: int = 16                     # 4: values in 4 bits as well (the Mixed variant); 16: half-precision values
     cache_capacity: int = 0             # tokens to pre-allocate per layer (0: prompt + 1024, grown by doubling)
 
     @staticmethod
@@ -471,12 +472,17 @@ class CausalLMOutputWithPast:
 
 class PolarDecoderLayer(nn.Module):
     attention_class = PolarGroupAttention
+    mixed_attention_class = None       # set below, once PolarMixedGroupAttention exists in the subclasses' modules
 
     def __init__(self, config, layer_idx):
         super().__init__()
         self.config, self.layer_idx = config, layer_idx
         self.hidden_size = config.hidden_size
-        self.self_attn = self.attention_class(config, layer_idx)
+        # config.vbits == 4 selects the Mixed variant (the reference switches by editing
+        # modeling_llama_polar.py:452-453); anything else keeps half-precision values
+        mixed = _cfg(config, "vbits", 16) == 4
+        cls = (self.mixed_attention_class or PolarMixedGroupAttention) if mixed else self.attention_class
+        self.self_attn = cls(config, layer_idx)
         self.mlp = MLP(config)
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
@@ -549,10 +555,11 @@ class PolarForCausalLM(nn.Module):
 
     def kv_cache_bytes_per_token(self) -> int:
         """Bytes one cached token costs across all layers: 1 code byte per pair, 4 metadata
-        halves per (group, pair) amortised over 128 tokens, fp16 V."""
+        halves per (group, pair) amortised over 128 tokens, fp16 V (or 4-bit V with config.vbits == 4)."""
         c = self.config
         nk = _cfg(c, "num_key_value_heads", c.num_attention_heads)
-        return c.num_hidden_layers * nk * (64 + 4 * 64 * 2 // 128 + 128 * 2)
+        v_bytes = 128 // 2 + 2 * 2 if _cfg(c, "vbits", 16) == 4 else 128 * 2      # 4-bit codes + half scale and zero-point
+        return c.num_hidden_layers * nk * (64 + 4 * 64 * 2 // 128 + v_bytes)
 
 
 # ----------------------------------------------------------------------------- generation (reference :565-666)

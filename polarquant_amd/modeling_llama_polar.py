@@ -18,6 +18,7 @@ class LlamaPolarMixedGroupAttention(PolarMixedGroupAttention):
 
 class LlamaPolarDecoderLayer(PolarDecoderLayer):
     attention_class = LlamaPolarGroupAttention
+    mixed_attention_class = LlamaPolarMixedGroupAttention
 
 
 class LlamaPolarModel(PolarModel):

@@ -28,6 +28,7 @@ def _same_cache(a, b):
 @pytest.mark.parametrize("cls,cfg,dtype", [
     (LlamaPolarForCausalLM, _tiny(), torch.float16),
     (Qwen2PolarForCausalLM, _tiny(7, 1, rbits=3, tbits=3, attention_bias=True), torch.bfloat16),
+    (LlamaPolarForCausalLM, _tiny(8, 2, vbits=4), torch.float16),          # Mixed variant: 4-bit values, 11-slot cache
 ])
 def test_graph_decoder_matches_eager_model(gpu, cls, cfg, dtype):
     """Three decoders in lock step over 140 tokens (two residual flushes): the eager drop-in model,
