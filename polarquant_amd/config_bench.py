@@ -1,0 +1,87 @@
+"""The other BASELINE configurations on one GPU, same kernels and timing as bench.py
+(which carries the headline, configs[1]):
+
+  configs[0]  score op, Llama-2-7B shape (batch 1, 32 heads MHA, context 4096)
+  configs[2]  ragged continuous-batch decode attention, Qwen2.5-7B shape (batch 64, GQA 7, 3/3 bits)
+  configs[3]  prompt quantization (append) of 131072 keys x 8 KV heads, then one decode step over them
+
+    python -m polarquant_amd.config_bench [--configs 0 2 3] [--values4]
+
+Prints one JSON line per measurement: µs per call, algorithmic bytes, GB/s and fraction of the
+8 TB/s HBM peak.  --values4 adds the decode step with 4-bit values (Mixed variant) for the
+uniform-length configurations.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+
+import torch
+
+from . import workloads as wl
+from .attention import polar_decode_attention, polar_decode_attention_v4
+from .kernel4group import attention_decode_forward_triton_impl
+from .quantize import quantize_and_pack_nbit
+from .values import quantize_values
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def _line(cfg, op, ms, nbytes, **extra):
+    gbps = nbytes / (ms * 1e-3) / 1e9
+    print(json.dumps(dict(config=cfg, op=op, us=round(ms * 1e3, 2), algorithmic_bytes=int(nbytes), hbm_gbps=round(gbps, 1),
+                          frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)), flush=True)
+
+
+def run(idx: int, dev, values4: bool, steps: int):
+    w = wl.build_workload(idx, dev, keep_keys=(idx == 3))
+    sh = w["shape"]
+    B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
+    if idx == 0:
+        ms = wl.time_events(lambda: attention_decode_forward_triton_impl(w["q"], w["codes"], *w["meta"], rbits=sh.rbits, tbits=sh.tbits),
+                            4 * steps, steps)
+        nbytes = w["codes"].numel() + 4 * w["meta"][0].numel() * 2 + B * N * sh.context * 4 + w["q"].numel() * 2
+        _line(idx, "scores (pq_decode_scores)", ms, nbytes)
+    if sh.ragged:
+        lens = w["lengths"]
+        lq, res = ((lens // 128) * 128).tolist(), (lens % 128).tolist()
+        total_groups = int((lens // 128).sum())
+    else:
+        lq, res, total_groups = [w["n_groups"] * 128] * B, [w["n_resid"]] * B, None
+    nbytes = wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits)
+    ms = wl.time_events(lambda: polar_decode_attention(
+        w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
+        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups), steps, 10)
+    _line(idx, "decode attention (pq_decode_attn)", ms, nbytes, tokens=int(sum(lq) + sum(res)))
+    if values4 and not sh.ragged:
+        L = w["n_groups"] * 128
+        vq = quantize_values(w["v"][:, :, :L])
+        vres = torch.zeros(B, Nk, 128, 128, dtype=w["v"].dtype, device=dev)
+        vres[:, :, :w["n_resid"]] = w["v"][:, :, L:L + w["n_resid"]]
+        ms4 = wl.time_events(lambda: polar_decode_attention_v4(
+            w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits), steps, 10)
+        _line(idx, "decode attention, 4-bit values (pq_decode_attn_v4)", ms4,
+              wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits, value_bits=4))
+        msq = wl.time_events(lambda: quantize_values(w["v"][:, :, :L], out=vq), max(steps // 2, 5), 3)
+        _line(idx, "value quantization (pq_quantize_values)", msq, B * Nk * L * (256 + 64 + 4))
+    if idx == 3:
+        k = w["keys"]
+        out = (torch.empty_like(w["codes"]), *[torch.empty_like(m) for m in w["meta"]])
+        ms = wl.time_events(lambda: quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=out), max(steps // 2, 5), 5)
+        _line(idx, "append / prompt quantization (pq_quantize_groups)", ms, k.numel() * 2 + out[0].numel() + 4 * out[1].numel() * 2)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--configs", type=int, nargs="*", default=[0, 2, 3])
+    ap.add_argument("--values4", action="store_true")
+    ap.add_argument("--steps", type=int, default=100)
+    args = ap.parse_args()
+    dev = torch.device("cuda:0")
+    for idx in args.configs:
+        run(idx, dev, args.values4, args.steps)
+        torch.cuda.empty_cache()
+
+
+if __name__ == "__main__":
+    main()

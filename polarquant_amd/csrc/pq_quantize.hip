@@ -147,18 +147,17 @@ template <> struct PkInit<BF16> { static constexpr uint32_t kMax = 0x00000000u, 
 // formula with the constants tmn = -pi and tscale = 2*pi / 2^tbits (both rounded to the key dtype);
 // the angle code is then known in the first pass and is what the angle word carries.
 struct AngleMode {
-    bool uniform;
     float two_pi;      // reference mode: the constant added to negative angles
     float tmn, tscale; // uniform mode
     int ttop;
 };
 
 // (angle word | radius word << 16) of one pair: wrap applied, sign bits cleared
-template <typename T>
+template <typename T, bool UNIFORM>
 __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const AngleMode& am) {
     float phi = rnd<T>(a);
     uint32_t aw;
-    if (am.uniform) {
+    if constexpr (UNIFORM) {
         aw = code_of<T>(phi, am.tmn, am.tscale, am.ttop);
     } else {
         if (phi < 0.0f) phi = rnd<T>(phi + am.two_pi);             // :144
@@ -167,7 +166,7 @@ __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const An
     return (aw | (static_cast<uint32_t>(f2lo<T>(r)) << 16)) & 0x7fff7fffu;
 }
 
-template <typename T>
+template <typename T, bool UNIFORM>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t st, int Nk, int rbits, int tbits, AngleMode am,
     uint8_t* __restrict__ codes, uint16_t* __restrict__ rscale, uint16_t* __restrict__ rmn,
@@ -199,7 +198,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
             float a, r;
             const bool risky = angle_radius_fast<T>(lo2f<T>(xs[i]), lo2f<T>(ys[i]), &a, &r);   // :143, :150
             risky_mask |= static_cast<uint32_t>(risky) << (it * 4 + i);
-            pr[it * 4 + i][tid] = pack_angle_radius<T>(a, rnd<T>(r), am);
+            pr[it * 4 + i][tid] = pack_angle_radius<T, UNIFORM>(a, rnd<T>(r), am);
         }
     }
     // ---- fix-up: each lane redoes ITS risky entries with the exact routines (a lane has ~0.1 of
@@ -211,7 +210,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         const float x = lo2f<T>(row[4 * pq4 + (e & 3)]), y = lo2f<T>(row[kPairs + 4 * pq4 + (e & 3)]);
         float a, r;
         angle_radius_exact<T>(x, y, &a, &r);
-        pr[e][tid] = pack_angle_radius<T>(a, r, am);
+        pr[e][tid] = pack_angle_radius<T, UNIFORM>(a, r, am);
     }
     // ---- per-pair max / min of angle and radius over the 128 tokens (packed: both at once)
     uint32_t vmax[4], vmin[4];
@@ -254,7 +253,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         tm[i] = lo2f<T>(static_cast<uint16_t>(wmin & 0xffffu));
         rm[i] = lo2f<T>(static_cast<uint16_t>(wmin >> 16));
         ts[i] = rnd<T>(rnd<T>(lo2f<T>(static_cast<uint16_t>(wmax & 0xffffu)) - tm[i]) / inv_t);   // :147
-        if (am.uniform) { tm[i] = am.tmn; ts[i] = am.tscale; }
+        if constexpr (UNIFORM) { tm[i] = am.tmn; ts[i] = am.tscale; }
         rs[i] = rnd<T>(rnd<T>(lo2f<T>(static_cast<uint16_t>(wmax >> 16)) - rm[i]) / inv_r);       // :152
     }
     const size_t plane = static_cast<size_t>(bh) * cap + off + grp;
@@ -280,7 +279,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
             const uint32_t v = pr[it * 4 + i][tid];
             const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
             const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
-            const uint32_t th = am.uniform ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop);    // :148
+            const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop);    // :148
             const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop);      // :153
             w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
         }
@@ -322,7 +321,7 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
     const float two_pi_f = 6.28318548202514648438f;   // (float)(2*pi)
     // eager torch-CPU casts the python scalar 2*pi to the tensor dtype first: 6.28125 in both dtypes
     AngleMode am;
-    am.uniform = (flags & 2u) != 0;
+    const bool uniform = (flags & 2u) != 0;
     am.two_pi = (flags & 1u) ? two_pi_f : 6.28125f;
     am.ttop = (1 << tbits) - 1;
     const bool bf = dtype != 0;
@@ -331,14 +330,13 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
     };
     am.tmn = round_dt(-3.14159274101257324219f);
     am.tscale = round_dt(round_dt(two_pi_f) / static_cast<float>(1 << tbits));
-    if (dtype == 0)
-        hipLaunchKernelGGL(quantize_kernel<F16>, grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],
-                           strides[2], Nk, rbits, tbits, am, codes, (uint16_t*)rscale, (uint16_t*)rmn,
-                           (uint16_t*)tscale, (uint16_t*)tmn, cap, off);
-    else
-        hipLaunchKernelGGL(quantize_kernel<BF16>, grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],
-                           strides[2], Nk, rbits, tbits, am, codes, (uint16_t*)rscale, (uint16_t*)rmn,
-                           (uint16_t*)tscale, (uint16_t*)tmn, cap, off);
+#define PQ_LAUNCH_Q(T, U)                                                                                            \
+    hipLaunchKernelGGL((quantize_kernel<T, U>), grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],     \
+                       strides[2], Nk, rbits, tbits, am, codes, (uint16_t*)rscale, (uint16_t*)rmn,                  \
+                       (uint16_t*)tscale, (uint16_t*)tmn, cap, off)
+    if (dtype == 0) { if (uniform) PQ_LAUNCH_Q(F16, true); else PQ_LAUNCH_Q(F16, false); }
+    else            { if (uniform) PQ_LAUNCH_Q(BF16, true); else PQ_LAUNCH_Q(BF16, false); }
+#undef PQ_LAUNCH_Q
     return static_cast<int>(hipGetLastError());
 }
 

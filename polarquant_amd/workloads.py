@@ -121,3 +121,62 @@ def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], re
                                + v_bytes + res * HEAD_DIM * 2 + res * HEAD_DIM * 2)
     total += 2 * len(quant_tokens) * n_heads * HEAD_DIM * 2
     return total
+
+
+# ----------------------------------------------------------------------------- GPU-resident workloads and timing
+def build_workload(idx, dev, dtype=torch.float16, keep_keys=False):
+    """configs[idx] resident in HBM: polar key cache of L/128 groups per (sequence, KV head),
+    fp16 V cache, one new token whose key sits in the fp16 residual buffer.  Ragged shapes
+    (configs[2]) carry per-sequence group / residual counts; their caches are sized for the longest."""
+    from .quantize import quantize_and_pack_nbit
+
+    sh = CONFIGS[idx]
+    B, N, Nk, L = sh.batch, sh.n_heads, sh.n_kv_heads, sh.context
+    Nb = L // 128
+    g = torch.Generator(device=dev).manual_seed(sh.seed)
+    codes = torch.empty(B, Nk, Nb, 128, 64, dtype=torch.uint8, device=dev)
+    meta = [torch.empty(B, Nk, Nb, 1, 64, dtype=dtype, device=dev) for _ in range(4)]
+    inv_freq = 1.0 / (sh.rope_theta ** (torch.arange(0, 128, 2, dtype=torch.float32, device=dev) / 128))
+    ang = torch.arange(L, dtype=torch.float32, device=dev)[:, None] * inv_freq[None, :]
+    cos, sin = torch.cat([ang, ang], -1).cos(), torch.cat([ang, ang], -1).sin()
+    outl = torch.randperm(128, generator=g, device=dev)[:4]
+    keys = []
+    for b in range(B):                      # keys of one sequence at a time
+        k = torch.randn(1, Nk, L, 128, generator=g, device=dev, dtype=torch.float32)
+        k[..., outl] *= 8.0
+        k = (k * cos + torch.cat([-k[..., 64:], k[..., :64]], -1) * sin).to(dtype)
+        quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=(codes[b:b + 1], *[m[b:b + 1] for m in meta]))
+        if keep_keys:
+            keys.append(k)
+    v = torch.empty(B, Nk, L + 1, 128, dtype=dtype, device=dev)
+    for b in range(B):
+        v[b] = torch.randn(Nk, L + 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    q = torch.randn(B, N, 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    k_new = torch.randn(B, Nk, 1, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+    kres = torch.zeros(B, Nk, 128, 128, dtype=dtype, device=dev)
+    kres[:, :, :1] = k_new
+    w = dict(shape=sh, q=q, codes=codes, meta=meta, kres=kres, v=v, n_groups=Nb, n_resid=1, lengths=None,
+             groups_per_seq=None, resid_per_seq=None, keys=torch.cat(keys, 0) if keep_keys else None)
+    if sh.ragged:
+        # per-sequence context lengths, uniform in [512, L]: full groups are quantized, the tail
+        # (L % 128 tokens) stays fp16 in the residual buffer, which is filled from the keys' tail
+        lens = torch.randint(512, L + 1, (B,), generator=torch.Generator().manual_seed(sh.seed))
+        w["lengths"] = lens
+        w["groups_per_seq"] = (lens // 128).int().to(dev)
+        w["resid_per_seq"] = (lens % 128).int().to(dev)
+        w["kres"] = torch.randn(B, Nk, 128, 128, generator=g, device=dev, dtype=torch.float32).to(dtype)
+        w["n_groups"], w["n_resid"] = 0, 0
+    return w
+
+
+def time_events(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps      # ms per call
