@@ -42,10 +42,8 @@ template <> __device__ __forceinline__ uint16_t f2lo<F16>(float f) {
     return __half_as_ushort(__float2half_rn(f));
 }
 template <> __device__ __forceinline__ uint16_t f2lo<BF16>(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<uint16_t>(u >> 16);
+    // one v_cvt_pk_bf16_f32 on gfx950 (round to nearest even, NaN stays NaN)
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).  Unlike
