@@ -247,6 +247,40 @@ int pq_decode_attn_v4(const void *q,
                       int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
                       void *out, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * A — the elementwise steps around the attention call of one decode step, each a
+ * chain of 8-12 eager launches on a [B,1,hidden] activation in the reference.
+ * Arithmetic follows the eager modules op by op (fp32 result rounded to the
+ * dtype after every op).
+ *
+ * pq_rope_append: HF apply_rotary_pos_emb on the new token's q and k
+ * (models/modeling_llama_polar.py:56-59), the key's append to the residual
+ * window (:77) and the value's append to the value cache (:98), in one launch.
+ * The position and the destination rows are read from device memory, so the
+ * launch can be replayed from a captured graph.
+ *   q_lin [B,N*128], k_lin / v_lin [B,Nk*128]  projection outputs, contiguous
+ *   cos_table / sin_table [table_rows,128]     in the dtype; row *pos is used
+ *   q_out [B,N,128]
+ *   k_dst [B,Nk,k_rows,128], row *k_row <- rotated key
+ *   v_dst [B,Nk,v_rows,128], row *v_row <- value
+ *
+ * pq_rmsnorm: y = weight * dtype(float(s) * rsqrt(mean(float(s)^2) + eps)) with
+ * s = x, or s = dtype(x + residual) (also written to sum_out if given; sum_out may
+ * alias x): the decoder layer's residual add + LlamaRMSNorm (:466-484).
+ *
+ * pq_silu_mul: y = dtype(silu(gate)) * up over n elements (LlamaMLP, called at :483).
+ * ------------------------------------------------------------------------- */
+int pq_rope_append(const void *q_lin, const void *k_lin, const void *v_lin,
+                   const void *cos_table, const void *sin_table, int64_t table_rows, const int64_t *pos,
+                   void *q_out, void *k_dst, int64_t k_rows, const int64_t *k_row,
+                   void *v_dst, int64_t v_rows, const int64_t *v_row,
+                   int B, int N, int Nk, int dtype, void *stream);
+
+int pq_rmsnorm(const void *x, const void *residual, const void *weight, void *y, void *sum_out,
+               int rows, int hidden, float eps, int dtype, void *stream);
+
+int pq_silu_mul(const void *gate, const void *up, void *y, size_t n, int dtype, void *stream);
+
 /* Split count for pq_decode_attn_v4 (as pq_decode_attn_plan, which see; the 4-bit
  * kernel runs two wavefronts per SIMD when N/Nk <= 4). No reference counterpart. */
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus);

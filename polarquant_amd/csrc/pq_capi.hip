@@ -236,6 +236,41 @@ int pq_decode_attn(const void* q,
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
 
+// ---- fused elementwise steps of the decode layer -----------------------------------------------
+int pq_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_table, const void* sin_table,
+                   int64_t table_rows, const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
+                   void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int dtype, void* stream) {
+    if (!q_lin || !k_lin || !v_lin || !cos_table || !sin_table || !pos || !q_out || !k_dst || !k_row || !v_dst || !v_row)
+        return PQ_ERR_NULL_POINTER;
+    if (B <= 0 || N <= 0 || Nk <= 0 || B > 65535) return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (table_rows <= 0 || k_rows <= 0 || v_rows <= 0) return PQ_ERR_BAD_STRIDE;
+    const int err = pq::launch_rope_append(q_lin, k_lin, v_lin, cos_table, sin_table, pos, q_out, k_dst, k_rows, k_row, v_dst,
+                                           v_rows, v_row, B, N, Nk, table_rows, dtype, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+int pq_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* sum_out, int rows, int hidden,
+               float eps, int dtype, void* stream) {
+    if (!x || !weight || !y) return PQ_ERR_NULL_POINTER;
+    if (rows <= 0 || hidden <= 0 || hidden % 8) return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (!aligned(x, 16) || !aligned(weight, 16) || !aligned(y, 16) || (residual && !aligned(residual, 16)) ||
+        (sum_out && !aligned(sum_out, 16)))
+        return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_rmsnorm(x, residual, weight, y, sum_out, rows, hidden, eps, dtype, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
+int pq_silu_mul(const void* gate, const void* up, void* y, size_t n, int dtype, void* stream) {
+    if (!gate || !up || !y) return PQ_ERR_NULL_POINTER;
+    if (n == 0 || n % 8) return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (!aligned(gate, 16) || !aligned(up, 16) || !aligned(y, 16)) return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_silu_mul(gate, up, y, n, dtype, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;

@@ -1,0 +1,193 @@
+// Small fused kernels for the decode step around the attention call
+// (models/modeling_llama_polar.py:47-59 projections -> RoPE -> cache append, and the
+// decoder layer's norms / MLP activation, :456-486), each replacing a chain of
+// 8-12 eager elementwise launches on a [B, 1, hidden] activation:
+//
+//   rope_append_kernel  q/k rotation (HF rotate-half) + write of the new key into the residual
+//                       window + write of the new value into the value cache, positions read
+//                       from device memory so that the step can be replayed from a graph
+//   rmsnorm_kernel      (optional residual add) + RMS norm
+//   silu_mul_kernel     silu(gate) * up
+//
+// Arithmetic follows the eager modules op by op in the activation dtype: every
+// product / sum is formed in fp32 and rounded to the dtype before the next op.
+#include "pq_device.h"
+#include "pq_internal.h"
+
+namespace pq {
+
+template <typename T>
+__device__ __forceinline__ float rnd_a(float f) { return lo2f<T>(f2lo<T>(f)); }
+
+// grid (N + 2*Nk, B), 64 threads: lane d owns the pair (d, d+64) of one head.
+//   q_lin [B, N*128], k_lin / v_lin [B, Nk*128]: outputs of the projections for the new token
+//   cos_tab / sin_tab [max_pos, 128] in the dtype; *pos = position of the new token
+//   q_out [B, N, 128]
+//   k_dst [B, Nk, k_rows, 128]: row *k_row receives the rotated key
+//   v_dst [B, Nk, v_rows, 128]: row *v_row receives the value
+template <typename T>
+__global__ __launch_bounds__(kWave) void rope_append_kernel(
+    const uint16_t* __restrict__ q_lin, const uint16_t* __restrict__ k_lin, const uint16_t* __restrict__ v_lin,
+    const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab, const int64_t* __restrict__ pos,
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_dst, int64_t k_rows, const int64_t* __restrict__ k_row,
+    uint16_t* __restrict__ v_dst, int64_t v_rows, const int64_t* __restrict__ v_row, int N, int Nk, int64_t max_pos) {
+    const int d = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
+    if (h >= N + Nk) {                               // value head: plain copy into the cache row
+        const int kvh = h - N - Nk;
+        int64_t r = *v_row;
+        r = r < 0 ? 0 : (r >= v_rows ? v_rows - 1 : r);
+        const uint16_t* src = v_lin + (static_cast<size_t>(b) * Nk + kvh) * kHeadDim;
+        uint16_t* dst = v_dst + ((static_cast<size_t>(b) * Nk + kvh) * v_rows + r) * kHeadDim;
+        dst[d] = src[d];
+        dst[d + kPairs] = src[d + kPairs];
+        return;
+    }
+    int64_t p = *pos;
+    p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);
+    const float c1 = lo2f<T>(cos_tab[p * kHeadDim + d]), c2 = lo2f<T>(cos_tab[p * kHeadDim + kPairs + d]);
+    const float s1 = lo2f<T>(sin_tab[p * kHeadDim + d]), s2 = lo2f<T>(sin_tab[p * kHeadDim + kPairs + d]);
+    const bool is_q = h < N;
+    const uint16_t* src = is_q ? q_lin + (static_cast<size_t>(b) * N + h) * kHeadDim
+                               : k_lin + (static_cast<size_t>(b) * Nk + (h - N)) * kHeadDim;
+    const float x1 = lo2f<T>(src[d]), x2 = lo2f<T>(src[d + kPairs]);
+    // (x * cos) + (rotate_half(x) * sin), rotate_half(x) = cat(-x2, x1)
+    const float o1 = rnd_a<T>(rnd_a<T>(x1 * c1) + rnd_a<T>(-x2 * s1));
+    const float o2 = rnd_a<T>(rnd_a<T>(x2 * c2) + rnd_a<T>(x1 * s2));
+    uint16_t* dst;
+    if (is_q) {
+        dst = q_out + (static_cast<size_t>(b) * N + h) * kHeadDim;
+    } else {
+        int64_t r = *k_row;
+        r = r < 0 ? 0 : (r >= k_rows ? k_rows - 1 : r);
+        dst = k_dst + ((static_cast<size_t>(b) * Nk + (h - N)) * k_rows + r) * kHeadDim;
+    }
+    dst[d] = f2lo<T>(o1);
+    dst[d + kPairs] = f2lo<T>(o2);
+}
+
+// One 256-thread block per row of `hidden` elements (hidden % 8 == 0).
+//   s = x (+ res, rounded to the dtype; written to sum_out if given)
+//   y = w * dtype( float(s) * rsqrt(mean(float(s)^2) + eps) )
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ res,
+                                                       const uint16_t* __restrict__ w, uint16_t* __restrict__ y,
+                                                       uint16_t* __restrict__ sum_out, int hidden, float eps) {
+    __shared__ float part[4];
+    const size_t row = static_cast<size_t>(blockIdx.x) * hidden;
+    float ss = 0.0f;
+    for (int i = threadIdx.x * 8; i < hidden; i += 256 * 8) {
+        const uint4 xv = *reinterpret_cast<const uint4*>(x + row + i);
+        uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+        if (res) {
+            const uint4 rv = *reinterpret_cast<const uint4*>(res + row + i);
+            const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint16_t lo = f2lo<T>(lo2f<T>(static_cast<uint16_t>(xw[j] & 0xffffu)) + lo2f<T>(static_cast<uint16_t>(rw[j] & 0xffffu)));
+                const uint16_t hi = f2lo<T>(lo2f<T>(static_cast<uint16_t>(xw[j] >> 16)) + lo2f<T>(static_cast<uint16_t>(rw[j] >> 16)));
+                xw[j] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+            }
+            if (sum_out) *reinterpret_cast<uint4*>(sum_out + row + i) = make_uint4(xw[0], xw[1], xw[2], xw[3]);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float a = lo2f<T>(static_cast<uint16_t>(xw[j] & 0xffffu)), c = lo2f<T>(static_cast<uint16_t>(xw[j] >> 16));
+            ss = __builtin_fmaf(a, a, ss);
+            ss = __builtin_fmaf(c, c, ss);
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / static_cast<float>(hidden) + eps);
+    const uint16_t* src = (res && sum_out) ? sum_out : nullptr;
+    for (int i = threadIdx.x * 8; i < hidden; i += 256 * 8) {
+        uint32_t xw[4];
+        if (src) {                                   // re-read the rounded sums this thread wrote
+            const uint4 sv = *reinterpret_cast<const uint4*>(src + row + i);
+            xw[0] = sv.x; xw[1] = sv.y; xw[2] = sv.z; xw[3] = sv.w;
+        } else {
+            const uint4 xv = *reinterpret_cast<const uint4*>(x + row + i);
+            xw[0] = xv.x; xw[1] = xv.y; xw[2] = xv.z; xw[3] = xv.w;
+            if (res) {
+                const uint4 rv = *reinterpret_cast<const uint4*>(res + row + i);
+                const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint16_t lo = f2lo<T>(lo2f<T>(static_cast<uint16_t>(xw[j] & 0xffffu)) + lo2f<T>(static_cast<uint16_t>(rw[j] & 0xffffu)));
+                    const uint16_t hi = f2lo<T>(lo2f<T>(static_cast<uint16_t>(xw[j] >> 16)) + lo2f<T>(static_cast<uint16_t>(rw[j] >> 16)));
+                    xw[j] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+                }
+            }
+        }
+        const uint4 wv = *reinterpret_cast<const uint4*>(w + i);
+        const uint32_t ww[4] = {wv.x, wv.y, wv.z, wv.w};
+        uint32_t yo[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float a = rnd_a<T>(lo2f<T>(static_cast<uint16_t>(xw[j] & 0xffffu)) * inv);
+            const float c = rnd_a<T>(lo2f<T>(static_cast<uint16_t>(xw[j] >> 16)) * inv);
+            const uint16_t lo = f2lo<T>(lo2f<T>(static_cast<uint16_t>(ww[j] & 0xffffu)) * a);
+            const uint16_t hi = f2lo<T>(lo2f<T>(static_cast<uint16_t>(ww[j] >> 16)) * c);
+            yo[j] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+        }
+        *reinterpret_cast<uint4*>(y + row + i) = make_uint4(yo[0], yo[1], yo[2], yo[3]);
+    }
+}
+
+// y = dtype(silu(gate)) * up, elementwise over n elements (n % 8 == 0); silu(x) = x / (1 + exp(-x)) in fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
+                                                        uint16_t* __restrict__ y, size_t n) {
+    const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
+    if (i >= n) return;
+    const uint4 gv = *reinterpret_cast<const uint4*>(gate + i), uv = *reinterpret_cast<const uint4*>(up + i);
+    const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+    uint32_t yo[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float g0 = lo2f<T>(static_cast<uint16_t>(gw[j] & 0xffffu)), g1 = lo2f<T>(static_cast<uint16_t>(gw[j] >> 16));
+        const float a0 = rnd_a<T>(g0 / (1.0f + __expf(-g0))), a1 = rnd_a<T>(g1 / (1.0f + __expf(-g1)));
+        const uint16_t lo = f2lo<T>(a0 * lo2f<T>(static_cast<uint16_t>(uw[j] & 0xffffu)));
+        const uint16_t hi = f2lo<T>(a1 * lo2f<T>(static_cast<uint16_t>(uw[j] >> 16)));
+        yo[j] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+    }
+    *reinterpret_cast<uint4*>(y + i) = make_uint4(yo[0], yo[1], yo[2], yo[3]);
+}
+
+int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_tab, const void* sin_tab,
+                       const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
+                       void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int64_t max_pos, int dtype,
+                       hipStream_t st) {
+    dim3 grid(N + 2 * Nk, B), block(kWave);
+#define PQ_RA(T)                                                                                                     \
+    hipLaunchKernelGGL(rope_append_kernel<T>, grid, block, 0, st, (const uint16_t*)q_lin, (const uint16_t*)k_lin,    \
+                       (const uint16_t*)v_lin, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, pos,              \
+                       (uint16_t*)q_out, (uint16_t*)k_dst, k_rows, k_row, (uint16_t*)v_dst, v_rows, v_row, N, Nk, max_pos)
+    if (dtype == 0) PQ_RA(F16); else PQ_RA(BF16);
+#undef PQ_RA
+    return static_cast<int>(hipGetLastError());
+}
+
+int launch_rmsnorm(const void* x, const void* res, const void* w, void* y, void* sum_out, int rows, int hidden, float eps,
+                   int dtype, hipStream_t st) {
+    if (dtype == 0)
+        hipLaunchKernelGGL(rmsnorm_kernel<F16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x, (const uint16_t*)res,
+                           (const uint16_t*)w, (uint16_t*)y, (uint16_t*)sum_out, hidden, eps);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<BF16>, dim3(rows), dim3(256), 0, st, (const uint16_t*)x, (const uint16_t*)res,
+                           (const uint16_t*)w, (uint16_t*)y, (uint16_t*)sum_out, hidden, eps);
+    return static_cast<int>(hipGetLastError());
+}
+
+int launch_silu_mul(const void* gate, const void* up, void* y, size_t n, int dtype, hipStream_t st) {
+    const unsigned blocks = static_cast<unsigned>((n / 8 + 255) / 256);
+    if (dtype == 0)
+        hipLaunchKernelGGL(silu_mul_kernel<F16>, dim3(blocks), dim3(256), 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, n);
+    else
+        hipLaunchKernelGGL(silu_mul_kernel<BF16>, dim3(blocks), dim3(256), 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, n);
+    return static_cast<int>(hipGetLastError());
+}
+
+}  // namespace pq

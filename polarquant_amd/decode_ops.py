@@ -1,0 +1,71 @@
+"""Fused elementwise steps of one decode layer (HIP): RoPE + cache append, residual add + RMS norm,
+SiLU * up.  Each replaces a chain of 8-12 eager launches on a [B, 1, hidden] activation
+(reference: models/modeling_llama_polar.py:47-59,77,98 and the decoder layer :456-486)."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _ffi
+from .kernel4group import _dtype_code, _stream_ptr
+
+
+def _gpu(t: torch.Tensor):
+    if not t.is_cuda:
+        raise RuntimeError("polarquant_amd: the fused decode ops need tensors on the GPU (no CPU fallback)")
+
+
+def rope_append(q_lin: torch.Tensor, k_lin: torch.Tensor, v_lin: torch.Tensor, cos_table: torch.Tensor,
+                sin_table: torch.Tensor, pos: torch.Tensor, k_dst: torch.Tensor, k_row: torch.Tensor,
+                v_dst: torch.Tensor, v_row: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
+    """q_lin [B,1,N*128], k_lin / v_lin [B,1,Nk*128] (projection outputs of the new token);
+    cos/sin tables [rows,128]; pos, k_row, v_row: int64 tensors of one element on the device.
+    Writes the rotated key into k_dst[:, :, k_row] and the value into v_dst[:, :, v_row]
+    ([B,Nk,rows,128] each); returns the rotated query [B,N,1,128]."""
+    _gpu(q_lin)
+    B = q_lin.shape[0]
+    assert q_lin.is_contiguous() and k_lin.is_contiguous() and v_lin.is_contiguous()
+    assert k_dst.is_contiguous() and v_dst.is_contiguous() and cos_table.is_contiguous() and sin_table.is_contiguous()
+    assert pos.dtype == k_row.dtype == v_row.dtype == torch.int64
+    assert q_lin.numel() == B * n_heads * 128 and k_lin.numel() == B * n_kv_heads * 128 == v_lin.numel()
+    assert k_dst.shape[:2] == (B, n_kv_heads) == v_dst.shape[:2] and k_dst.shape[3] == 128 == v_dst.shape[3]
+    q_out = torch.empty((B, n_heads, 1, 128), dtype=q_lin.dtype, device=q_lin.device)
+    with torch.cuda.device(q_lin.device):
+        rc = _ffi.lib().pq_rope_append(q_lin.data_ptr(), k_lin.data_ptr(), v_lin.data_ptr(), cos_table.data_ptr(),
+                                       sin_table.data_ptr(), cos_table.shape[0], pos.data_ptr(), q_out.data_ptr(),
+                                       k_dst.data_ptr(), k_dst.shape[2], k_row.data_ptr(), v_dst.data_ptr(), v_dst.shape[2],
+                                       v_row.data_ptr(), B, n_heads, n_kv_heads, _dtype_code(q_lin), _stream_ptr(q_lin.device))
+    _ffi.check(rc, "pq_rope_append")
+    return q_out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None,
+            sum_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """weight * rms_norm(x), or of x + residual (the sum, rounded to the dtype, goes to sum_out,
+    which may be x itself)."""
+    _gpu(x)
+    hidden = x.shape[-1]
+    assert x.is_contiguous() and weight.is_contiguous() and weight.dtype == x.dtype and weight.numel() == hidden
+    if residual is not None:
+        assert residual.is_contiguous() and residual.shape == x.shape and residual.dtype == x.dtype
+    if sum_out is not None:
+        assert sum_out.is_contiguous() and sum_out.shape == x.shape and sum_out.dtype == x.dtype
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _ffi.lib().pq_rmsnorm(x.data_ptr(), None if residual is None else residual.data_ptr(), weight.data_ptr(),
+                                   y.data_ptr(), None if sum_out is None else sum_out.data_ptr(), x.numel() // hidden, hidden,
+                                   float(eps), _dtype_code(x), _stream_ptr(x.device))
+    _ffi.check(rc, "pq_rmsnorm")
+    return y
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    _gpu(gate)
+    assert gate.is_contiguous() and up.is_contiguous() and gate.shape == up.shape and gate.dtype == up.dtype
+    y = torch.empty_like(gate)
+    with torch.cuda.device(gate.device):
+        rc = _ffi.lib().pq_silu_mul(gate.data_ptr(), up.data_ptr(), y.data_ptr(), gate.numel(), _dtype_code(gate),
+                                    _stream_ptr(gate.device))
+    _ffi.check(rc, "pq_silu_mul")
+    return y

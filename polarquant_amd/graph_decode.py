@@ -28,7 +28,11 @@ from .modeling_common import GROUP, apply_rotary_pos_emb
 
 
 class PolarGraphDecoder:
-    def __init__(self, model, max_len: int, use_graph: bool = True):
+    def __init__(self, model, max_len: int, use_graph: bool = True, fused_ops: bool = True):
+        """fused_ops: run RoPE + cache append, the norms and the MLP activation as one HIP launch each
+        (polarquant_amd.decode_ops) instead of the eager modules' chains of elementwise launches.  The
+        rotation is bit-identical to the eager ops; the norms and SiLU agree to the dtype's last bit."""
+        self.fused_ops = fused_ops
         self.model = model
         self.cfg = model.config
         self.max_len = int(max_len)
@@ -77,8 +81,44 @@ class PolarGraphDecoder:
         return out.logits
 
     # ------------------------------------------------------------------ one token
+    def _attend(self, att, ar, q):
+        common = dict(rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
+                      n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits)
+        if self.mixed:
+            return polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0, **common)
+        return polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, **common)
+
+    def _step_body_fused(self):
+        """The decode step with one launch per elementwise stage: 2 norms (each with the residual add
+        folded in), RoPE + append, SiLU * up, plus the GEMMs and the attention, per layer."""
+        from .decode_ops import rmsnorm, rope_append, silu_mul
+        model, B = self.model, self.B
+        layers = model.model.layers
+        x = model.model.embed_tokens(self.ids).contiguous()                 # residual stream [B,1,H], updated in place
+        h = rmsnorm(x, layers[0].input_layernorm.weight, layers[0].input_layernorm.variance_epsilon)
+        for li, (layer, ar) in enumerate(zip(layers, self.arenas)):
+            att, mlp = layer.self_attn, layer.mlp
+            q_lin, k_lin, v_lin = att.q_proj(h), att.k_proj(h), att.v_proj(h)
+            v_dst, v_row = (ar.vres, self.resid_idx) if self.mixed else (ar.v, self.pos)
+            q = rope_append(q_lin, k_lin, v_lin, self.cos_table, self.sin_table, self.pos, ar.kres, self.resid_idx,
+                            v_dst, v_row, att.num_heads, att.num_key_value_heads)
+            o = self._attend(att, ar, q)
+            a = att.o_proj(o.reshape(B, 1, -1))
+            pn = layer.post_attention_layernorm
+            h = rmsnorm(x, pn.weight, pn.variance_epsilon, residual=a, sum_out=x)
+            m = mlp.down_proj(silu_mul(mlp.gate_proj(h), mlp.up_proj(h)))
+            nn_ = layers[li + 1].input_layernorm if li + 1 < len(layers) else model.model.norm
+            h = rmsnorm(x, nn_.weight, nn_.variance_epsilon, residual=m, sum_out=x)
+        logits = model.lm_head(h)
+        self.pos.add_(1)
+        self.resid_idx.add_(1)
+        self.n_resid_dev.add_(1)
+        return logits
+
     def _step_body(self):
         """The decode step on the static state; identical arithmetic to the eager modules."""
+        if self.fused_ops:
+            return self._step_body_fused()
         model = self.model
         x = model.model.embed_tokens(self.ids)
         cos = self.cos_table.index_select(0, self.pos).unsqueeze(0)        # [1,1,128]

@@ -1,0 +1,93 @@
+"""The fused elementwise kernels of the decode step against the eager torch ops they replace
+(HF apply_rotary_pos_emb + cache writes, residual add + RMSNorm, SiLU * up)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from polarquant_amd.decode_ops import rmsnorm, rope_append, silu_mul
+from polarquant_amd.modeling_common import RMSNorm, apply_rotary_pos_emb
+
+pytestmark = pytest.mark.gpu
+
+
+def _ulps_off(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """Largest |got - ref| in units of the dtype's spacing at |ref|."""
+    return float(((got.float() - ref.float()).abs() / _ulp(ref)).max())
+
+
+def _ulp(ref: torch.Tensor) -> torch.Tensor:
+    """Spacing of the dtype at |ref| (as float)."""
+    bits = 10 if ref.dtype == torch.float16 else 7
+    mag = ref.float().abs().clamp_min(2.0 ** -14)
+    return torch.exp2(torch.floor(torch.log2(mag)) - bits)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N,Nk", [(8, 2), (7, 1), (4, 4)])
+def test_rope_append_is_bit_identical_to_the_eager_ops(gpu, dtype, N, Nk):
+    torch.manual_seed(N * 10 + Nk)
+    B, rows, max_pos = 3, 128, 700
+    inv = 1.0 / (5e5 ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * inv[None]
+    emb = torch.cat([ang, ang], -1)
+    cos_t, sin_t = emb.cos().to(dtype).to(gpu), emb.sin().to(dtype).to(gpu)
+    q_lin = torch.randn(B, 1, N * 128, device=gpu).to(dtype)
+    k_lin = torch.randn(B, 1, Nk * 128, device=gpu).to(dtype)
+    v_lin = torch.randn(B, 1, Nk * 128, device=gpu).to(dtype)
+    for p, kr in [(0, 0), (321, 65), (699, 127)]:
+        pos = torch.tensor([p], dtype=torch.int64, device=gpu)
+        k_row = torch.tensor([kr], dtype=torch.int64, device=gpu)
+        k_dst = torch.full((B, Nk, rows, 128), 7.0, dtype=dtype, device=gpu)
+        v_dst = torch.full((B, Nk, max_pos, 128), 7.0, dtype=dtype, device=gpu)
+        q = rope_append(q_lin, k_lin, v_lin, cos_t, sin_t, pos, k_dst, k_row, v_dst, pos, N, Nk)
+        # the eager chain (reference :50-59, :77, :98)
+        qe = q_lin.view(B, 1, N, 128).transpose(1, 2)
+        ke = k_lin.view(B, 1, Nk, 128).transpose(1, 2)
+        ve = v_lin.view(B, 1, Nk, 128).transpose(1, 2)
+        qr, kr_ = apply_rotary_pos_emb(qe, ke, cos_t[p:p + 1][None], sin_t[p:p + 1][None])
+        assert q.shape == (B, N, 1, 128) and torch.equal(q, qr)
+        assert torch.equal(k_dst[:, :, kr], kr_[:, :, 0]) and torch.equal(v_dst[:, :, p], ve[:, :, 0])
+        k_dst[:, :, kr] = 7.0
+        v_dst[:, :, p] = 7.0
+        assert bool((k_dst == 7.0).all()) and bool((v_dst == 7.0).all())     # nothing else was touched
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [512, 4096, 3584])
+def test_rmsnorm_matches_module(gpu, dtype, hidden):
+    torch.manual_seed(hidden)
+    mod = RMSNorm(hidden, 1e-5).to(dtype).to(gpu)
+    with torch.no_grad():
+        mod.weight.copy_((1 + 0.1 * torch.randn(hidden)).to(dtype))
+    x = (torch.randn(5, 1, hidden, device=gpu) * 3).to(dtype)
+    res = torch.randn(5, 1, hidden, device=gpu).to(dtype)
+    with torch.no_grad():
+        ref = mod(x)
+        got = rmsnorm(x, mod.weight, mod.variance_epsilon)
+        # w * dtype(x * inv): a last-bit difference of the fp32 inv can move the inner rounding by one
+        # step, which the multiplication by w can turn into two steps of the result
+        assert _ulps_off(got, ref) <= 2, _ulps_off(got, ref)
+        assert (got != ref).float().mean().item() < 0.05                    # and such differences are rare
+        s_ref = x + res
+        ref2 = mod(s_ref)
+        s = torch.empty_like(x)
+        got2 = rmsnorm(x, mod.weight, mod.variance_epsilon, residual=res, sum_out=s)
+        assert torch.equal(s, s_ref)
+        assert _ulps_off(got2, ref2) <= 2, _ulps_off(got2, ref2)
+        assert (got2 != ref2).float().mean().item() < 0.05
+        xin = x.clone()
+        got3 = rmsnorm(xin, mod.weight, mod.variance_epsilon, residual=res, sum_out=xin)      # in place
+        assert torch.equal(xin, s_ref) and torch.equal(got3, got2)
+        got4 = rmsnorm(x, mod.weight, mod.variance_epsilon, residual=res)                   # sum not wanted
+        assert torch.equal(got4, got2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_silu_mul_matches_eager(gpu, dtype):
+    torch.manual_seed(1)
+    g = (torch.randn(4, 1, 14336, device=gpu) * 3).to(dtype)
+    u = torch.randn(4, 1, 14336, device=gpu).to(dtype)
+    ref = F.silu(g) * u
+    got = silu_mul(g, u)
+    assert _ulps_off(got, ref) <= 2, _ulps_off(got, ref)
+    assert (got != ref).float().mean().item() < 0.05
