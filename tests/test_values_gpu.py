@@ -157,3 +157,52 @@ def test_attention_v4_peaked_softmax_keeps_code_and_zero_point_terms_consistent(
         err = (out.double() - ref64).abs().max().item()
         print("peaked, n_splits", ns, "max abs err %.2e (|out| up to %.2f)" % (err, ref64.abs().max().item()), flush=True)
         assert err < 1.5e-3 * max(1.0, ref64.abs().max().item()), (ns, err)
+
+
+def test_attention_v4_ragged_batch_matches_per_sequence_oracle(gpu):
+    """Per-sequence group / residual counts (device arrays) with 4-bit values: every sequence must
+    equal the oracle run on that sequence alone, including one with no quantized group and one
+    with a full residual window; rows past a sequence's fill hold NaN and must not contribute."""
+    g = torch.Generator().manual_seed(41)
+    B, N, Nk, cap = 5, 8, 2, 6
+    groups = [0, 1, 6, 3, 2]
+    resid = [7, 128, 1, 64, 33]
+    q = wl.make_half((B, N, 1, 128), g)
+    codes = torch.zeros(B, Nk, cap, 128, 64, dtype=torch.uint8)
+    meta = [torch.full((B, Nk, cap, 1, 64), float("nan"), dtype=torch.float16) for _ in range(4)]
+    vcodes = torch.full((B, Nk, cap * 128, 16), -1, dtype=torch.int32)
+    vmeta = [torch.full((B, Nk, cap * 128, 1), float("nan"), dtype=torch.float16) for _ in range(2)]
+    kres = torch.full((B, Nk, 128, 128), float("nan"), dtype=torch.float16)
+    vres = torch.full((B, Nk, 128, 128), float("nan"), dtype=torch.float16)
+    mask = torch.ones(B, cap * 128 + 128, dtype=torch.uint8)
+    refs = []
+    for b in range(B):
+        nb, nr = groups[b], resid[b]
+        L = nb * 128 + nr
+        k = wl.make_keys(1, Nk, L, 1e6, g)
+        v = wl.make_half((1, Nk, L, 128), g)
+        quant, vq = (None,) * 5, (None,) * 3
+        if nb:
+            quant = po.quantize_and_pack_nbit(k[:, :, :nb * 128].contiguous())
+            vq = po.quantize_values_along_last_dim(v[:, :, :nb * 128].contiguous())
+            codes[b, :, :nb] = quant[0][0]
+            for m, t in zip(meta, quant[1:]):
+                m[b, :, :nb] = t[0]
+            vcodes[b, :, :nb * 128] = vq[0][0]
+            for m, t in zip(vmeta, vq[1:]):
+                m[b, :, :nb * 128] = t[0]
+        kres[b, :, :nr], vres[b, :, :nr] = k[0, :, nb * 128:], v[0, :, nb * 128:]
+        mb = torch.ones(1, L, dtype=torch.int64)
+        mb[0, :min(5 * b, L - 1)] = 0
+        mask[b, :L] = mb[0]
+        refs.append(po.decode_attention_mixed_exact(q[b:b + 1], k[:, :, nb * 128:], *quant, v[:, :, nb * 128:], *vq, mb))
+    dev = lambda t: t.to(gpu)
+    for kw in (dict(), dict(n_splits=3), dict(n_splits=6, min_groups_per_split=2)):
+        out = polar_decode_attention_v4(dev(q), dev(codes), *[dev(m) for m in meta], dev(kres), dev(vres), dev(vcodes),
+                                        *[dev(m) for m in vmeta], 0, 0, attention_mask=dev(mask),
+                                        n_groups_per_seq=torch.tensor(groups, dtype=torch.int32, device=gpu),
+                                        n_resid_per_seq=torch.tensor(resid, dtype=torch.int32, device=gpu), **kw).cpu()
+        assert torch.isfinite(out.float()).all()
+        for b in range(B):
+            nbad, emax = _close(out[b:b + 1], refs[b])
+            assert nbad == 0, (kw, b, nbad, emax)
