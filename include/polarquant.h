@@ -161,6 +161,8 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *            ceil(groups / n_splits)) always covers the sequence.
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
+ * Limits: v_capacity <= 2^24 tokens and group_capacity <= 2^17 groups per (batch, KV head)
+ * plane (32-bit byte offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */
 int pq_decode_attn(const void *q,
                    const uint8_t *codes, const void *rscale, const void *rmn,

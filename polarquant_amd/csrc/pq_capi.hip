@@ -156,6 +156,9 @@ int pq_validate_decode_attn(const void* q,
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
     if (group_capacity < 0 || resid_capacity < 0 || n_groups < 0 || n_resid < 0 || v_capacity <= 0)
         return PQ_ERR_BAD_STRIDE;
+    // the kernels address one (batch, KV head) plane with 32-bit byte offsets: at most 2^24 tokens
+    // of 256-byte value rows (and 2^17 groups of 8 KiB of codes) per plane
+    if (v_capacity > (int64_t{1} << 24) || group_capacity > (1 << 17) || resid_capacity > (1 << 24)) return PQ_ERR_BAD_SHAPE;
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     if (any_groups && (!codes || !rscale || !rmn || !tscale || !tmn)) return PQ_ERR_NULL_POINTER;
     const bool any_resid = n_resid_per_seq ? resid_capacity > 0 : n_resid > 0;
@@ -331,6 +334,7 @@ int pq_validate_decode_attn_v4(const void* q,
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     if (any_groups && (!v_codes || !v_scale || !v_zero)) return PQ_ERR_NULL_POINTER;
     if (v4_capacity < 0) return PQ_ERR_BAD_STRIDE;
+    if (v4_capacity > (int64_t{1} << 24)) return PQ_ERR_BAD_SHAPE;          // 32-bit byte offsets inside a plane
     if (!n_groups_per_seq && static_cast<int64_t>(n_groups) * PQ_GROUP > v4_capacity) return PQ_ERR_BAD_STRIDE;
     if ((v_codes && !aligned(v_codes, 4)) || (v_resid && !aligned(v_resid, 16))) return PQ_ERR_MISALIGNED;
     // everything else as in the fp16-value entry point; its V-capacity rule is met by construction here

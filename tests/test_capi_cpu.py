@@ -105,6 +105,7 @@ def test_validate_decode_attn_and_plan(lib):
     assert bad(24, 0) == -7 and bad(27, wsb - 1) == -7 and bad(25, -1) == -7
     assert bad(20, 5) == -2 and bad(22, 5) == -3 and bad(23, 3) == -4
     assert bad(13, P + 8) == -5
+    assert bad(14, (1 << 24) + 1) == -2 and bad(6, (1 << 17) + 1) == -2      # plane too large for 32-bit offsets
     a = list(ok); a[15] = P; a[16] = 100          # mask row shorter than the context
     assert lib.pq_validate_decode_attn(*a) == -6
     # no quantized groups yet: codes may be NULL
