@@ -103,16 +103,17 @@ __device__ __forceinline__ void angle_radius_exact(float x, float y, float* phi,
     *rad = rnd<T>(__fsqrt_rn(__builtin_fmaf(x, x, y * y)));
 }
 
+// floor(dtype((v - mn) / scale)) clamped to [0, top] (:148, :153).  `topf` is the clamp bound as a
+// float, or 0 for a degenerate pair (scale == 0 or NaN: x/0 and 0/0 are undefined in the reference
+// and defined as code 0 here).  v_med3_f32 returns the minimum of its operands when one is NaN, so
+// a NaN quotient also comes out as 0 without a separate test.
 template <typename T>
-__device__ __forceinline__ uint32_t code_of(float v, float mn, float scale, int top) {
+__device__ __forceinline__ uint32_t code_of(float v, float mn, float scale, float topf) {
     const float d = rnd<T>(v - mn);
-    float qf = rnd<T>(d / scale);
-    qf = floorf(qf);
-    if (!math::isfinite_(qf)) return 0u;   // 0/0 or x/0: undefined in the reference, 0 here
-    qf = fminf(fmaxf(qf, 0.0f), 255.0f);
-    const uint32_t c = static_cast<uint32_t>(qf);
-    return c > static_cast<uint32_t>(top) ? static_cast<uint32_t>(top) : c;
+    const float qf = floorf(rnd<T>(d / scale));
+    return static_cast<uint32_t>(__builtin_amdgcn_fmed3f(qf, 0.0f, topf));
 }
+__device__ __forceinline__ float clamp_bound(float scale, int top) { return scale > 0.0f ? static_cast<float>(top) : 0.0f; }
 
 constexpr int kQThreads = 256;
 constexpr int kTokPerThread = kGroup / 16;   // 8
@@ -158,7 +159,7 @@ __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const An
     float phi = rnd<T>(a);
     uint32_t aw;
     if constexpr (UNIFORM) {
-        aw = code_of<T>(phi, am.tmn, am.tscale, am.ttop);
+        aw = code_of<T>(phi, am.tmn, am.tscale, static_cast<float>(am.ttop));
     } else {
         if (phi < 0.0f) phi = rnd<T>(phi + am.two_pi);             // :144
         aw = f2lo<T>(phi);
@@ -269,7 +270,12 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         *reinterpret_cast<uint2*>(rmn + mi) = pack4(rm);
     }
     // ---- pass 2: codes
-    const int ttop = (1 << tbits) - 1, rtop = (1 << rbits) - 1;
+    float ttop[4], rtop[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ttop[i] = clamp_bound(ts[i], (1 << tbits) - 1);
+        rtop[i] = clamp_bound(rs[i], (1 << rbits) - 1);
+    }
     uint8_t* cb = codes + plane * (kGroup * kPairs);
 #pragma unroll
     for (int it = 0; it < kTokPerThread; it++) {
@@ -279,8 +285,8 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
             const uint32_t v = pr[it * 4 + i][tid];
             const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
             const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
-            const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop);    // :148
-            const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop);      // :153
+            const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop[i]);    // :148
+            const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop[i]);      // :153
             w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
         }
         *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPairs + 4 * pq4) = w;
