@@ -37,6 +37,12 @@ the checks live in tests/test_oracle_pins.py):
                            packed int32 and the rounding mode are taken from the
                            published KIVI source, which nothing in the reference
                            tree confirms.
+  snapkv_scores / snapkv_select / prefill_cache_snapkv (SnapKV prompt eviction in
+                           front of the polar cache): compositions of torch library
+                           routines (matmul, softmax, avg_pool1d, topk, gather), the
+                           literal reference lines; pinned by a hand-built prompt whose
+                           heavy keys are known, by permutation invariance of the kept
+                           set, and by bookkeeping properties.
   Degenerate groups (tscale==0 or rscale==0 -> 0/0) are undefined behaviour in
   the reference (NaN -> uint8); this oracle defines the code as 0 there, which
   is what torch-CPU's cast yields.  That choice is "parity unpinned".
@@ -287,6 +293,62 @@ def decode_step(query_states, key_states, value_states, past_key_value, attentio
         ind, rs, rm, ts, tm = cat(ind, i2), cat(rs, rs2), cat(rm, rm2), cat(ts, ts2), cat(tm, tm2)
         k_full = None
     return out, (k_full, ind, rs, rm, ts, tm, v_full, kv_len + 1)
+
+
+# --------------------------------------------------------------------------
+# SnapKV prompt eviction in front of the polar cache (LlamaSnapKVAttention,
+# models/modeling_llama_polar.py:295-443).  Decode is the plain polar decode step
+# (:343-388, no mask, batch 1); only the prompt pass differs.
+# --------------------------------------------------------------------------
+def snapkv_scores(query_states, key_states, window_size: int = 128, kernel_size: int = 7):
+    """Pooled attention mass the last `window_size` queries put on each earlier key (:398-410)
+    -> [B, Nk, L - window_size] in the query dtype.  query [B,N,L,128], key [B,Nk,L,128]."""
+    B, N, L, hd = query_states.shape
+    Nk = key_states.shape[1]
+    rep = N // Nk
+    w = torch.matmul(query_states[:, :, -window_size:, :], repeat_kv(key_states, rep).transpose(2, 3))           # :398 (no 1/sqrt(d))
+    mask = torch.full((window_size, window_size), torch.finfo(w.dtype).min)
+    cond = torch.arange(window_size)
+    mask.masked_fill_(cond < (cond + 1).view(window_size, 1), 0)                                                # :399-401
+    w[:, :, -window_size:, -window_size:] += mask[None, None].to(w.dtype)                                       # :405
+    w = torch.softmax(w, dim=-1, dtype=torch.float32).to(query_states.dtype)                                    # :407
+    s = w[:, :, -window_size:, :-window_size].sum(dim=-2)                                                       # :408
+    pooled = torch.nn.functional.avg_pool1d(s, kernel_size=kernel_size, padding=kernel_size // 2, stride=1)     # :410
+    return pooled.view(B, Nk, rep, -1).mean(dim=2)                                                              # :412
+
+
+def snapkv_select(query_states, key_states, window_size: int = 128, kernel_size: int = 7,
+                  max_capacity_prompt: int = 1024 + 128) -> torch.Tensor:
+    """-> indices [B, Nk, max_capacity_prompt - window_size] of the kept earlier tokens (:414)."""
+    return snapkv_scores(query_states, key_states, window_size, kernel_size).topk(max_capacity_prompt - window_size, dim=-1).indices
+
+
+def prefill_cache_snapkv(query_states, key_states, value_states, rbits=4, tbits=4, window_size=128, kernel_size=7,
+                         max_capacity_prompt=1024 + 128, residual_length=GROUP_SIZE, indices=None):
+    """Prompt q/k/v -> the 8-tuple LlamaSnapKVAttention leaves (:392-441): when the prompt is longer
+    than max_capacity_prompt only the selected earlier tokens and the last window are cached, and the
+    tuple's last slot still holds the FULL prompt length (positions continue from there).
+    `indices` overrides the selection (tests pass the product's own, to compare caches exactly)."""
+    L = key_states.shape[2]
+    if L > max_capacity_prompt:
+        if indices is None:
+            indices = snapkv_select(query_states, key_states, window_size, kernel_size, max_capacity_prompt)
+        idx = indices.unsqueeze(-1).expand(-1, -1, -1, key_states.shape[-1])
+        k_past = key_states[:, :, :-window_size, :].gather(dim=2, index=idx)                                    # :417
+        v_past = value_states[:, :, :-window_size, :].gather(dim=2, index=idx)
+        key_states = torch.cat([k_past, key_states[:, :, -window_size:, :]], dim=2)                            # :420
+        value_states = torch.cat([v_past, value_states[:, :, -window_size:, :]], dim=2)
+    kept = key_states.shape[2]
+    r = kept % residual_length                                                                                  # :426
+    if r == 0:
+        k_full, k_quant = None, key_states
+    else:
+        k_full = key_states if L < residual_length else key_states[:, :, -r:, :]                               # :431 tests the FULL length
+        k_quant = None if L < residual_length else key_states[:, :, :-r, :]
+    ind = rs = rm = ts = tm = None
+    if k_quant is not None:
+        ind, rs, rm, ts, tm = quantize_and_pack_nbit(k_quant.contiguous(), rbits, tbits, residual_length)
+    return (k_full, ind, rs, rm, ts, tm, value_states, L)
 
 
 # --------------------------------------------------------------------------

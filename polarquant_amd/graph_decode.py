@@ -57,6 +57,7 @@ class PolarGraphDecoder:
             cfg.cache_capacity = old
         self.arenas = [c.arena for c in out.past_key_values]
         a0 = self.arenas[0]
+        assert a0.pos_offset == 0, "prompt eviction (SnapKV) is not handled by the graph decoder"
         self.B, self.kv_len, self.n_resid = B, a0.kv_len, a0.n_resid
         dtype = a0.dtype
         # device-side step state

@@ -57,6 +57,7 @@ class PolarConfig:
     rbits: int = 4
     tbits: int = 4
     vbits: int = 16                     # 4: values in 4 bits as well (the Mixed variant); 16: half-precision values
+    snapkv: bool = False                # SnapKV prompt eviction in front of the polar cache (batch 1 decode)
     cache_capacity: int = 0             # tokens to pre-allocate per layer (0: prompt + 1024, grown by doubling)
 
     @staticmethod
@@ -152,6 +153,7 @@ class _Arena:
         self.B, self.Nk, self.dtype, self.device = B, Nk, dtype, device
         self.rbits, self.tbits = rbits, tbits
         self.n_groups = self.n_resid = self.kv_len = 0
+        self.pos_offset = 0      # tokens the prompt held beyond the cached ones (SnapKV eviction): tuple[-1] = kv_len + pos_offset
         self.kres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
         self._alloc(max(capacity_tokens, GROUP))
 
@@ -185,7 +187,7 @@ class _Arena:
             q5 = [self.codes[:, :, :self.n_groups]] + [m[:, :, :self.n_groups] for m in self.meta]
         else:
             q5 = [None] * 5
-        return PolarCache((kf, *q5, self.v[:, :, :self.kv_len], self.kv_len), self)
+        return PolarCache((kf, *q5, self.v[:, :, :self.kv_len], self.kv_len + self.pos_offset), self)
 
 
 class PolarCache(tuple):
@@ -244,11 +246,13 @@ class PolarGroupAttention(nn.Module):
 
     def _arena_of(self, past_key_value, dtype, device) -> _Arena:
         arena = getattr(past_key_value, "arena", None)
-        if arena is not None and arena.kv_len == past_key_value[-1]:
+        if arena is not None and arena.kv_len + arena.pos_offset == past_key_value[-1]:
             return arena
         # a plain tuple in the reference's format: copy it into a fresh arena
-        kf, ind, rs, rm, ts, tm, v, n = past_key_value
+        kf, ind, rs, rm, ts, tm, v, seen = past_key_value
+        n = v.shape[2]                       # cached tokens; `seen` may be larger (evicted prompt tokens)
         arena = self._new_arena(v.shape[0], dtype, device, n + 1)
+        arena.pos_offset = seen - n
         if ind is not None:
             g = ind.shape[2]
             arena.codes[:, :, :g] = ind
@@ -357,7 +361,7 @@ class _MixedArena(_Arena):
             v3 = [self.vcodes[:, :, :g * GROUP]] + [m[:, :, :g * GROUP] for m in self.vmeta]
         else:
             q5, v3 = [None] * 5, [None] * 3
-        return PolarCache((kf, *q5, vf, *v3, self.kv_len), self)
+        return PolarCache((kf, *q5, vf, *v3, self.kv_len + self.pos_offset), self)
 
 
 class PolarMixedGroupAttention(PolarGroupAttention):
@@ -376,10 +380,11 @@ class PolarMixedGroupAttention(PolarGroupAttention):
 
     def _arena_of(self, past_key_value, dtype, device) -> _MixedArena:
         arena = getattr(past_key_value, "arena", None)
-        if arena is not None and arena.kv_len == past_key_value[-1]:
+        if arena is not None and arena.kv_len + arena.pos_offset == past_key_value[-1]:
             return arena
         # a plain 11-tuple in the reference's format: copy it into a fresh arena
         kf, ind, rs, rm, ts, tm, vf, vc, vs, vm, n = past_key_value
+        assert n == (0 if ind is None else ind.shape[2] * GROUP) + (0 if kf is None else kf.shape[2])
         B = (kf if kf is not None else ind).shape[0]
         arena = self._new_arena(B, dtype, device, n + 1)
         if ind is not None:
@@ -448,6 +453,74 @@ class PolarMixedGroupAttention(PolarGroupAttention):
         return attn_output, past_key_value
 
 
+# ----------------------------------------------------------------------------- SnapKV prompt eviction + polar cache
+class PolarSnapKVAttention(PolarGroupAttention):
+    """The reference's LlamaSnapKVAttention (models/modeling_llama_polar.py:295-443): prompts longer
+    than max_capacity_prompt keep only the earlier tokens that the last `window_size` queries attend
+    to most (pooled, top-k per KV head) plus that window; the kept keys then go through the usual
+    polar cache.  Decode is the polar decode step without mask, batch 1 (:327).  The selection runs
+    once per prompt with torch ops; the cache and the decode step use the HIP path."""
+
+    def __init__(self, config, layer_idx: Optional[int] = None):
+        super().__init__(config, layer_idx)
+        self.window_size = 128                                             # :298-300
+        self.kernel_size = 7
+        self.max_capacity_prompt = 1024 + self.window_size
+
+    def select(self, query_states, key_states):
+        """-> indices [B, Nk, max_capacity_prompt - window_size] of the earlier tokens to keep (:398-414)."""
+        bsz, ws = query_states.shape[0], self.window_size
+        w = torch.matmul(query_states[:, :, -ws:, :], repeat_kv(key_states, self.num_key_value_groups).transpose(2, 3))
+        mask = torch.full((ws, ws), torch.finfo(w.dtype).min, device=w.device)
+        cond = torch.arange(ws, device=w.device)
+        mask.masked_fill_(cond < (cond + 1).view(ws, 1), 0)
+        w[:, :, -ws:, -ws:] += mask[None, None, :, :].to(w.dtype)
+        w = F.softmax(w, dim=-1, dtype=torch.float32).to(query_states.dtype)
+        s = w[:, :, -ws:, :-ws].sum(dim=-2)
+        pooled = F.avg_pool1d(s, kernel_size=self.kernel_size, padding=self.kernel_size // 2, stride=1)
+        pooled = pooled.view(bsz, self.num_key_value_heads, self.num_key_value_groups, -1).mean(dim=2)
+        return pooled.topk(self.max_capacity_prompt - ws, dim=-1).indices
+
+    def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
+                past_key_value=None, position_embeddings: Tuple[torch.Tensor, torch.Tensor] = None, **kwargs):
+        bsz, q_len, _ = hidden_states.size()
+        if q_len == 1:
+            assert bsz == 1                                                # :327 (no per-sequence mask after eviction)
+            return super().forward(hidden_states, None, past_key_value, position_embeddings, **kwargs)
+        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
+        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
+        cos, sin = position_embeddings
+        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        if self.capture is not None:
+            self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
+        assert past_key_value is None
+        kv_seq_len = key_states.shape[2]
+        attn_output = _prefill_attention(query_states, key_states, value_states, attention_mask,
+                                         self.num_key_value_groups, self.is_causal)
+        self.last_selection = None
+        if kv_seq_len > self.max_capacity_prompt:                          # :396
+            ws = self.window_size
+            idx = self.select(query_states, key_states)
+            self.last_selection = idx
+            idx = idx.unsqueeze(-1).expand(-1, -1, -1, self.head_dim)
+            key_states = torch.cat([key_states[:, :, :-ws, :].gather(dim=2, index=idx), key_states[:, :, -ws:, :]], dim=2)
+            value_states = torch.cat([value_states[:, :, :-ws, :].gather(dim=2, index=idx), value_states[:, :, -ws:, :]], dim=2)
+        kept = key_states.shape[2]
+        arena = self._new_arena(bsz, key_states.dtype, key_states.device, kept + 1)
+        residual_length = kept % self.residual_length                      # :426
+        n_quant = kept - residual_length if kv_seq_len >= self.residual_length else 0
+        if n_quant:
+            arena.quantize_into(key_states[:, :, :n_quant])
+        if kept - n_quant:
+            arena.kres[:, :, :kept - n_quant] = key_states[:, :, n_quant:]
+        arena.n_resid = kept - n_quant
+        arena.v[:, :, :kept] = value_states
+        arena.kv_len, arena.pos_offset = kept, kv_seq_len - kept           # the tuple reports the full prompt length (:441)
+        attn_output = self.o_proj(attn_output.reshape(bsz, q_len, -1).contiguous())
+        return attn_output, arena.as_tuple()
+
+
 def _prefill_attention(q, k, v, attention_mask, n_rep, is_causal):
     """Causal prompt attention; returns [B, L, N, hd] like the reference's flash-attention call (:106-114).
     `attention_mask` [B, L] of {0,1} marks left padding."""
@@ -472,7 +545,8 @@ class CausalLMOutputWithPast:
 
 class PolarDecoderLayer(nn.Module):
     attention_class = PolarGroupAttention
-    mixed_attention_class = None       # set below, once PolarMixedGroupAttention exists in the subclasses' modules
+    mixed_attention_class = None       # subclasses name their own variants; None falls back to the generic classes
+    snapkv_attention_class = None
 
     def __init__(self, config, layer_idx):
         super().__init__()
@@ -482,6 +556,8 @@ class PolarDecoderLayer(nn.Module):
         # modeling_llama_polar.py:452-453); anything else keeps half-precision values
         mixed = _cfg(config, "vbits", 16) == 4
         cls = (self.mixed_attention_class or PolarMixedGroupAttention) if mixed else self.attention_class
+        if _cfg(config, "snapkv", False):       # the reference's third variant (modeling_llama_polar.py:454)
+            cls = self.snapkv_attention_class or PolarSnapKVAttention
         self.self_attn = cls(config, layer_idx)
         self.mlp = MLP(config)
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)

@@ -213,3 +213,72 @@ def test_mixed_attention_forward_matches_reference_restatement(gpu, L):
         o1, c1 = att(x[:, -1:], None, cache, _rope(cfg, L + steps, 1, torch.float16, gpu))
         o2, c2 = att(x[:, -1:], None, plain, _rope(cfg, L + steps, 1, torch.float16, gpu))
     assert torch.equal(o1, o2) and c1[-1] == c2[-1] == L + steps + 1
+
+
+@pytest.mark.parametrize("L", [700, 1400])
+def test_snapkv_attention_matches_reference_restatement(gpu, L):
+    """LlamaSnapKVAttention: prompt eviction (when L > 1152) + polar cache + decode across a flush.
+    The kept set is checked against the oracle's pooled scores (every kept token scores at least the
+    oracle's threshold up to half-precision noise; the sets overlap almost entirely), then the oracle
+    is given the product's indices and the caches must be bit-identical; decode outputs within tolerance
+    and positions continue from the full prompt length."""
+    from polarquant_amd.modeling_llama_polar import LlamaSnapKVAttention
+    torch.manual_seed(8)
+    cfg = _tiny(8, 2)
+    att = LlamaSnapKVAttention(cfg, 0).half().to(gpu)
+    assert (att.window_size, att.kernel_size, att.max_capacity_prompt) == (128, 7, 1152)
+    att.capture = []
+    steps = 140
+    x = (torch.randn(1, L + steps, cfg.hidden_size) * 0.5).half().to(gpu)
+    with torch.no_grad():
+        out, cache = att(x[:, :L], None, None, _rope(cfg, 0, L, torch.float16, gpu))
+    q, k, v = [t.cpu() for t in att.capture[-1]]
+    assert len(cache) == 8 and cache[-1] == L and cache[6].shape[2] == min(L, 1152)
+    idx = None
+    if L > 1152:
+        idx = att.last_selection.cpu()
+        s = po.snapkv_scores(q, k).float()
+        kth = s.topk(1024, dim=-1).values[..., -1:]
+        ref_idx = po.snapkv_select(q, k)
+        for h in range(2):
+            got, want = set(idx[0, h].tolist()), set(ref_idx[0, h].tolist())
+            assert len(got) == 1024 and len(got & want) >= 1000, len(got & want)
+            assert bool((s[0, h, idx[0, h]] >= kth[0, h] - 2e-3 * s[0, h].max()).all())
+    else:
+        assert att.last_selection is None
+    ref_cache = po.prefill_cache_snapkv(q, k, v, indices=idx)
+    _check_cache(cache, ref_cache)
+    o_proj = att.o_proj.weight.detach().float().cpu()
+    for i in range(steps):
+        with torch.no_grad():
+            out, cache = att(x[:, L + i:L + i + 1], None, cache, _rope(cfg, L + i, 1, torch.float16, gpu))
+        q, k, v = [t.cpu() for t in att.capture[-1]]
+        ref_attn, ref_cache = po.decode_step(q, k, v, ref_cache)
+        ref_out = ref_attn.reshape(1, 1, -1).float() @ o_proj.T
+        err = (out.float().cpu() - ref_out).abs().max().item()
+        assert err < 2e-2 * max(1.0, ref_out.abs().max().item()), (i, err)
+        if i in (0, 1, steps - 1) or cache[0] is None or cache[0].shape[2] == 1:
+            _check_cache(cache, ref_cache)
+    assert cache[-1] == L + steps and cache[6].shape[2] == min(L, 1152) + steps
+    # a plain tuple (no arena) whose length slot exceeds its cached tokens is accepted as well
+    plain = tuple(t.clone() if torch.is_tensor(t) else t for t in cache)
+    with torch.no_grad():
+        o1, c1 = att(x[:, -1:], None, cache, _rope(cfg, L + steps, 1, torch.float16, gpu))
+        o2, c2 = att(x[:, -1:], None, plain, _rope(cfg, L + steps, 1, torch.float16, gpu))
+    assert torch.equal(o1, o2) and c1[-1] == c2[-1] == L + steps + 1
+    with pytest.raises(AssertionError):
+        att(x[:, -1:].repeat(2, 1, 1), None, c1, _rope(cfg, 0, 1, torch.float16, gpu))      # batch 1 only at decode time
+
+
+def test_model_shell_selects_the_variants(gpu):
+    from polarquant_amd.modeling_llama_polar import LlamaPolarMixedGroupAttention, LlamaSnapKVAttention
+    assert isinstance(LlamaPolarForCausalLM(_tiny(layers=1, vbits=4)).model.layers[0].self_attn, LlamaPolarMixedGroupAttention)
+    assert isinstance(LlamaPolarForCausalLM(_tiny(layers=1, snapkv=True)).model.layers[0].self_attn, LlamaSnapKVAttention)
+    assert type(LlamaPolarForCausalLM(_tiny(layers=1)).model.layers[0].self_attn) is LlamaPolarGroupAttention
+    # greedy generation through the SnapKV variant: positions run on from the full prompt length
+    torch.manual_seed(9)
+    cfg = _tiny(layers=2, snapkv=True)
+    model = LlamaPolarForCausalLM(cfg).half().to(gpu).eval()
+    ids = torch.randint(0, cfg.vocab_size, (1, 1300), device=gpu)
+    out = generate(model, ids, torch.ones_like(ids), GenerationConfig(eos_token_id=[999999]), max_new_tokens=5)
+    assert out.shape == (1, 5)

@@ -403,3 +403,64 @@ def test_mixed_cache_bookkeeping(L):
         if vc is not None:
             assert vc.shape == (1, 2, nq, 16) and vs.shape == vm.shape == (1, 2, nq, 1)
         assert out.shape == (1, 4, 1, 128)
+
+
+# ------------------------------------------------------------------ SnapKV prompt eviction
+def test_snapkv_selection_keeps_the_keys_the_window_attends_to():
+    """Hand-built prompt: a few earlier keys are aligned with every query of the last window, the rest
+    are noise.  With a pooling kernel of 7 each heavy key lifts its 6 neighbours; the kept set must
+    contain all of those neighbourhoods, for every KV head."""
+    torch.manual_seed(0)
+    B, N, Nk, L, ws, cap = 1, 4, 2, 600, 64, 64 + 80
+    u = torch.randn(128)
+    u = u / u.norm()
+    q = (0.05 * torch.randn(B, N, L, 128) + 3.0 * u).half()
+    k = (0.05 * torch.randn(B, Nk, L, 128)).half()
+    heavy = [20, 75, 130, 222, 301, 377, 444, 500]
+    k[:, :, heavy] = (4.0 * u).half()
+    idx = po.snapkv_select(q, k, window_size=ws, kernel_size=7, max_capacity_prompt=cap)
+    assert idx.shape == (B, Nk, cap - ws) and int(idx.max()) < L - ws
+    want = {p + d for p in heavy for d in range(-3, 4)}
+    for h in range(Nk):
+        got = set(idx[0, h].tolist())
+        assert len(got) == cap - ws and want <= got
+    # with no pooling the choice depends on each key alone: permuting the earlier keys permutes the kept set
+    perm = torch.randperm(L - ws)
+    k2 = k.clone()
+    k2[:, :, :L - ws] = k[:, :, perm]
+    a = po.snapkv_select(q, k, ws, 1, cap)
+    b = po.snapkv_select(q, k2, ws, 1, cap)
+    s = po.snapkv_scores(q, k, ws, 1)
+    kth = s.topk(cap - ws, dim=-1).values[..., -1:]
+    for h in range(Nk):
+        strictly_in = set(torch.nonzero(s[0, h] > kth[0, h]).flatten().tolist())      # ties at the threshold may go either way
+        assert strictly_in <= set(a[0, h].tolist()) and strictly_in <= {int(perm[j]) for j in b[0, h].tolist()}
+
+
+@pytest.mark.parametrize("L", [100, 128, 700, 1152, 1153, 1400])
+def test_snapkv_cache_bookkeeping(L):
+    """Prompts up to max_capacity_prompt are cached whole (the plain polar prefill); longer ones keep
+    1024 selected tokens + the last 128, all quantized (1152 = 9 groups), their values gathered with
+    the same indices, and the tuple still reports the full prompt length."""
+    g = torch.Generator().manual_seed(L)
+    q, k, v = wl.make_half((1, 4, L, 128), g), wl.make_keys(1, 2, L, 1e4, g), wl.make_half((1, 2, L, 128), g)
+    cache = po.prefill_cache_snapkv(q, k, v)
+    assert len(cache) == 8 and cache[-1] == L
+    kept = min(L, 1152)
+    assert cache[6].shape[2] == kept
+    nq = 0 if cache[1] is None else cache[1].shape[2] * 128
+    nr = 0 if cache[0] is None else cache[0].shape[2]
+    assert nq + nr == kept and (nq == (kept // 128) * 128 if L >= 128 else nq == 0)
+    if L <= 1152:
+        plain = po.prefill_cache(k, v)
+        for a, b in zip(cache[:-1], plain[:-1]):
+            assert (a is None) == (b is None) and (a is None or torch.equal(a, b))
+    else:
+        idx = po.snapkv_select(q, k)
+        assert torch.equal(cache[6][:, :, :1024], v[:, :, :-128].gather(2, idx.unsqueeze(-1).expand(-1, -1, -1, 128)))
+        assert torch.equal(cache[6][:, :, 1024:], v[:, :, -128:])
+        kk = torch.cat([k[:, :, :-128].gather(2, idx.unsqueeze(-1).expand(-1, -1, -1, 128)), k[:, :, -128:]], 2)
+        assert torch.equal(cache[1], po.quantize_and_pack_nbit(kk)[0])
+        # decode continues at position L and appends to the 1152 cached tokens
+        out, c2 = po.decode_step(wl.make_half((1, 4, 1, 128), g), k[:, :, :1], v[:, :, :1], cache)
+        assert c2[-1] == L + 1 and c2[6].shape[2] == 1153 and c2[0].shape[2] == 1
