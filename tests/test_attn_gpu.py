@@ -158,3 +158,29 @@ def test_attn_sharp_softmax(gpu):
     ref64 = po.decode_attention_exact(q, kres, *quant, v)
     out = polar_decode_attention(q.to(gpu), *[t.to(gpu) for t in quant], kres.to(gpu), v.to(gpu), ng, 3, n_splits=2)
     assert _close(out.cpu(), ref64)[0] == 0
+
+
+def test_attn_empty_and_fully_masked_sequences(gpu):
+    """A ragged batch may hold a sequence with no cached token at all, and a mask may hide every
+    token of a sequence: both have nothing to attend to and must yield zeros (no NaN from 0/0),
+    without disturbing their neighbours."""
+    g = torch.Generator().manual_seed(14)
+    B, N, Nk = 3, 8, 2
+    L = 2 * 128 + 9
+    k = wl.make_keys(B, Nk, L, 5e5, g)
+    q = wl.make_half((B, N, 1, 128), g)
+    v = wl.make_half((B, Nk, L, 128), g)
+    quant = po.quantize_and_pack_nbit(k[:, :, :256].contiguous())
+    kres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16)
+    kres[:, :, :9] = k[:, :, 256:]
+    groups = torch.tensor([2, 0, 2], dtype=torch.int32)
+    resid = torch.tensor([9, 0, 9], dtype=torch.int32)           # sequence 1 is empty
+    mask = torch.ones(B, L, dtype=torch.uint8)
+    mask[2] = 0                                                  # sequence 2 is masked out entirely
+    out = polar_decode_attention(q.to(gpu), *[t.to(gpu) for t in quant], kres.to(gpu), v.to(gpu), 0, 0,
+                                 attention_mask=mask.to(gpu), n_groups_per_seq=groups.to(gpu),
+                                 n_resid_per_seq=resid.to(gpu), n_splits=2).cpu()
+    assert torch.isfinite(out.float()).all()
+    assert bool((out[1] == 0).all()) and bool((out[2] == 0).all())
+    ref = po.decode_attention_exact(q[:1], k[:1, :, 256:], *[t[:1] for t in quant], v[:1])
+    assert _close(out[:1], ref)[0] == 0
