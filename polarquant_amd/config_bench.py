@@ -1,4 +1,4 @@
-"""The other BASELINE configurations on one GPU, same kernels and timing as bench.py
+"""The other benchmark configurations on one GPU, same kernels and timing as bench.py
 (which carries the headline, configs[1]):
 
   configs[0]  score op, Llama-2-7B shape (batch 1, 32 heads MHA, context 4096)

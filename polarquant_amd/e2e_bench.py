@@ -1,4 +1,4 @@
-"""End-to-end greedy decode with the polar-key attention (BASELINE configs[4]):
+"""End-to-end greedy decode with the polar-key attention (workload configs[4]):
 random-init Llama-3-8B architecture (32 layers, hidden 4096, 32 q / 8 KV heads, FFN 14336,
 vocab 128256), bf16 weights ~N(0, 0.02), batch 8, prompt 16384 random ids, 256 new tokens.
 Reports prefill seconds, decode tokens/s and KV-cache bytes per token.  Mirrors the

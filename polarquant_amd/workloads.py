@@ -31,7 +31,7 @@ class Shape:
     ragged: bool = False
 
 
-# index k == BASELINE configs[k] (config 4, the end-to-end model, has its own builder)
+# index k == benchmark workload configs[k] (config 4, the end-to-end model, has its own builder)
 CONFIGS = [
     Shape("cfg0-llama2-7b-scores-b1-4k", 1, 32, 32, 4096, 4, 4, 1e4, 1000),
     Shape("cfg1-llama3-8b-b16-32k", 16, 32, 8, 32768, 4, 4, 5e5, 1001),

@@ -1,4 +1,4 @@
-"""Parity at BASELINE.json's full sizes (configs[1], [2], [3]).
+"""Parity at the full sizes of the benchmark configurations (configs[1], [2], [3]).
 
 The CPU oracle cannot chew through a gigabyte of cache in seconds, so each
 full-size case combines (a) the oracle on whole (sequence, KV head) planes picked

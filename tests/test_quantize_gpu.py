@@ -47,7 +47,7 @@ def test_quantize_bit_exact(gpu, dtype, rbits, tbits):
 
 
 def test_quantize_cfg0_full_flip_count(gpu):
-    """BASELINE configs[0] keys: [1,32,4096,128] fp16, RoPE theta 1e4, 4/4 bits."""
+    """Workload configs[0] keys: [1,32,4096,128] fp16, RoPE theta 1e4, 4/4 bits."""
     sh = wl.CONFIGS[0]
     inp = wl.make_decode_inputs(sh)
     ref = po.quantize_and_pack_nbit(inp.k, 4, 4)

@@ -43,7 +43,7 @@ def test_scores_match_oracle(gpu, dtype, heads, kv, rbits, tbits):
 
 
 def test_scores_cfg0_full(gpu):
-    """BASELINE configs[0]: batch 1, 32 heads MHA, context 4096, 4/4 bits."""
+    """Workload configs[0]: batch 1, 32 heads MHA, context 4096, 4/4 bits."""
     sh = wl.CONFIGS[0]
     inp = wl.make_decode_inputs(sh)
     quant = po.quantize_and_pack_nbit(inp.k, sh.rbits, sh.tbits)
