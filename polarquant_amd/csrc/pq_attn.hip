@@ -135,10 +135,15 @@ __device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[
 // exactly; so the A operand costs two v_and per word and one v_perm per register, like the
 // half-precision rows it replaces, and the accumulators are brought back to real units once,
 // after the last quantized tile (finish_v4).  The probabilities go through half precision for
-// this product whatever the model dtype; kV4Pre keeps p * scale inside its range.
-constexpr float kV4Pre = 0x1p-6f;
-constexpr float kV4PostEven = 0x1p30f;   // 2^24 / kV4Pre
-constexpr float kV4PostOdd = 0x1p26f;    // nibble left at 16 * code
+// this product whatever the model dtype.  The weight p * scale must stay inside half precision's
+// range at both ends: the running maximum is allowed to lag by only 2^kLazyThresholdV4 here, so
+// that weight <= 4 * scale (scale <= 8734 for any half-precision row), and no further pre-scaling
+// is applied, so that the tail of the softmax keeps the resolution the reference's
+// half-precision probabilities have (a weight below 2^-25 drops out; with a pre-scale of 2^-6 a
+// long flat tail 12 nats under the peak, still 10 % of the mass over 32k tokens, was lost).
+constexpr float kLazyThresholdV4 = 2.0f;
+constexpr float kV4PostEven = 0x1p24f;   // subnormal nibble = code * 2^-24
+constexpr float kV4PostOdd = 0x1p20f;    // odd nibbles are left at 16 * code
 
 // Tokens of a 16-token block are handed to the MFMA k-index transposed (k = 4g+i <-> token 4i+g),
 // so that one load instruction of a wavefront covers 4 whole consecutive rows (256 contiguous
@@ -152,7 +157,7 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
                                                    float sc, float zp, uint32_t pbuf, int lane) {
     bool raise = false;
 #pragma unroll
-    for (int j = 0; j < REPP; j++) raise |= t[j] > st.m[j] + kLazyThreshold;
+    for (int j = 0; j < REPP; j++) raise |= t[j] > st.m[j] + kLazyThresholdV4;
     if (__any(raise)) {
         float alpha[REPP];
 #pragma unroll
@@ -170,12 +175,12 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
         for (int e = 0; e < 8; e++) st.acc[e] *= a;
     }
     const int slot = v4_slot(lane);
-    // The weight the matrix cores see is w = half(p * scale * kV4Pre).  The zero-point term must use
-    // the SAME rounded weight (w * zero / (scale * kV4Pre)), not p: code * scale and zero are each a few
+    // The weight the matrix cores see is w = half(p * scale).  The zero-point term must use
+    // the SAME rounded weight (w * zero / scale), not p: code * scale and zero are each a few
     // units large and cancel to a value of order 1, so a weight that differs between the two terms by
     // its rounding error (2^-11) would leave an error of that size times ~3 when one token dominates.
     // A constant row has scale 0 and all codes 0: any scale serves, take 1.
-    const float scp = (sc == 0.0f ? 1.0f : sc) * kV4Pre;
+    const float scp = sc == 0.0f ? 1.0f : sc;
     const float zq = zp / scp;
 #pragma unroll
     for (int j = 0; j < REPP; j++) {

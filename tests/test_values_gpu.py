@@ -1,6 +1,8 @@
 """4-bit values of the Mixed variant on the GPU against the CPU oracle: the value quantizer is
 bit-exact (codes, scale, zero-point), the fused decode attention over polar keys + 4-bit values
 meets the output bar against the literal restatement and the fp64 evaluation."""
+import math
+
 import pytest
 import torch
 
@@ -206,3 +208,42 @@ def test_attention_v4_ragged_batch_matches_per_sequence_oracle(gpu):
         for b in range(B):
             nbad, emax = _close(out[b:b + 1], refs[b])
             assert nbad == 0, (kw, b, nbad, emax)
+
+
+@pytest.mark.parametrize("values4", [True, False])
+def test_attention_long_flat_tail_under_a_peak_is_not_dropped(gpu, values4):
+    """One key scores 12.5 nats above 32767 others.  Each of those carries 3.7e-6 of the peak's
+    weight, together 12 % of the mass: half-precision weights must keep them (the reference's
+    half-precision probabilities do), which shows in a value channel with a non-zero mean."""
+    g = torch.Generator().manual_seed(91)
+    B, N, Nk, nb = 1, 4, 1, 256
+    L = nb * 128
+    u = torch.randn(128, generator=g)
+    u = u / u.norm()
+    k = (0.01 * torch.randn(B, Nk, L + 1, 128, generator=g)).half()
+    k[0, 0, 20000] = (12.5 * math.sqrt(128) / 10.0 * u).half()
+    q = (10.0 * u).half().expand(B, N, 1, 128).contiguous()
+    v = wl.make_half((B, Nk, L + 1, 128), g)
+    v[..., 5] += 2.0
+    v[0, 0, 20000, 5] = -3.0                          # the peak's own value is far from the tail's mean
+    quant = po.quantize_and_pack_nbit(k[:, :, :L].contiguous())
+    kres, vres = k[:, :, L:].contiguous(), v[:, :, L:].contiguous()
+    dq = [t.to(gpu) for t in quant]
+    if values4:
+        vq = po.quantize_values_along_last_dim(v[:, :, :L].contiguous())
+        ref64 = po.decode_attention_mixed_exact(q, kres, *quant, vres, *vq)
+        dk = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=gpu)
+        dv = torch.zeros_like(dk)
+        dk[:, :, :1], dv[:, :, :1] = kres.to(gpu), vres.to(gpu)
+        run = lambda ns: polar_decode_attention_v4(q.to(gpu), *dq, dk, dv, *[t.to(gpu) for t in vq], nb, 1, n_splits=ns)
+    else:
+        from polarquant_amd.attention import polar_decode_attention
+        ref64 = po.decode_attention_exact(q, kres, *quant, v)
+        run = lambda ns: polar_decode_attention(q.to(gpu), *dq, kres.to(gpu), v.to(gpu), nb, 1, n_splits=ns)
+    # the tail really is a tenth of the mass: without it channel 5 would be off by ~0.5
+    assert abs(ref64[0, 0, 0, 5].item() - (-3.0)) > 0.3
+    for ns in (1, 16, 128):
+        out = run(ns).cpu()
+        nbad, emax = _close(out, ref64)
+        print("flat tail, values4", values4, "n_splits", ns, "max abs err %.2e" % emax, flush=True)
+        assert nbad == 0, (ns, nbad, emax)
