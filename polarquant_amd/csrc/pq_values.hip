@@ -18,6 +18,9 @@ namespace pq {
 template <typename T>
 __device__ __forceinline__ float rnd_v(float f) { return lo2f<T>(f2lo<T>(f)); }
 
+template <typename T> struct IsF16 { static constexpr bool value = false; };
+template <> struct IsF16<F16> { static constexpr bool value = true; };
+
 constexpr int kVThreads = 256;
 constexpr int kRowsPerBlock = kVThreads / 16;
 
@@ -30,37 +33,71 @@ __global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
     const int bh = blockIdx.y;
     const bool live = t < n_tok;                       // whole 16-lane row groups are live or not
     const int b = bh / Nk, h = bh - b * Nk;
-    float x[8];
-    float lo = INFINITY, hi = -INFINITY;
-    if (live) {
-        const uint4 w = *reinterpret_cast<const uint4*>(v + b * sb + h * sh + static_cast<int64_t>(t) * st + 8 * n);
+    const int64_t row = static_cast<int64_t>(bh) * cap + off + t;
+    uint4 w = make_uint4(0, 0, 0, 0);
+    if (live) w = *reinterpret_cast<const uint4*>(v + b * sb + h * sh + static_cast<int64_t>(t) * st + 8 * n);
+    if constexpr (IsF16<T>::value) {
+        // half precision: the eager ops ARE half-precision instructions here (v_pk_min/max_f16,
+        // v_sub_f16, the compiler's correctly rounded half division, v_med3_f16, v_rndne_f16)
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        const half2v p0 = __builtin_bit_cast(half2v, w.x), p1 = __builtin_bit_cast(half2v, w.y);
+        const half2v p2 = __builtin_bit_cast(half2v, w.z), p3 = __builtin_bit_cast(half2v, w.w);
+        const half2v mn2 = __builtin_elementwise_min(__builtin_elementwise_min(p0, p1), __builtin_elementwise_min(p2, p3));
+        const half2v mx2 = __builtin_elementwise_max(__builtin_elementwise_max(p0, p1), __builtin_elementwise_max(p2, p3));
+        // (min, -max) in one register: both reduce with a packed min
+        half2v red = {live ? (mn2.x < mn2.y ? mn2.x : mn2.y) : static_cast<_Float16>(INFINITY),
+                      live ? -(mx2.x > mx2.y ? mx2.x : mx2.y) : static_cast<_Float16>(INFINITY)};
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+            const int other = __shfl_xor(__builtin_bit_cast(int, red), o);
+            red = __builtin_elementwise_min(red, __builtin_bit_cast(half2v, other));
+        }
+        if (!live) return;
+        const _Float16 lo = red.x, hi = -red.y;
+        const _Float16 sc = static_cast<_Float16>(hi - lo) / static_cast<_Float16>(15.0f);
+        const half2v ps[4] = {p0, p1, p2, p3};
+        uint32_t word = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const _Float16 x = (i & 1) ? ps[i >> 1].y : ps[i >> 1].x;
+            _Float16 q = static_cast<_Float16>(x - lo) / sc;
+            q = __builtin_amdgcn_fmed3h(q, static_cast<_Float16>(0.0f), static_cast<_Float16>(15.0f));   // NaN (0/0) -> 0
+            q = __builtin_rintf16(q);                      // round half to even
+            word |= static_cast<uint32_t>(static_cast<unsigned short>(q)) << (4 * i);
+        }
+        codes[row * 16 + n] = static_cast<int32_t>(word);
+        if (n == 0) { scale[row] = __builtin_bit_cast(uint16_t, sc); mn[row] = __builtin_bit_cast(uint16_t, lo); }
+    } else {
+        float x[8];
+        float lo = INFINITY, hi = -INFINITY;
         const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             x[2 * i] = lo2f<T>(static_cast<uint16_t>(ww[i] & 0xffffu));
             x[2 * i + 1] = lo2f<T>(static_cast<uint16_t>(ww[i] >> 16));
         }
+        if (live) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
-    }
+            for (int i = 0; i < 8; i++) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
+        }
 #pragma unroll
-    for (int o = 1; o < 16; o <<= 1) {
-        lo = fminf(lo, __shfl_xor(lo, o));
-        hi = fmaxf(hi, __shfl_xor(hi, o));
-    }
-    if (!live) return;
-    const float sc = rnd_v<T>(rnd_v<T>(hi - lo) / 15.0f);
-    uint32_t word = 0;
+        for (int o = 1; o < 16; o <<= 1) {
+            lo = fminf(lo, __shfl_xor(lo, o));
+            hi = fmaxf(hi, __shfl_xor(hi, o));
+        }
+        if (!live) return;
+        const float sc = rnd_v<T>(rnd_v<T>(hi - lo) / 15.0f);
+        uint32_t word = 0;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        float q = rnd_v<T>(rnd_v<T>(x[i] - lo) / sc);
-        q = fminf(fmaxf(q, 0.0f), 15.0f);          // NaN (0/0 on a constant row) comes out of fmaxf as 0
-        q = __builtin_rintf(q);                    // round half to even
-        word |= static_cast<uint32_t>(q) << (4 * i);
+        for (int i = 0; i < 8; i++) {
+            float q = rnd_v<T>(rnd_v<T>(x[i] - lo) / sc);
+            q = __builtin_amdgcn_fmed3f(q, 0.0f, 15.0f);   // NaN (0/0 on a constant row) comes out as the minimum, 0
+            q = __builtin_rintf(q);                        // round half to even
+            word |= static_cast<uint32_t>(q) << (4 * i);
+        }
+        codes[row * 16 + n] = static_cast<int32_t>(word);
+        if (n == 0) { scale[row] = f2lo<T>(sc); mn[row] = f2lo<T>(lo); }
     }
-    const int64_t row = static_cast<int64_t>(bh) * cap + off + t;
-    codes[row * 16 + n] = static_cast<int32_t>(word);
-    if (n == 0) { scale[row] = f2lo<T>(sc); mn[row] = f2lo<T>(lo); }
 }
 
 int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int B, int Nk, int T,
