@@ -195,3 +195,21 @@ def test_python_wrappers_refuse_cpu_tensors():
         attention_decode_forward_triton_impl(k[:, :, :1], torch.zeros(1, 1, 1, 128, 64, dtype=torch.uint8), *[k[:, :, :1, :64].unsqueeze(2)] * 4)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         polar_decode_attention(k[:, :, :1], None, None, None, None, None, k, k, 0, 1)
+
+
+def test_header_compiles_as_c_and_library_links_without_python(tmp_path):
+    """gcc -std=c11 against include/polarquant.h, linked with the shared library only."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.join(root, "polarquant_amd")
+    if not os.path.exists(os.path.join(libdir, "libpolarquant_hip.so")):
+        pytest.skip("library not built")
+    exe = str(tmp_path / "capi_link")
+    cmd = ["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(root, "include"),
+           os.path.join(root, "tests", "capi_link_main.c"), "-o", exe, "-L", libdir, "-lpolarquant_hip",
+           "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"]
+    build = subprocess.run(cmd, capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-3000:]
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr[-2000:])
+    assert run.stdout.startswith("capi ok")
