@@ -1,0 +1,103 @@
+"""Seeded random differential test: random batch / head / bit-width / length / mask / split
+combinations of the fused decode attention, with half-precision or 4-bit values, uniform or
+per-sequence lengths, against the fp64 oracle evaluated sequence by sequence."""
+import os
+import random
+
+import pytest
+import torch
+
+from oracle import polar_oracle as po
+from polarquant_amd import workloads as wl
+from polarquant_amd.attention import polar_decode_attention, polar_decode_attention_v4
+
+pytestmark = pytest.mark.gpu
+HEADS = [(1, 1), (2, 1), (4, 4), (8, 2), (3, 1), (6, 1), (7, 1), (8, 1), (16, 2), (12, 4)]
+BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 4)]
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))   # more seeds: PQ_RANDOM_CASES=300
+def test_random_decode_attention_case(gpu, seed):
+    rnd = random.Random(1000 + seed)
+    N, Nk = rnd.choice(HEADS)
+    rb, tb = rnd.choice(BITS)
+    B = rnd.randint(1, 4)
+    dtype = torch.bfloat16 if seed % 6 == 5 else torch.float16
+    values4 = rnd.random() < 0.5
+    ragged = rnd.random() < 0.5
+    cap = rnd.randint(1, 7)
+    groups = [rnd.randint(0, cap) for _ in range(B)] if ragged else [rnd.randint(0, cap)] * B
+    resid = [rnd.randint(1, 128) for _ in range(B)] if ragged else [rnd.randint(1, 128)] * B
+    use_mask = rnd.random() < 0.4
+    n_splits = rnd.choice([None, 1, 2, 3, 5])
+    print("case", dict(seed=seed, N=N, Nk=Nk, bits=(rb, tb), B=B, dtype=str(dtype), values4=values4, groups=groups,
+                       resid=resid, mask=use_mask, n_splits=n_splits), flush=True)
+    g = torch.Generator().manual_seed(seed)
+    q = wl.make_half((B, N, 1, 128), g, dtype)
+    codes = torch.zeros(B, Nk, cap, 128, 64, dtype=torch.uint8)
+    meta = [torch.zeros(B, Nk, cap, 1, 64, dtype=dtype) for _ in range(4)]
+    vcodes = torch.zeros(B, Nk, cap * 128, 16, dtype=torch.int32)
+    vmeta = [torch.zeros(B, Nk, cap * 128, 1, dtype=dtype) for _ in range(2)]
+    kres = torch.zeros(B, Nk, 128, 128, dtype=dtype)
+    vres = torch.zeros(B, Nk, 128, 128, dtype=dtype)
+    vfull = torch.zeros(B, Nk, cap * 128 + 128, 128, dtype=dtype)
+    mask = torch.ones(B, cap * 128 + 128, dtype=torch.uint8)
+    refs = []
+    for b in range(B):
+        nb, nr = groups[b], resid[b]
+        L = nb * 128 + nr
+        k = wl.make_keys(1, Nk, L, 5e5, g, dtype)
+        v = wl.make_half((1, Nk, L, 128), g, dtype)
+        v[..., 3] += 1.5
+        quant, vq = (None,) * 5, (None,) * 3
+        if nb:
+            quant = po.quantize_and_pack_nbit(k[:, :, :nb * 128].contiguous(), rb, tb)
+            codes[b, :, :nb] = quant[0][0]
+            for m, t in zip(meta, quant[1:]):
+                m[b, :, :nb] = t[0]
+            if values4:
+                vq = po.quantize_values_along_last_dim(v[:, :, :nb * 128].contiguous())
+                vcodes[b, :, :nb * 128] = vq[0][0]
+                for m, t in zip(vmeta, vq[1:]):
+                    m[b, :, :nb * 128] = t[0]
+        kres[b, :, :nr], vres[b, :, :nr] = k[0, :, nb * 128:], v[0, :, nb * 128:]
+        vfull[b, :, :L] = v[0]
+        mb = None
+        if use_mask:
+            mb = torch.ones(1, L, dtype=torch.int64)
+            mb[0, :rnd.randint(0, L - 1)] = 0
+            mask[b, :L] = mb[0]
+        kr, vr = k[:, :, nb * 128:], v[:, :, nb * 128:]
+        if values4:
+            exact = po.decode_attention_mixed_exact(q[b:b + 1], kr, *quant, vr, *vq, mb, rb, tb)
+            literal = po.decode_attention_mixed(q[b:b + 1], kr, *quant, vr, *vq, mb, rb, tb)
+        else:
+            exact = po.decode_attention_exact(q[b:b + 1], kr, *quant, v, mb, rb, tb)
+            literal = po.decode_attention(q[b:b + 1], kr, *quant, v, mb, rb, tb)
+        refs.append((exact, (literal.double() - exact).abs()))
+    dev = lambda t: t.to(gpu)
+    kw = dict(rbits=rb, tbits=tb, n_splits=n_splits, attention_mask=dev(mask) if use_mask else None)
+    if ragged:
+        kw.update(n_groups_per_seq=torch.tensor(groups, dtype=torch.int32, device=gpu),
+                  n_resid_per_seq=torch.tensor(resid, dtype=torch.int32, device=gpu))
+        ng, nr = 0, 0
+    else:
+        ng, nr = groups[0], resid[0]
+    have_groups = any(groups) or ragged
+    cq = [dev(codes)] + [dev(m) for m in meta] if have_groups else [None] * 5
+    if values4:
+        vq_d = [dev(vcodes)] + [dev(m) for m in vmeta] if have_groups else [None] * 3
+        out = polar_decode_attention_v4(dev(q), *cq, dev(kres), dev(vres), *vq_d, ng, nr, **kw)
+    else:
+        out = polar_decode_attention(dev(q), *cq, dev(kres), dev(vfull), ng, nr, **kw)
+    out = out.cpu()
+    assert torch.isfinite(out.float()).all()
+    # the band is centred on the fp64 value and widened, element by element, by the distance of the
+    # reference path's own half-precision evaluation from it (scores of the residual window and
+    # probabilities rounded to the dtype matter when only a few dozen tokens are attended to)
+    rtol, atol = (1e-2, 1e-3) if dtype == torch.float16 else (2e-2, 4e-3)
+    for b in range(B):
+        exact, ref_noise = refs[b]
+        err = (out[b:b + 1].double() - exact).abs()
+        bad = int((err > atol + rtol * exact.abs() + ref_noise).sum())
+        assert bad == 0, (b, bad, float(err.max()))
