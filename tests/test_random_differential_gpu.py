@@ -101,3 +101,40 @@ def test_random_decode_attention_case(gpu, seed):
         err = (out[b:b + 1].double() - exact).abs()
         bad = int((err > atol + rtol * exact.abs() + ref_noise).sum())
         assert bad == 0, (b, bad, float(err.max()))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))
+def test_random_quantizer_case(gpu, seed):
+    """Key and value quantizers, bit for bit against the oracle, on keys / values of random scale
+    (1e-6 .. 1e4), distribution (normal, heavy-tailed, sparse, nearly constant) and bit widths."""
+    from polarquant_amd.quantize import quantize_and_pack_nbit
+    from polarquant_amd.values import quantize_values
+    rnd = random.Random(5000 + seed)
+    dtype = torch.bfloat16 if seed % 3 == 2 else torch.float16
+    rb, tb = rnd.choice(BITS)
+    mode = rnd.choice(["group", "group", "uniform"])
+    scale = 10.0 ** rnd.uniform(-6, 4 if dtype == torch.bfloat16 else 3.5)
+    kind = rnd.choice(["normal", "cauchy", "sparse", "flat"])
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(2, 2, 256, 128, generator=g)
+    if kind == "cauchy":
+        x = x / torch.randn(2, 2, 256, 128, generator=g).abs().clamp_min(1e-3)
+    elif kind == "sparse":
+        x = x * (torch.rand(2, 2, 256, 128, generator=g) < 0.1)
+    elif kind == "flat":
+        x = 1.0 + 1e-3 * x
+    x = (x * scale).clamp(-6e4, 6e4).to(dtype)
+    print("case", dict(seed=seed, dtype=str(dtype), bits=(rb, tb), mode=mode, scale=scale, kind=kind), flush=True)
+    ref = po.quantize_and_pack_nbit(x, rb, tb, angle_mode=mode)
+    got = quantize_and_pack_nbit(x.to(gpu), rb, tb, angle_mode=mode)
+    flips = int((got[0].cpu() != ref[0]).sum())
+    assert flips == 0, "code flips: %d of %d" % (flips, ref[0].numel())
+    for name, a, b in zip(["rscale", "rmn", "tscale", "tmn"], got[1:], ref[1:]):
+        a, b = a.cpu().float(), b.float()
+        assert bool(((a == b) | (a.isnan() & b.isnan())).all()), name
+    vref = po.quantize_values_along_last_dim(x)
+    vgot = quantize_values(x.to(gpu))
+    assert torch.equal(vgot[0].cpu(), vref[0]), "value code words differ: %d" % int((vgot[0].cpu() != vref[0]).sum())
+    for name, a, b in zip(["scale", "mn"], vgot[1:], vref[1:]):
+        a, b = a.cpu().float(), b.float()
+        assert bool(((a == b) | (a.isnan() & b.isnan())).all()), name
