@@ -260,7 +260,9 @@ int pq_decode_attn_v4(const void *q,
  * window (:77) and the value's append to the value cache (:98), in one launch.
  * The position and the destination rows are read from device memory, so the
  * launch can be replayed from a captured graph.
- *   q_lin [B,N*128], k_lin / v_lin [B,Nk*128]  projection outputs, contiguous
+ *   q_lin [B,N*128], k_lin / v_lin [B,Nk*128]  projection outputs; batch rows q_row_stride /
+ *            kv_row_stride elements apart (0 = dense; (N+2Nk)*128 when the three are slices of
+ *            one fused projection output)
  *   cos_table / sin_table [table_rows,128]     in the dtype; row *pos is used
  *   q_out [B,N,128]
  *   k_dst [B,Nk,k_rows,128], row *k_row <- rotated key
@@ -270,18 +272,21 @@ int pq_decode_attn_v4(const void *q,
  * s = x, or s = dtype(x + residual) (also written to sum_out if given; sum_out may
  * alias x): the decoder layer's residual add + LlamaRMSNorm (:466-484).
  *
- * pq_silu_mul: y = dtype(silu(gate)) * up over n elements (LlamaMLP, called at :483).
+ * pq_silu_mul: y = dtype(silu(gate)) * up for `rows` rows of `cols` elements (LlamaMLP, called at
+ * :483); gate / up rows are in_row_stride elements apart (0 = dense; 2*cols when they are the two
+ * halves of one fused gate|up projection output), y is dense.
  * ------------------------------------------------------------------------- */
 int pq_rope_append(const void *q_lin, const void *k_lin, const void *v_lin,
                    const void *cos_table, const void *sin_table, int64_t table_rows, const int64_t *pos,
                    void *q_out, void *k_dst, int64_t k_rows, const int64_t *k_row,
                    void *v_dst, int64_t v_rows, const int64_t *v_row,
-                   int B, int N, int Nk, int dtype, void *stream);
+                   int B, int N, int Nk, int dtype, int64_t q_row_stride, int64_t kv_row_stride, void *stream);
 
 int pq_rmsnorm(const void *x, const void *residual, const void *weight, void *y, void *sum_out,
                int rows, int hidden, float eps, int dtype, void *stream);
 
-int pq_silu_mul(const void *gate, const void *up, void *y, size_t n, int dtype, void *stream);
+int pq_silu_mul(const void *gate, const void *up, void *y, int rows, int cols, int64_t in_row_stride,
+                int dtype, void *stream);
 
 /* Split count for pq_decode_attn_v4 (as pq_decode_attn_plan, which see; the 4-bit
  * kernel runs two wavefronts per SIMD when N/Nk <= 4). No reference counterpart. */

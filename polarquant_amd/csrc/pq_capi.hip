@@ -242,14 +242,20 @@ int pq_decode_attn(const void* q,
 // ---- fused elementwise steps of the decode layer -----------------------------------------------
 int pq_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_table, const void* sin_table,
                    int64_t table_rows, const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
-                   void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int dtype, void* stream) {
+                   void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int dtype,
+                   int64_t q_row_stride, int64_t kv_row_stride, void* stream) {
     if (!q_lin || !k_lin || !v_lin || !cos_table || !sin_table || !pos || !q_out || !k_dst || !k_row || !v_dst || !v_row)
         return PQ_ERR_NULL_POINTER;
     if (B <= 0 || N <= 0 || Nk <= 0 || B > 65535) return PQ_ERR_BAD_SHAPE;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
     if (table_rows <= 0 || k_rows <= 0 || v_rows <= 0) return PQ_ERR_BAD_STRIDE;
+    if (q_row_stride == 0) q_row_stride = static_cast<int64_t>(N) * PQ_HEAD_DIM;          // dense
+    if (kv_row_stride == 0) kv_row_stride = static_cast<int64_t>(Nk) * PQ_HEAD_DIM;
+    if (q_row_stride < static_cast<int64_t>(N) * PQ_HEAD_DIM || kv_row_stride < static_cast<int64_t>(Nk) * PQ_HEAD_DIM)
+        return PQ_ERR_BAD_STRIDE;
     const int err = pq::launch_rope_append(q_lin, k_lin, v_lin, cos_table, sin_table, pos, q_out, k_dst, k_rows, k_row, v_dst,
-                                           v_rows, v_row, B, N, Nk, table_rows, dtype, static_cast<hipStream_t>(stream));
+                                           v_rows, v_row, B, N, Nk, table_rows, dtype, q_row_stride, kv_row_stride,
+                                           static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
@@ -265,12 +271,14 @@ int pq_rmsnorm(const void* x, const void* residual, const void* weight, void* y,
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
-int pq_silu_mul(const void* gate, const void* up, void* y, size_t n, int dtype, void* stream) {
+int pq_silu_mul(const void* gate, const void* up, void* y, int rows, int cols, int64_t in_row_stride, int dtype, void* stream) {
     if (!gate || !up || !y) return PQ_ERR_NULL_POINTER;
-    if (n == 0 || n % 8) return PQ_ERR_BAD_SHAPE;
+    if (rows <= 0 || rows > 65535 || cols <= 0 || cols % 8) return PQ_ERR_BAD_SHAPE;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
-    if (!aligned(gate, 16) || !aligned(up, 16) || !aligned(y, 16)) return PQ_ERR_MISALIGNED;
-    const int err = pq::launch_silu_mul(gate, up, y, n, dtype, static_cast<hipStream_t>(stream));
+    if (in_row_stride == 0) in_row_stride = cols;                                       // dense
+    if (in_row_stride < cols) return PQ_ERR_BAD_STRIDE;
+    if (!aligned(gate, 16) || !aligned(up, 16) || !aligned(y, 16) || in_row_stride % 8) return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_silu_mul(gate, up, y, rows, cols, in_row_stride, dtype, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 

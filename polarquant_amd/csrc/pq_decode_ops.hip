@@ -20,7 +20,9 @@ template <typename T>
 __device__ __forceinline__ float rnd_a(float f) { return lo2f<T>(f2lo<T>(f)); }
 
 // grid (N + 2*Nk, B), 64 threads: lane d owns the pair (d, d+64) of one head.
-//   q_lin [B, N*128], k_lin / v_lin [B, Nk*128]: outputs of the projections for the new token
+//   q_lin [B, N*128], k_lin / v_lin [B, Nk*128]: outputs of the projections for the new token; batch
+//   rows are `lin_stride` elements apart (N*128 etc. when separate and dense, (N+2Nk)*128 when the
+//   three are slices of one fused projection output)
 //   cos_tab / sin_tab [max_pos, 128] in the dtype; *pos = position of the new token
 //   q_out [B, N, 128]
 //   k_dst [B, Nk, k_rows, 128]: row *k_row receives the rotated key
@@ -30,13 +32,14 @@ __global__ __launch_bounds__(kWave) void rope_append_kernel(
     const uint16_t* __restrict__ q_lin, const uint16_t* __restrict__ k_lin, const uint16_t* __restrict__ v_lin,
     const uint16_t* __restrict__ cos_tab, const uint16_t* __restrict__ sin_tab, const int64_t* __restrict__ pos,
     uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_dst, int64_t k_rows, const int64_t* __restrict__ k_row,
-    uint16_t* __restrict__ v_dst, int64_t v_rows, const int64_t* __restrict__ v_row, int N, int Nk, int64_t max_pos) {
+    uint16_t* __restrict__ v_dst, int64_t v_rows, const int64_t* __restrict__ v_row, int N, int Nk, int64_t max_pos,
+    int64_t q_stride, int64_t kv_stride) {
     const int d = threadIdx.x, h = blockIdx.x, b = blockIdx.y;
     if (h >= N + Nk) {                               // value head: plain copy into the cache row
         const int kvh = h - N - Nk;
         int64_t r = *v_row;
         r = r < 0 ? 0 : (r >= v_rows ? v_rows - 1 : r);
-        const uint16_t* src = v_lin + (static_cast<size_t>(b) * Nk + kvh) * kHeadDim;
+        const uint16_t* src = v_lin + static_cast<size_t>(b) * kv_stride + static_cast<size_t>(kvh) * kHeadDim;
         uint16_t* dst = v_dst + ((static_cast<size_t>(b) * Nk + kvh) * v_rows + r) * kHeadDim;
         dst[d] = src[d];
         dst[d + kPairs] = src[d + kPairs];
@@ -47,8 +50,8 @@ __global__ __launch_bounds__(kWave) void rope_append_kernel(
     const float c1 = lo2f<T>(cos_tab[p * kHeadDim + d]), c2 = lo2f<T>(cos_tab[p * kHeadDim + kPairs + d]);
     const float s1 = lo2f<T>(sin_tab[p * kHeadDim + d]), s2 = lo2f<T>(sin_tab[p * kHeadDim + kPairs + d]);
     const bool is_q = h < N;
-    const uint16_t* src = is_q ? q_lin + (static_cast<size_t>(b) * N + h) * kHeadDim
-                               : k_lin + (static_cast<size_t>(b) * Nk + (h - N)) * kHeadDim;
+    const uint16_t* src = is_q ? q_lin + static_cast<size_t>(b) * q_stride + static_cast<size_t>(h) * kHeadDim
+                               : k_lin + static_cast<size_t>(b) * kv_stride + static_cast<size_t>(h - N) * kHeadDim;
     const float x1 = lo2f<T>(src[d]), x2 = lo2f<T>(src[d + kPairs]);
     // (x * cos) + (rotate_half(x) * sin), rotate_half(x) = cat(-x2, x1)
     const float o1 = rnd_a<T>(rnd_a<T>(x1 * c1) + rnd_a<T>(-x2 * s1));
@@ -136,13 +139,16 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const uint16_t* __restrict
     }
 }
 
-// y = dtype(silu(gate)) * up, elementwise over n elements (n % 8 == 0); silu(x) = x / (1 + exp(-x)) in fp32.
+// y[r][c] = dtype(silu(gate[r][c])) * up[r][c] for `rows` rows of `cols` elements (cols % 8 == 0); gate and
+// up rows are `in_stride` elements apart (cols when dense, 2*cols when they are the two halves of one
+// fused projection output), y is dense.  silu(x) = x / (1 + exp(-x)) in fp32.
 template <typename T>
 __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ gate, const uint16_t* __restrict__ up,
-                                                        uint16_t* __restrict__ y, size_t n) {
-    const size_t i = (static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x) * 8;
-    if (i >= n) return;
-    const uint4 gv = *reinterpret_cast<const uint4*>(gate + i), uv = *reinterpret_cast<const uint4*>(up + i);
+                                                        uint16_t* __restrict__ y, int cols, int64_t in_stride) {
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (c >= cols) return;
+    const size_t in = static_cast<size_t>(blockIdx.y) * in_stride + c, out = static_cast<size_t>(blockIdx.y) * cols + c;
+    const uint4 gv = *reinterpret_cast<const uint4*>(gate + in), uv = *reinterpret_cast<const uint4*>(up + in);
     const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
     uint32_t yo[4];
 #pragma unroll
@@ -153,18 +159,19 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
         const uint16_t hi = f2lo<T>(a1 * lo2f<T>(static_cast<uint16_t>(uw[j] >> 16)));
         yo[j] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
     }
-    *reinterpret_cast<uint4*>(y + i) = make_uint4(yo[0], yo[1], yo[2], yo[3]);
+    *reinterpret_cast<uint4*>(y + out) = make_uint4(yo[0], yo[1], yo[2], yo[3]);
 }
 
 int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_tab, const void* sin_tab,
                        const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
                        void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int64_t max_pos, int dtype,
-                       hipStream_t st) {
+                       int64_t q_stride, int64_t kv_stride, hipStream_t st) {
     dim3 grid(N + 2 * Nk, B), block(kWave);
 #define PQ_RA(T)                                                                                                     \
     hipLaunchKernelGGL(rope_append_kernel<T>, grid, block, 0, st, (const uint16_t*)q_lin, (const uint16_t*)k_lin,    \
                        (const uint16_t*)v_lin, (const uint16_t*)cos_tab, (const uint16_t*)sin_tab, pos,              \
-                       (uint16_t*)q_out, (uint16_t*)k_dst, k_rows, k_row, (uint16_t*)v_dst, v_rows, v_row, N, Nk, max_pos)
+                       (uint16_t*)q_out, (uint16_t*)k_dst, k_rows, k_row, (uint16_t*)v_dst, v_rows, v_row, N, Nk, max_pos,   \
+                       q_stride, kv_stride)
     if (dtype == 0) PQ_RA(F16); else PQ_RA(BF16);
 #undef PQ_RA
     return static_cast<int>(hipGetLastError());
@@ -181,12 +188,12 @@ int launch_rmsnorm(const void* x, const void* res, const void* w, void* y, void*
     return static_cast<int>(hipGetLastError());
 }
 
-int launch_silu_mul(const void* gate, const void* up, void* y, size_t n, int dtype, hipStream_t st) {
-    const unsigned blocks = static_cast<unsigned>((n / 8 + 255) / 256);
+int launch_silu_mul(const void* gate, const void* up, void* y, int rows, int cols, int64_t in_stride, int dtype, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>((cols / 8 + 255) / 256), static_cast<unsigned>(rows)), block(256);
     if (dtype == 0)
-        hipLaunchKernelGGL(silu_mul_kernel<F16>, dim3(blocks), dim3(256), 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, n);
+        hipLaunchKernelGGL(silu_mul_kernel<F16>, grid, block, 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, cols, in_stride);
     else
-        hipLaunchKernelGGL(silu_mul_kernel<BF16>, dim3(blocks), dim3(256), 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, n);
+        hipLaunchKernelGGL(silu_mul_kernel<BF16>, grid, block, 0, st, (const uint16_t*)gate, (const uint16_t*)up, (uint16_t*)y, cols, in_stride);
     return static_cast<int>(hipGetLastError());
 }
 

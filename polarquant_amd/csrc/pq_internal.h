@@ -22,10 +22,10 @@ int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int
 int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_tab, const void* sin_tab,
                        const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
                        void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int64_t max_pos, int dtype,
-                       hipStream_t st);
+                       int64_t q_stride, int64_t kv_stride, hipStream_t st);
 int launch_rmsnorm(const void* x, const void* res, const void* w, void* y, void* sum_out, int rows, int hidden, float eps,
                    int dtype, hipStream_t st);
-int launch_silu_mul(const void* gate, const void* up, void* y, size_t n, int dtype, hipStream_t st);
+int launch_silu_mul(const void* gate, const void* up, void* y, int rows, int cols, int64_t in_stride, int dtype, hipStream_t st);
 
 struct AttnArgs {
     const void* q;

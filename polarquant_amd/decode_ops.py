@@ -19,23 +19,26 @@ def _gpu(t: torch.Tensor):
 def rope_append(q_lin: torch.Tensor, k_lin: torch.Tensor, v_lin: torch.Tensor, cos_table: torch.Tensor,
                 sin_table: torch.Tensor, pos: torch.Tensor, k_dst: torch.Tensor, k_row: torch.Tensor,
                 v_dst: torch.Tensor, v_row: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
-    """q_lin [B,1,N*128], k_lin / v_lin [B,1,Nk*128] (projection outputs of the new token);
+    """q_lin [B,1,N*128], k_lin / v_lin [B,1,Nk*128] (projection outputs of the new token; each may be a
+    slice along the last dim of one fused projection output: unit element stride, any batch stride);
     cos/sin tables [rows,128]; pos, k_row, v_row: int64 tensors of one element on the device.
     Writes the rotated key into k_dst[:, :, k_row] and the value into v_dst[:, :, v_row]
     ([B,Nk,rows,128] each); returns the rotated query [B,N,1,128]."""
     _gpu(q_lin)
     B = q_lin.shape[0]
-    assert q_lin.is_contiguous() and k_lin.is_contiguous() and v_lin.is_contiguous()
+    assert q_lin.stride(-1) == 1 and k_lin.stride(-1) == 1 and v_lin.stride(-1) == 1
+    assert k_lin.stride(0) == v_lin.stride(0) or B == 1
     assert k_dst.is_contiguous() and v_dst.is_contiguous() and cos_table.is_contiguous() and sin_table.is_contiguous()
     assert pos.dtype == k_row.dtype == v_row.dtype == torch.int64
-    assert q_lin.numel() == B * n_heads * 128 and k_lin.numel() == B * n_kv_heads * 128 == v_lin.numel()
+    assert q_lin.shape[-1] == n_heads * 128 and k_lin.shape[-1] == n_kv_heads * 128 == v_lin.shape[-1] and q_lin.numel() == B * n_heads * 128
     assert k_dst.shape[:2] == (B, n_kv_heads) == v_dst.shape[:2] and k_dst.shape[3] == 128 == v_dst.shape[3]
     q_out = torch.empty((B, n_heads, 1, 128), dtype=q_lin.dtype, device=q_lin.device)
     with torch.cuda.device(q_lin.device):
         rc = _ffi.lib().pq_rope_append(q_lin.data_ptr(), k_lin.data_ptr(), v_lin.data_ptr(), cos_table.data_ptr(),
                                        sin_table.data_ptr(), cos_table.shape[0], pos.data_ptr(), q_out.data_ptr(),
                                        k_dst.data_ptr(), k_dst.shape[2], k_row.data_ptr(), v_dst.data_ptr(), v_dst.shape[2],
-                                       v_row.data_ptr(), B, n_heads, n_kv_heads, _dtype_code(q_lin), _stream_ptr(q_lin.device))
+                                       v_row.data_ptr(), B, n_heads, n_kv_heads, _dtype_code(q_lin),
+                                       q_lin.stride(0), k_lin.stride(0), _stream_ptr(q_lin.device))
     _ffi.check(rc, "pq_rope_append")
     return q_out
 
@@ -61,11 +64,19 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
 
 
 def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """silu(gate) * up; gate and up [..., cols] with unit element stride and a common row stride (they
+    may be the two halves of one fused projection output)."""
     _gpu(gate)
-    assert gate.is_contiguous() and up.is_contiguous() and gate.shape == up.shape and gate.dtype == up.dtype
-    y = torch.empty_like(gate)
+    cols = gate.shape[-1]
+    assert gate.shape == up.shape and gate.dtype == up.dtype and gate.stride(-1) == 1 and up.stride(-1) == 1
+    rows = gate.numel() // cols
+    stride = gate.stride(-2) if gate.dim() > 1 else cols
+    assert up.dim() == gate.dim() and (up.dim() == 1 or up.stride(-2) == stride)
+    assert gate.dim() <= 2 or all(gate.stride(i) == gate.stride(i + 1) * gate.shape[i + 1] for i in range(gate.dim() - 2)), \
+        "rows must be evenly spaced"
+    y = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
     with torch.cuda.device(gate.device):
-        rc = _ffi.lib().pq_silu_mul(gate.data_ptr(), up.data_ptr(), y.data_ptr(), gate.numel(), _dtype_code(gate),
+        rc = _ffi.lib().pq_silu_mul(gate.data_ptr(), up.data_ptr(), y.data_ptr(), rows, cols, stride, _dtype_code(gate),
                                     _stream_ptr(gate.device))
     _ffi.check(rc, "pq_silu_mul")
     return y

@@ -163,7 +163,7 @@ def test_validate_value_quantizer_and_v4_attention(lib):
 
 def test_fused_decode_ops_reject_bad_arguments(lib):
     """Argument checks of the elementwise entry points run before any launch."""
-    ok = [P, P, P, P, P, 4096, P, P, P, 128, P, P, 4096, P, 2, 32, 8, 0, None]
+    ok = [P, P, P, P, P, 4096, P, P, P, 128, P, P, 4096, P, 2, 32, 8, 0, 0, 0, None]
     def bad(i, v):
         a = list(ok); a[i] = v
         return lib.pq_rope_append(*a)
@@ -172,15 +172,17 @@ def test_fused_decode_ops_reject_bad_arguments(lib):
     assert bad(14, 0) == -2 and bad(15, 0) == -2 and bad(16, 0) == -2
     assert bad(17, 2) == -4
     assert bad(5, 0) == -6 and bad(9, 0) == -6 and bad(12, 0) == -6
+    assert bad(18, 100) == -6 and bad(19, 100) == -6                 # row strides shorter than a row
     assert lib.pq_rmsnorm(None, None, P, P, None, 2, 4096, 1e-5, 0, None) == -1
     assert lib.pq_rmsnorm(P, None, None, P, None, 2, 4096, 1e-5, 0, None) == -1
     assert lib.pq_rmsnorm(P, None, P, P, None, 0, 4096, 1e-5, 0, None) == -2
     assert lib.pq_rmsnorm(P, None, P, P, None, 2, 4100, 1e-5, 0, None) == -2      # hidden % 8
     assert lib.pq_rmsnorm(P, None, P, P, None, 2, 4096, 1e-5, 5, None) == -4
     assert lib.pq_rmsnorm(P + 2, None, P, P, None, 2, 4096, 1e-5, 0, None) == -5
-    assert lib.pq_silu_mul(None, P, P, 64, 0, None) == -1
-    assert lib.pq_silu_mul(P, P, P, 0, 0, None) == -2 and lib.pq_silu_mul(P, P, P, 12, 0, None) == -2
-    assert lib.pq_silu_mul(P, P, P, 64, 9, None) == -4 and lib.pq_silu_mul(P, P + 4, P, 64, 0, None) == -5
+    assert lib.pq_silu_mul(None, P, P, 2, 64, 0, 0, None) == -1
+    assert lib.pq_silu_mul(P, P, P, 0, 64, 0, 0, None) == -2 and lib.pq_silu_mul(P, P, P, 2, 12, 0, 0, None) == -2
+    assert lib.pq_silu_mul(P, P, P, 2, 64, 0, 9, None) == -4 and lib.pq_silu_mul(P, P + 4, P, 2, 64, 0, 0, None) == -5
+    assert lib.pq_silu_mul(P, P, P, 2, 64, 32, 0, None) == -6                      # rows would overlap
 
 
 def test_python_wrappers_refuse_cpu_tensors():

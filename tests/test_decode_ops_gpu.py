@@ -91,3 +91,6 @@ def test_silu_mul_matches_eager(gpu, dtype):
     got = silu_mul(g, u)
     assert _ulps_off(got, ref) <= 2, _ulps_off(got, ref)
     assert (got != ref).float().mean().item() < 0.05
+    # the two halves of one fused gate|up projection output
+    gu = torch.cat([g, u], dim=-1)
+    assert torch.equal(silu_mul(gu[..., :14336], gu[..., 14336:]), got)
