@@ -35,9 +35,9 @@ def build_cfg1(dev, dtype=torch.float16):
     return build_workload(1, dev, dtype)
 
 
-def build_workload(idx, dev, dtype=torch.float16, keep_keys=False):
+def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False):
     from polarquant_amd import workloads as wl
-    return wl.build_workload(idx, dev, dtype, keep_keys)
+    return wl.build_workload(idx, dev, dtype, keep_keys, packed)
 
 
 def time_events(fn, steps, warmup):
@@ -181,7 +181,7 @@ def main():
     commons = [[x["q"].data_ptr(), x["codes"].data_ptr(), *[m.data_ptr() for m in x["meta"]], x["codes"].shape[2],
                 x["n_groups"], None, x["kres"].data_ptr(), x["kres"].shape[2], x["n_resid"], None,
                 x["v"].data_ptr(), x["v"].shape[2], None, 0, sm_scale, B, N, Nk, sh.rbits, sh.tbits, _ffi.PQ_F16,
-                n_splits, 0, ws.data_ptr(), ws.numel() * 4] for x in sets]
+                n_splits, 0, ws.data_ptr(), ws.numel() * 4, 0] for x in sets]
 
     def partials_only():
         rc = lib.pq_decode_attn_partials(*commons[turn[0] & 1], _stream_ptr(dev))

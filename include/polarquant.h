@@ -59,6 +59,13 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
                                dtype and written to the metadata tensors like any other, so
                                the decode kernels need no switch.  No reference counterpart. */
 
+/* flag for the decode entry points (and for pq_quantize_groups): the code rows hold 64 packed 6-bit
+ * codes (48 bytes per token, code i in bits [6i, 6i+6) of the row) instead of one byte per code.
+ * For rbits + tbits <= 6; the decode kernels take it for tbits == 3 (the 3/3 configuration).  The
+ * reference stores one byte per pair for every bit width (models/kernel4group.py:1-3); this is the
+ * sub-byte store it announces there.  Code tensors are then [B,Nk,capacity,128,48]. */
+#define PQ_CODES_PACKED6 4u
+
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pq_version(void);
 
@@ -81,12 +88,12 @@ const char *pq_status_string(int status);
  * ------------------------------------------------------------------------- */
 int pq_decode_scores(const void *q, const uint8_t *codes, const void *rscale, const void *rmn,
                      const void *tscale, const void *tmn, float *out,
-                     int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, void *stream);
+                     int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, unsigned flags, void *stream);
 
 /* Host-only argument check of pq_decode_scores (same return codes, launches nothing). */
 int pq_validate_decode_scores(const void *q, const uint8_t *codes, const void *rscale, const void *rmn,
                               const void *tscale, const void *tmn, const float *out,
-                              int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype);
+                              int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, unsigned flags);
 
 /* ---------------------------------------------------------------------------
  * Q — polar quantizer (quantize-on-append and prompt quantization).
@@ -161,6 +168,7 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *            ceil(groups / n_splits)) always covers the sequence.
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
+ *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48)
  * Limits: v_capacity <= 2^24 tokens and group_capacity <= 2^17 groups per (batch, KV head)
  * plane (32-bit byte offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */
@@ -173,7 +181,7 @@ int pq_decode_attn(const void *q,
                    const uint8_t *mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                    int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
-                   void *out, void *stream);
+                   void *out, unsigned flags, void *stream);
 
 int pq_validate_decode_attn(const void *q,
                             const uint8_t *codes, const void *rscale, const void *rmn,
@@ -184,7 +192,7 @@ int pq_validate_decode_attn(const void *q,
                             const uint8_t *mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                             int n_splits, int min_groups_per_split, const void *workspace, size_t workspace_bytes,
-                            const void *out);
+                            const void *out, unsigned flags);
 
 /* The two launches of pq_decode_attn as separate calls, same arguments and
  * checks: pq_decode_attn_partials writes the n_splits partial results
@@ -201,7 +209,8 @@ int pq_decode_attn_partials(const void *q,
                             const void *v, int64_t v_capacity,
                             const uint8_t *mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes, void *stream);
+                            int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
+                            unsigned flags, void *stream);
 
 int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
                          void *out, void *stream);
@@ -247,7 +256,7 @@ int pq_decode_attn_v4(const void *q,
                       const uint8_t *mask, int64_t mask_stride,
                       float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                       int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
-                      void *out, void *stream);
+                      void *out, unsigned flags, void *stream);
 
 /* ---------------------------------------------------------------------------
  * A — the elementwise steps around the attention call of one decode step, each a
@@ -302,7 +311,7 @@ int pq_validate_decode_attn_v4(const void *q,
                                const uint8_t *mask, int64_t mask_stride,
                                float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                                int n_splits, int min_groups_per_split, const void *workspace, size_t workspace_bytes,
-                               const void *out);
+                               const void *out, unsigned flags);
 
 /* Suggested n_splits for a shape (host-only; `max_groups` = largest group count
  * of any sequence, `n_cus` = compute units of the device or 0 for 256). */

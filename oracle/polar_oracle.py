@@ -147,6 +147,31 @@ def quantize_brute_fp64(key_states: torch.Tensor, rbits: int, tbits: int, group_
 
 
 # --------------------------------------------------------------------------
+# Packed 6-bit code rows.  The reference stores one byte per pair code for every
+# bit width and announces a sub-byte store as future work (models/kernel4group.py:1-3);
+# the build's optional packed layout is defined here independently of the kernels:
+# the 64 codes of a token (each < 64) as 384 consecutive bits, code i in bits [6i, 6i+6)
+# of the 48-byte row, little-endian.
+# --------------------------------------------------------------------------
+def pack_codes6(indices: torch.Tensor) -> torch.Tensor:
+    """u8 [..., 64] (values < 64) -> u8 [..., 48]."""
+    assert indices.dtype == torch.uint8 and indices.shape[-1] == 64 and int(indices.max()) < 64
+    c = indices.to(torch.int64).reshape(*indices.shape[:-1], 16, 4)
+    x = c[..., 0] | (c[..., 1] << 6) | (c[..., 2] << 12) | (c[..., 3] << 18)            # 24 bits per 4 codes
+    b = torch.stack([x & 0xFF, (x >> 8) & 0xFF, (x >> 16) & 0xFF], dim=-1)              # 3 bytes, little-endian
+    return b.reshape(*indices.shape[:-1], 48).to(torch.uint8)
+
+
+def unpack_codes6(packed: torch.Tensor) -> torch.Tensor:
+    """u8 [..., 48] -> u8 [..., 64]."""
+    assert packed.dtype == torch.uint8 and packed.shape[-1] == 48
+    b = packed.to(torch.int64).reshape(*packed.shape[:-1], 16, 3)
+    x = b[..., 0] | (b[..., 1] << 8) | (b[..., 2] << 16)
+    c = torch.stack([x & 0x3F, (x >> 6) & 0x3F, (x >> 12) & 0x3F, (x >> 18) & 0x3F], dim=-1)
+    return c.reshape(*packed.shape[:-1], 64).to(torch.uint8)
+
+
+# --------------------------------------------------------------------------
 # dequantize (models/kernel4group.py:151-153; fp32 bin centres as the Triton
 # kernel evaluates them, kernel4group.py:67,73)
 # --------------------------------------------------------------------------

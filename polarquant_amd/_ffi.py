@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(HERE, "libpolarquant_hip.so")
 PQ_F16, PQ_BF16 = 0, 1
 PQ_WRAP_FP32 = 1
 PQ_ANGLE_UNIFORM = 2
+PQ_CODES_PACKED6 = 4
 
 STATUS_NAMES = {
     0: "PQ_OK", -1: "PQ_ERR_NULL_POINTER", -2: "PQ_ERR_BAD_SHAPE", -3: "PQ_ERR_BAD_BITS", -4: "PQ_ERR_BAD_DTYPE",
@@ -27,8 +28,8 @@ STATUS_NAMES = {
 SIGNATURES = {
     "pq_version": (c_int, []),
     "pq_status_string": (c_char_p, [c_int]),
-    "pq_decode_scores": (c_int, [c_void_p] * 7 + [c_int] * 7 + [c_void_p]),
-    "pq_validate_decode_scores": (c_int, [c_void_p] * 7 + [c_int] * 7),
+    "pq_decode_scores": (c_int, [c_void_p] * 7 + [c_int] * 7 + [c_uint, c_void_p]),
+    "pq_validate_decode_scores": (c_int, [c_void_p] * 7 + [c_int] * 7 + [c_uint]),
     "pq_quantize_groups": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_uint]
                            + [c_void_p] * 5 + [c_int, c_int, c_void_p]),
     "pq_validate_quantize_groups": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_uint]
@@ -36,13 +37,13 @@ SIGNATURES = {
     "pq_selftest_quantizer_math": (c_int, [c_int, c_void_p, c_void_p]),
     "pq_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_int64, c_void_p, c_int64, c_float]
-                       + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_void_p]),
+                       + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p]),
     "pq_validate_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
-                                + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
+                                + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint]),
     "pq_decode_attn_partials": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
-                                + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
+                                + [c_int] * 8 + [c_void_p, c_size_t, c_uint, c_void_p]),
     "pq_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "pq_quantize_values": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_int64, c_void_p]),
@@ -51,7 +52,7 @@ SIGNATURES = {
     "pq_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                    c_void_p, c_int64, c_float]
-                          + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_void_p]),
+                          + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p]),
     "pq_validate_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                             c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                             c_void_p, c_int64, c_float]

@@ -39,7 +39,7 @@ def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.
 
 def polar_decode_attention(
     query_states: torch.Tensor,               # [B,N,1,128] or [B,N,128]
-    indices: Optional[torch.Tensor],          # [B,Nk,cap,128,64] u8 (cap >= used groups) or None
+    indices: Optional[torch.Tensor],          # [B,Nk,cap,128,64] u8 (cap >= used groups; last dim 48: packed 6-bit codes) or None
     rscale: Optional[torch.Tensor], rmn: Optional[torch.Tensor],
     tscale: Optional[torch.Tensor], tmn: Optional[torch.Tensor],   # [B,Nk,cap,1,64]
     key_resid: Optional[torch.Tensor],        # [B,Nk,res_cap,128] fp16 keys not yet quantized (new key included)
@@ -74,8 +74,9 @@ def polar_decode_attention(
         assert indices.is_contiguous() and all(m.is_contiguous() for m in (rscale, rmn, tscale, tmn))
         g_cap = indices.shape[2]
         cptr = [indices.data_ptr(), rscale.data_ptr(), rmn.data_ptr(), tscale.data_ptr(), tmn.data_ptr()]
+        flags = _ffi.PQ_CODES_PACKED6 if indices.shape[-1] == 48 else 0      # [.., 128, 48]: packed 6-bit codes
     else:
-        g_cap, cptr = 0, [None] * 5
+        g_cap, cptr, flags = 0, [None] * 5, 0
     if key_resid is not None:
         assert key_resid.is_contiguous() and key_resid.dtype == query_states.dtype
         r_cap, kptr = key_resid.shape[2], key_resid.data_ptr()
@@ -110,7 +111,7 @@ def polar_decode_attention(
         rc = _ffi.lib().pq_decode_attn(
             q.data_ptr(), *cptr, g_cap, n_groups, gps, kptr, r_cap, n_resid, rps,
             value_states.data_ptr(), v_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
-            n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
+            n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn")
     return out
 
@@ -152,8 +153,9 @@ def polar_decode_attention_v4(
         g_cap, v4_cap = indices.shape[2], value_codes.shape[2]
         cptr = [indices.data_ptr(), rscale.data_ptr(), rmn.data_ptr(), tscale.data_ptr(), tmn.data_ptr()]
         vptr = [value_codes.data_ptr(), value_scale.data_ptr(), value_mn.data_ptr()]
+        flags = _ffi.PQ_CODES_PACKED6 if indices.shape[-1] == 48 else 0
     else:
-        g_cap, v4_cap, cptr, vptr = 0, 0, [None] * 5, [None] * 3
+        g_cap, v4_cap, cptr, vptr, flags = 0, 0, [None] * 5, [None] * 3, 0
     mptr, mstride = None, 0
     if attention_mask is not None:
         m8 = attention_mask if attention_mask.dtype == torch.uint8 else (attention_mask != 0).to(torch.uint8)
@@ -173,6 +175,6 @@ def polar_decode_attention_v4(
         rc = _ffi.lib().pq_decode_attn_v4(
             q.data_ptr(), *cptr, g_cap, n_groups, gps, key_resid.data_ptr(), r_cap, n_resid, rps,
             value_resid.data_ptr(), *vptr, v4_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
-            n_splits, min_groups_per_split, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), _stream_ptr(dev))
+            n_splits, min_groups_per_split, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn_v4")
     return out

@@ -5,7 +5,7 @@
   configs[2]  ragged continuous-batch decode attention, Qwen2.5-7B shape (batch 64, GQA 7, 3/3 bits)
   configs[3]  prompt quantization (append) of 131072 keys x 8 KV heads, then one decode step over them
 
-    python -m polarquant_amd.config_bench [--configs 0 2 3] [--values4]
+    python -m polarquant_amd.config_bench [--configs 0 2 3] [--values4] [--packed]
 
 Prints one JSON line per measurement: µs per call, algorithmic bytes, GB/s and fraction of the
 8 TB/s HBM peak.  --values4 adds the decode step with 4-bit values (Mixed variant) for the
@@ -33,8 +33,8 @@ def _line(cfg, op, ms, nbytes, **extra):
                           frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)), flush=True)
 
 
-def run(idx: int, dev, values4: bool, steps: int):
-    w = wl.build_workload(idx, dev, keep_keys=(idx == 3))
+def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
+    w = wl.build_workload(idx, dev, keep_keys=(idx == 3), packed=packed)
     sh = w["shape"]
     B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
     if idx == 0:
@@ -55,11 +55,12 @@ def run(idx: int, dev, values4: bool, steps: int):
         total_groups = int((lens // 128).sum())
     else:
         lq, res, total_groups = [w["n_groups"] * 128] * B, [w["n_resid"]] * B, None
-    nbytes = wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits)
+    nbytes = wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits, code_bytes_per_pair=0.75 if packed else 1.0)
     ms = wl.time_events(lambda: polar_decode_attention(
         w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
         n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups), steps, 10)
-    _line(idx, "decode attention (pq_decode_attn)", ms, nbytes, tokens=int(sum(lq) + sum(res)))
+    _line(idx, "decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else ""), ms, nbytes,
+          tokens=int(sum(lq) + sum(res)))
     if values4 and not sh.ragged:
         L = w["n_groups"] * 128
         vq = quantize_values(w["v"][:, :, :L])
@@ -82,12 +83,16 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--configs", type=int, nargs="*", default=[0, 2, 3])
     ap.add_argument("--values4", action="store_true")
+    ap.add_argument("--packed", action="store_true", help="also run the 3/3-bit configuration with packed 6-bit code rows")
     ap.add_argument("--steps", type=int, default=100)
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     for idx in args.configs:
         run(idx, dev, args.values4, args.steps)
         torch.cuda.empty_cache()
+        if args.packed and wl.CONFIGS[idx].rbits + wl.CONFIGS[idx].tbits <= 6:
+            run(idx, dev, False, args.steps, packed=True)
+            torch.cuda.empty_cache()
 
 
 if __name__ == "__main__":

@@ -287,7 +287,7 @@ struct V4Args {
     int64_t capacity;          // tokens per (batch, KV head) plane
 };
 
-template <typename T, int TB, int REPP, bool V4>
+template <typename T, int TB, int REPP, bool V4, bool PK6>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
 void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                  const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
@@ -373,13 +373,15 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                 qy[j] = ok ? lo2f<T>(qb[j * kHeadDim + kPairs + lane]) : 0.0f;
             }
             const size_t plane = static_cast<size_t>(bh) * group_capacity;
-            const __amdgpu_buffer_rsrc_t rc = make_rsrc(codes + plane * (kGroup * kPairs),
-                                                        static_cast<uint32_t>(nb) * (kGroup * kPairs));
-            const uint32_t voff_c = static_cast<uint32_t>(lane) * kPairs;
+            // a token's code row: 64 bytes, or 48 when the 6-bit codes are stored packed
+            constexpr int kRowB = PK6 ? kPackedRowBytes : kPairs, kRowLoads = kRowB / 16;
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(codes + plane * (kGroup * kRowB),
+                                                        static_cast<uint32_t>(nb) * (kGroup * kRowB));
+            const uint32_t voff_c = static_cast<uint32_t>(lane) * kRowB;
             // software pipeline: codes of the next tile and metadata of the next group are in flight
-            uint4 cnext[4];
+            uint4 cnext[kRowLoads];
 #pragma unroll
-            for (int i = 0; i < 4; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(g0) * (kGroup * kPairs) + 16 * i);
+            for (int i = 0; i < kRowLoads; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(g0) * (kGroup * kRowB) + 16 * i);
             const uint16_t* prs = rscale + plane * kPairs + lane;
             const uint16_t* prm = rmn + plane * kPairs + lane;
             const uint16_t* pts = tscale + plane * kPairs + lane;
@@ -422,14 +424,23 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     // past the last tile of this slice the loads run off the buffer's end and return zeros
                     load_values(half ^ 1, tok0 + kWave, half == 0 || grp + 1 < g1);
                     uint32_t cw[16];
+                    if constexpr (PK6) {
+                        uint32_t pk[12];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        cw[4 * i] = cnext[i].x; cw[4 * i + 1] = cnext[i].y; cw[4 * i + 2] = cnext[i].z; cw[4 * i + 3] = cnext[i].w;
+                        for (int i = 0; i < 3; i++) {
+                            pk[4 * i] = cnext[i].x; pk[4 * i + 1] = cnext[i].y; pk[4 * i + 2] = cnext[i].z; pk[4 * i + 3] = cnext[i].w;
+                        }
+                        unpack6(pk, cw);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            cw[4 * i] = cnext[i].x; cw[4 * i + 1] = cnext[i].y; cw[4 * i + 2] = cnext[i].z; cw[4 * i + 3] = cnext[i].w;
+                        }
                     }
                     if (half == 0 || grp + 1 < g1) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++)
-                            cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(tt + 1) * (kWave * kPairs) + 16 * i);
+                        for (int i = 0; i < kRowLoads; i++)
+                            cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(tt + 1) * (kWave * kRowB) + 16 * i);
                     }
                     float s[REPP];
 #pragma unroll
@@ -585,13 +596,23 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     const float scale_log2 = a.sm_scale * kLog2e;
     V4Args v4{static_cast<const uint32_t*>(a.v4_codes), static_cast<const uint16_t*>(a.v4_scale),
               static_cast<const uint16_t*>(a.v4_zero), a.v4_capacity};
-#define PQ_LAUNCH_V(REPP, V4)                                                                                        \
-    hipLaunchKernelGGL((attn_kernel<T, TB, REPP, V4>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,            \
+#define PQ_LAUNCH_VP(REPP, V4, PK6)                                                                                  \
+    hipLaunchKernelGGL((attn_kernel<T, TB, REPP, V4, PK6>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,       \
                        (const uint16_t*)a.rscale, (const uint16_t*)a.rmn, (const uint16_t*)a.tscale,                 \
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.N, a.Nk, rep,        \
                        a.n_splits, a.min_groups_per_split, a.workspace, v4)
+    // packed 6-bit code rows exist for tbits == 3 only (the 3/3 configuration)
+#define PQ_LAUNCH_V(REPP, V4)                                                                                        \
+    do {                                                                                                             \
+        if constexpr (TB == 3) {                                                                                     \
+            if (a.packed6) PQ_LAUNCH_VP(REPP, V4, true);                                                             \
+            else PQ_LAUNCH_VP(REPP, V4, false);                                                                      \
+        } else {                                                                                                     \
+            PQ_LAUNCH_VP(REPP, V4, false);                                                                           \
+        }                                                                                                            \
+    } while (0)
 #define PQ_LAUNCH(REPP)                                                                                              \
     do {                                                                                                             \
         if (a.v4_codes) PQ_LAUNCH_V(REPP, true);                                                                     \
@@ -605,6 +626,7 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     }
 #undef PQ_LAUNCH
 #undef PQ_LAUNCH_V
+#undef PQ_LAUNCH_VP
     return static_cast<int>(hipGetLastError());
 }
 

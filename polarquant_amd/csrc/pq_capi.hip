@@ -14,6 +14,13 @@ int check_bits(int rbits, int tbits) {
     return PQ_OK;
 }
 
+// decode-side flags: only the packed 6-bit code layout, which exists for tbits == 3 (rbits <= 3)
+int check_decode_flags(unsigned flags, int rbits, int tbits) {
+    if (flags & ~static_cast<unsigned>(PQ_CODES_PACKED6)) return PQ_ERR_BAD_SHAPE;
+    if ((flags & PQ_CODES_PACKED6) && (tbits != 3 || rbits + tbits > 6)) return PQ_ERR_BAD_BITS;
+    return PQ_OK;
+}
+
 int check_heads(int B, int N, int Nk) {
     if (B <= 0 || N <= 0 || Nk <= 0 || N % Nk != 0) return PQ_ERR_BAD_SHAPE;
     if (N / Nk > PQ_MAX_REP) return PQ_ERR_BAD_SHAPE;
@@ -44,8 +51,9 @@ const char* pq_status_string(int status) {
 
 int pq_validate_decode_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn,
                               const void* tscale, const void* tmn, const float* out,
-                              int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype) {
+                              int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, unsigned flags) {
     if (!q || !codes || !rscale || !rmn || !tscale || !tmn || !out) return PQ_ERR_NULL_POINTER;
+    if (int rc = check_decode_flags(flags, rbits, tbits)) return rc;
     if (int rc = check_heads(B, N, Nk)) return rc;
     if (Nb <= 0 || Nb > 65535 || static_cast<long long>(B) * Nk > 0x7fffffffLL) return PQ_ERR_BAD_SHAPE;
     if (int rc = check_bits(rbits, tbits)) return rc;
@@ -58,13 +66,13 @@ int pq_validate_decode_scores(const void* q, const uint8_t* codes, const void* r
 
 int pq_decode_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn,
                      const void* tscale, const void* tmn, float* out,
-                     int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, void* stream) {
-    if (int rc = pq_validate_decode_scores(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, rbits, tbits, dtype))
+                     int B, int N, int Nk, int Nb, int rbits, int tbits, int dtype, unsigned flags, void* stream) {
+    if (int rc = pq_validate_decode_scores(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, rbits, tbits, dtype, flags))
         return rc;
     // grid is (Nb, B*Nk): y is limited to 65535 blocks
     if (static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
     const int err = pq::launch_scores(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, dtype,
-                                      static_cast<hipStream_t>(stream));
+                                      (flags & PQ_CODES_PACKED6) != 0, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
@@ -82,7 +90,8 @@ int pq_validate_quantize_groups(const void* k, const int64_t* k_strides, int dty
         return PQ_ERR_BAD_SHAPE;
     if (rbits < 1 || tbits < 1 || rbits + tbits > 8) return PQ_ERR_BAD_BITS;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
-    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM)) return PQ_ERR_BAD_SHAPE;
+    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM | PQ_CODES_PACKED6)) return PQ_ERR_BAD_SHAPE;
+    if ((flags & PQ_CODES_PACKED6) && rbits + tbits > 6) return PQ_ERR_BAD_BITS;
     if (k_strides[3] != 1) return PQ_ERR_BAD_STRIDE;
     if (k_strides[0] < 0 || k_strides[1] < 0 || k_strides[2] < PQ_HEAD_DIM) return PQ_ERR_BAD_STRIDE;
     if (out_group_offset < 0 || out_group_capacity < out_group_offset + Nb) return PQ_ERR_BAD_STRIDE;
@@ -148,8 +157,9 @@ int pq_validate_decode_attn(const void* q,
                             const uint8_t* mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                             int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
-                            const void* out) {
+                            const void* out, unsigned flags) {
     if (!q || !v || !workspace || !out) return PQ_ERR_NULL_POINTER;
+    if (int rc = check_decode_flags(flags, rbits, tbits)) return rc;
     if (int rc = check_heads(B, N, Nk)) return rc;
     if (static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
     if (int rc = check_bits(rbits, tbits)) return rc;
@@ -188,12 +198,13 @@ int pq_decode_attn_partials(const void* q,
                             const void* v, int64_t v_capacity,
                             const uint8_t* mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes, void* stream) {
+                            int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
+                            unsigned flags, void* stream) {
     // `out` is not touched by this half: validate with a stand-in non-null, aligned pointer
     if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                          mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
-                                         workspace, workspace_bytes, workspace))
+                                         workspace, workspace_bytes, workspace, flags))
         return rc;
     pq::AttnArgs a;
     a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
@@ -202,6 +213,7 @@ int pq_decode_attn_partials(const void* q,
     a.v = v; a.v_capacity = v_capacity; a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
     a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
     a.min_groups_per_split = min_groups_per_split;
+    a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
@@ -229,12 +241,12 @@ int pq_decode_attn(const void* q,
                    const uint8_t* mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                    int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                   void* out, void* stream) {
+                   void* out, unsigned flags, void* stream) {
     if (!out) return PQ_ERR_NULL_POINTER;
     if (int rc = pq_decode_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                          mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
-                                         workspace, workspace_bytes, stream))
+                                         workspace, workspace_bytes, flags, stream))
         return rc;
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
@@ -335,7 +347,7 @@ int pq_validate_decode_attn_v4(const void* q,
                                const uint8_t* mask, int64_t mask_stride,
                                float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                                int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
-                               const void* out) {
+                               const void* out, unsigned flags) {
     // the residual window of values has the same capacity and fill as that of the keys
     const bool any_resid = n_resid_per_seq ? resid_capacity > 0 : n_resid > 0;
     if (any_resid && !v_resid) return PQ_ERR_NULL_POINTER;
@@ -351,7 +363,7 @@ int pq_validate_decode_attn_v4(const void* q,
     return pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                    k_resid, resid_capacity, n_resid, n_resid_per_seq, dummy_v, vcap, mask, mask_stride,
                                    sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
-                                   workspace_bytes, out);
+                                   workspace_bytes, out, flags);
 }
 
 int pq_decode_attn_v4(const void* q,
@@ -364,12 +376,12 @@ int pq_decode_attn_v4(const void* q,
                       const uint8_t* mask, int64_t mask_stride,
                       float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                       int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                      void* out, void* stream) {
+                      void* out, unsigned flags, void* stream) {
     if (int rc = pq_validate_decode_attn_v4(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups,
                                             n_groups_per_seq, k_resid, resid_capacity, n_resid, n_resid_per_seq,
                                             v_resid, v_codes, v_scale, v_zero, v4_capacity, mask, mask_stride, sm_scale,
                                             B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
-                                            workspace_bytes, out))
+                                            workspace_bytes, out, flags))
         return rc;
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     pq::AttnArgs a;
@@ -379,6 +391,7 @@ int pq_decode_attn_v4(const void* q,
     a.mask = mask; a.mask_stride = mask_stride; a.sm_scale = sm_scale;
     a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
     a.min_groups_per_split = min_groups_per_split;
+    a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     if (any_groups) {
         a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token

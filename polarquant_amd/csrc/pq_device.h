@@ -249,6 +249,21 @@ __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes
 }
 #pragma clang diagnostic pop
 
+// Packed 6-bit code rows (PQ_CODES_PACKED6): a token's 64 pair codes, each (rho << tbits) + theta < 64,
+// are stored as 384 consecutive bits (48 bytes, code i in bits [6i, 6i+6)) instead of one byte each.
+// unpack6 rebuilds the byte-per-code words the score loop works on: word c holds codes 4c..4c+3.
+constexpr int kPackedRowBytes = 48;
+__device__ __forceinline__ void unpack6(const uint32_t (&p)[12], uint32_t (&cw)[16]) {
+    static_for<16>([&](auto CC) {
+        constexpr int c = decltype(CC)::value, bit = 24 * c, j = bit >> 5, sh = bit & 31;
+        uint32_t x;
+        if constexpr (sh == 0) x = p[j];
+        else if constexpr (j + 1 < 12) x = __builtin_amdgcn_alignbit(p[j + 1], p[j], sh);
+        else x = p[j] >> sh;
+        cw[c] = (x & 0x3Fu) | ((x << 2) & 0x3F00u) | ((x << 4) & 0x3F0000u) | ((x << 6) & 0x3F000000u);
+    });
+}
+
 // Broadcast the 64 per-pair c_d values (lane d holds c_d) into wave-uniform registers.
 __device__ __forceinline__ void broadcast_cd(float cdv, float (&cds)[kPairs]) {
 #pragma unroll

@@ -8,7 +8,7 @@
 namespace pq {
 
 int launch_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
-                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, hipStream_t st);
+                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, bool packed6, hipStream_t st);
 
 int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int Nk, int Nb, int rbits, int tbits,
                     unsigned flags, uint8_t* codes, void* rscale, void* rmn, void* tscale, void* tmn,
@@ -45,6 +45,7 @@ struct AttnArgs {
     int64_t mask_stride;
     float sm_scale;
     int B, N, Nk, tbits, dtype, n_splits, min_groups_per_split;
+    bool packed6 = false;        // code rows are 48 bytes of packed 6-bit codes (tbits == 3 only)
     float* workspace;
     void* out;
 };

@@ -167,7 +167,7 @@ __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const An
     return (aw | (static_cast<uint32_t>(f2lo<T>(r)) << 16)) & 0x7fff7fffu;
 }
 
-template <typename T, bool UNIFORM>
+template <typename T, bool UNIFORM, bool PK6>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t st, int Nk, int rbits, int tbits, AngleMode am,
     uint8_t* __restrict__ codes, uint16_t* __restrict__ rscale, uint16_t* __restrict__ rmn,
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         ttop[i] = clamp_bound(ts[i], (1 << tbits) - 1);
         rtop[i] = clamp_bound(rs[i], (1 << rbits) - 1);
     }
-    uint8_t* cb = codes + plane * (kGroup * kPairs);
+    uint8_t* cb = codes + plane * (kGroup * (PK6 ? kPackedRowBytes : kPairs));
 #pragma unroll
     for (int it = 0; it < kTokPerThread; it++) {
         uint32_t w = 0;
@@ -289,7 +289,18 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
             const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop[i]);      // :153
             w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
         }
-        *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPairs + 4 * pq4) = w;
+        if constexpr (PK6) {
+            // 4 codes -> 24 bits; the 4 lanes that share 12 bytes of the row assemble its 3 words:
+            // lane 4k+0 writes x0 | x1 << 24, lane 4k+1 x1 >> 8 | x2 << 16, lane 4k+2 x2 >> 16 | x3 << 8
+            const uint32_t x = (w & 0x3Fu) | ((w >> 2) & 0xFC0u) | ((w >> 4) & 0x3F000u) | ((w >> 6) & 0xFC0000u);
+            const uint32_t nx = static_cast<uint32_t>(__shfl_down(static_cast<int>(x), 1));
+            const int k = pq4 & 3;
+            const uint32_t word = (x >> (8 * k)) | (nx << (24 - 8 * k));
+            if (k < 3)
+                *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPackedRowBytes + 12 * (pq4 >> 2) + 4 * k) = word;
+        } else {
+            *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPairs + 4 * pq4) = w;
+        }
     }
 }
 
@@ -336,13 +347,20 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
     };
     am.tmn = round_dt(-3.14159274101257324219f);
     am.tscale = round_dt(round_dt(two_pi_f) / static_cast<float>(1 << tbits));
-#define PQ_LAUNCH_Q(T, U)                                                                                            \
-    hipLaunchKernelGGL((quantize_kernel<T, U>), grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],     \
+    const bool packed6 = (flags & 4u) != 0;
+#define PQ_LAUNCH_QP(T, U, P)                                                                                        \
+    hipLaunchKernelGGL((quantize_kernel<T, U, P>), grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],  \
                        strides[2], Nk, rbits, tbits, am, codes, (uint16_t*)rscale, (uint16_t*)rmn,                  \
                        (uint16_t*)tscale, (uint16_t*)tmn, cap, off)
+#define PQ_LAUNCH_Q(T, U)                                                                                            \
+    do {                                                                                                             \
+        if (packed6) PQ_LAUNCH_QP(T, U, true);                                                                       \
+        else PQ_LAUNCH_QP(T, U, false);                                                                              \
+    } while (0)
     if (dtype == 0) { if (uniform) PQ_LAUNCH_Q(F16, true); else PQ_LAUNCH_Q(F16, false); }
     else            { if (uniform) PQ_LAUNCH_Q(BF16, true); else PQ_LAUNCH_Q(BF16, false); }
 #undef PQ_LAUNCH_Q
+#undef PQ_LAUNCH_QP
     return static_cast<int>(hipGetLastError());
 }
 

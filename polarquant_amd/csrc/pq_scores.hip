@@ -6,7 +6,7 @@
 
 namespace pq {
 
-template <typename T, int TB, int REPP>
+template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) void scores_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                                                        const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
                                                        const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
@@ -20,13 +20,15 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) v
     const int b = bh / Nk, kvh = bh - b * Nk;
     const size_t gidx = static_cast<size_t>(bh) * Nb + grp;
 
-    // token codes of tile 0 and 1 (issued first: longest latency)
-    const uint4* crow = reinterpret_cast<const uint4*>(codes + gidx * (kGroup * kPairs));
-    uint4 cw[2][4];
+    // token codes of tile 0 and 1 (issued first: longest latency); rows of 64 bytes, or 48 when the
+    // 6-bit codes are stored packed
+    constexpr int kRowB = PK6 ? kPackedRowBytes : kPairs, kRowLoads = kRowB / 16;
+    const uint4* crow = reinterpret_cast<const uint4*>(codes + gidx * (kGroup * kRowB));
+    uint4 cw[2][kRowLoads];
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) cw[t][i] = crow[(t * kWave + lane) * 4 + i];
+        for (int i = 0; i < kRowLoads; i++) cw[t][i] = crow[(t * kWave + lane) * kRowLoads + i];
 
     float qx[REPP], qy[REPP];
     const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
@@ -47,10 +49,20 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) v
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         uint32_t cwords[16];
+        if constexpr (PK6) {
+            uint32_t pk[12];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            cwords[4 * i + 0] = cw[t][i].x; cwords[4 * i + 1] = cw[t][i].y;
-            cwords[4 * i + 2] = cw[t][i].z; cwords[4 * i + 3] = cw[t][i].w;
+            for (int i = 0; i < 3; i++) {
+                pk[4 * i + 0] = cw[t][i].x; pk[4 * i + 1] = cw[t][i].y;
+                pk[4 * i + 2] = cw[t][i].z; pk[4 * i + 3] = cw[t][i].w;
+            }
+            unpack6(pk, cwords);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                cwords[4 * i + 0] = cw[t][i].x; cwords[4 * i + 1] = cw[t][i].y;
+                cwords[4 * i + 2] = cw[t][i].z; cwords[4 * i + 3] = cw[t][i].w;
+            }
         }
         float acc[REPP];
 #pragma unroll
@@ -64,13 +76,23 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) v
 
 template <typename T, int TB>
 static int launch_tb(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
-                     const void* tmn, float* out, int B, int N, int Nk, int Nb, hipStream_t st) {
+                     const void* tmn, float* out, int B, int N, int Nk, int Nb, bool packed6, hipStream_t st) {
     const int rep = N / Nk;
     dim3 grid(Nb, B * Nk), block(kWave);
-#define PQ_LAUNCH(REPP)                                                                                         \
-    hipLaunchKernelGGL((scores_kernel<T, TB, REPP>), grid, block, 0, st, (const uint16_t*)q, codes,             \
+#define PQ_LAUNCH_P(REPP, PK6)                                                                                  \
+    hipLaunchKernelGGL((scores_kernel<T, TB, REPP, PK6>), grid, block, 0, st, (const uint16_t*)q, codes,        \
                        (const uint16_t*)rscale, (const uint16_t*)rmn, (const uint16_t*)tscale,                  \
                        (const uint16_t*)tmn, out, N, Nk, Nb, rep)
+    // packed 6-bit code rows exist for tbits == 3 only
+#define PQ_LAUNCH(REPP)                                                                                         \
+    do {                                                                                                        \
+        if constexpr (TB == 3) {                                                                                \
+            if (packed6) PQ_LAUNCH_P(REPP, true);                                                               \
+            else PQ_LAUNCH_P(REPP, false);                                                                      \
+        } else {                                                                                                \
+            PQ_LAUNCH_P(REPP, false);                                                                           \
+        }                                                                                                       \
+    } while (0)
     switch (rep_pad(rep)) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;
@@ -78,24 +100,25 @@ static int launch_tb(const void* q, const uint8_t* codes, const void* rscale, co
         default: PQ_LAUNCH(8); break;
     }
 #undef PQ_LAUNCH
+#undef PQ_LAUNCH_P
     return static_cast<int>(hipGetLastError());
 }
 
 template <typename T>
 static int launch_t(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
-                    const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, hipStream_t st) {
+                    const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, bool packed6, hipStream_t st) {
     switch (tbits) {
-        case 1: return launch_tb<T, 1>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
-        case 2: return launch_tb<T, 2>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
-        case 3: return launch_tb<T, 3>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
-        default: return launch_tb<T, 4>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, st);
+        case 1: return launch_tb<T, 1>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        case 2: return launch_tb<T, 2>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        case 3: return launch_tb<T, 3>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        default: return launch_tb<T, 4>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
     }
 }
 
 int launch_scores(const void* q, const uint8_t* codes, const void* rscale, const void* rmn, const void* tscale,
-                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, hipStream_t st) {
-    return dtype == 0 ? launch_t<F16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, st)
-                      : launch_t<BF16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, st);
+                  const void* tmn, float* out, int B, int N, int Nk, int Nb, int tbits, int dtype, bool packed6, hipStream_t st) {
+    return dtype == 0 ? launch_t<F16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, packed6, st)
+                      : launch_t<BF16>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, tbits, packed6, st);
 }
 
 }  // namespace pq

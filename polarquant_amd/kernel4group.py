@@ -38,8 +38,10 @@ def attention_decode_forward_hip_impl(
         raise RuntimeError("polarquant_amd: decode scores need tensors on the GPU (no CPU fallback)")
     B, Nk, Nb, G, D = indices.shape
     N = query_states.shape[1]
-    if G != 128 or D != 64 or query_states.shape[2] != 1 or query_states.shape[3] != 2 * D:
+    # last dim 64: one byte per pair code (the reference's layout); 48: packed 6-bit codes
+    if G != 128 or D not in (64, 48) or query_states.shape[2] != 1 or query_states.shape[3] != 128:
         raise ValueError("polarquant_amd: expected group 128, head_dim 128 and one query token")
+    flags = _ffi.PQ_CODES_PACKED6 if D == 48 else 0
     if indices.dtype != torch.uint8:
         raise TypeError("indices must be uint8")
     dt = _dtype_code(query_states)
@@ -53,7 +55,7 @@ def attention_decode_forward_hip_impl(
     out = torch.empty((B, N, 1, Nb * G), device=q.device, dtype=torch.float32)
     with torch.cuda.device(q.device):
         rc = _ffi.lib().pq_decode_scores(q.data_ptr(), indices.data_ptr(), *[m.data_ptr() for m in meta],
-                                         out.data_ptr(), B, N, Nk, Nb, rbits, tbits, dt, _stream_ptr(q.device))
+                                         out.data_ptr(), B, N, Nk, Nb, rbits, tbits, dt, flags, _stream_ptr(q.device))
     _ffi.check(rc, "pq_decode_scores")
     return out
 

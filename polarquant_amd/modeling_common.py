@@ -58,6 +58,7 @@ class PolarConfig:
     tbits: int = 4
     vbits: int = 16                     # 4: values in 4 bits as well (the Mixed variant); 16: half-precision values
     snapkv: bool = False                # SnapKV prompt eviction in front of the polar cache (batch 1 decode)
+    packed_codes: bool = False          # 3/3-bit key codes as packed 6-bit rows (48 instead of 64 bytes per token and head)
     cache_capacity: int = 0             # tokens to pre-allocate per layer (0: prompt + 1024, grown by doubling)
 
     @staticmethod
@@ -149,9 +150,11 @@ class MLP(nn.Module):
 class _Arena:
     """Pre-allocated per-layer polar KV cache.  codes/meta/v grow by doubling."""
 
-    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits):
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False):
         self.B, self.Nk, self.dtype, self.device = B, Nk, dtype, device
         self.rbits, self.tbits = rbits, tbits
+        self.packed = packed          # code rows of 48 bytes (packed 6-bit codes) instead of 64
+        self.row = 48 if packed else 64
         self.n_groups = self.n_resid = self.kv_len = 0
         self.pos_offset = 0      # tokens the prompt held beyond the cached ones (SnapKV eviction): tuple[-1] = kv_len + pos_offset
         self.kres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
@@ -161,7 +164,7 @@ class _Arena:
         gcap = (cap_tokens + GROUP - 1) // GROUP
         vcap = gcap * GROUP + GROUP
         B, Nk, dev, dt = self.B, self.Nk, self.device, self.dtype
-        codes = torch.empty(B, Nk, gcap, GROUP, 64, dtype=torch.uint8, device=dev)
+        codes = torch.empty(B, Nk, gcap, GROUP, self.row, dtype=torch.uint8, device=dev)
         meta = [torch.empty(B, Nk, gcap, 1, 64, dtype=dt, device=dev) for _ in range(4)]
         v = torch.empty(B, Nk, vcap, 128, dtype=dt, device=dev)
         if self.kv_len:
@@ -178,7 +181,8 @@ class _Arena:
     def quantize_into(self, keys):
         """keys [B,Nk,n*128,128] (any strides with unit dim stride) -> groups appended."""
         n = keys.shape[2] // GROUP
-        quantize_and_pack_nbit(keys, self.rbits, self.tbits, out=(self.codes, *self.meta), group_offset=self.n_groups)
+        quantize_and_pack_nbit(keys, self.rbits, self.tbits, packed=self.packed, out=(self.codes, *self.meta),
+                               group_offset=self.n_groups)
         self.n_groups += n
 
     def as_tuple(self) -> "PolarCache":
@@ -237,12 +241,16 @@ class PolarGroupAttention(nn.Module):
         self.tbits = _cfg(config, "tbits", 4)
         self.group_size = 128
         self.residual_length = 128
+        # not in the reference (which stores one byte per pair for every bit width, kernel4group.py:1-3):
+        # 3/3-bit codes stored as packed 6-bit rows, indices [B,Nk,Nb,128,48] in the cache tuple
+        self.packed_codes = bool(_cfg(config, "packed_codes", False))
+        assert not self.packed_codes or (self.tbits == 3 and self.rbits + self.tbits <= 6), "packed codes: tbits 3, rbits <= 3"
         self.capture = None   # test hook: a list that receives post-RoPE (q, k, v) of every call
 
     # -- cache plumbing --------------------------------------------------------
     def _new_arena(self, B, dtype, device, tokens):
         cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
-        return _Arena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits)
+        return _Arena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes)
 
     def _arena_of(self, past_key_value, dtype, device) -> _Arena:
         arena = getattr(past_key_value, "arena", None)
@@ -324,14 +332,14 @@ class _MixedArena(_Arena):
     """Per-layer cache of the Mixed variant: polar key groups, 4-bit value rows for the same tokens,
     and a shared 128-token residual window of half-precision keys and values."""
 
-    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits):
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False):
         self.vres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
-        super().__init__(B, Nk, dtype, device, capacity_tokens, rbits, tbits)
+        super().__init__(B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed)
 
     def _alloc(self, cap_tokens):
         gcap = (cap_tokens + GROUP - 1) // GROUP
         B, Nk, dev, dt = self.B, self.Nk, self.device, self.dtype
-        codes = torch.empty(B, Nk, gcap, GROUP, 64, dtype=torch.uint8, device=dev)
+        codes = torch.empty(B, Nk, gcap, GROUP, self.row, dtype=torch.uint8, device=dev)
         meta = [torch.empty(B, Nk, gcap, 1, 64, dtype=dt, device=dev) for _ in range(4)]
         vcodes = torch.empty(B, Nk, gcap * GROUP, 16, dtype=torch.int32, device=dev)
         vmeta = [torch.empty(B, Nk, gcap * GROUP, 1, dtype=dt, device=dev) for _ in range(2)]
@@ -376,7 +384,7 @@ class PolarMixedGroupAttention(PolarGroupAttention):
 
     def _new_arena(self, B, dtype, device, tokens):
         cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
-        return _MixedArena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits)
+        return _MixedArena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes)
 
     def _arena_of(self, past_key_value, dtype, device) -> _MixedArena:
         arena = getattr(past_key_value, "arena", None)
@@ -635,7 +643,8 @@ class PolarForCausalLM(nn.Module):
         c = self.config
         nk = _cfg(c, "num_key_value_heads", c.num_attention_heads)
         v_bytes = 128 // 2 + 2 * 2 if _cfg(c, "vbits", 16) == 4 else 128 * 2      # 4-bit codes + half scale and zero-point
-        return c.num_hidden_layers * nk * (64 + 4 * 64 * 2 // 128 + v_bytes)
+        code_bytes = 48 if _cfg(c, "packed_codes", False) else 64
+        return c.num_hidden_layers * nk * (code_bytes + 4 * 64 * 2 // 128 + v_bytes)
 
 
 # ----------------------------------------------------------------------------- generation (reference :565-666)

@@ -15,7 +15,7 @@ PAIRS = 64
 
 
 def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4, group_size: int = GROUP,
-                           wrap_fp32: bool = False, angle_mode: str = "group",
+                           wrap_fp32: bool = False, angle_mode: str = "group", packed: bool = False,
                            out: Optional[Tuple[torch.Tensor, ...]] = None, group_offset: int = 0):
     """key_states [B,Nk,L,128] half/bf16 on the GPU (any batch/head/token strides, unit dim stride)
     -> (indices u8 [B,Nk,Nb,128,64], rscale, rmn, tscale, tmn [B,Nk,Nb,1,64]).
@@ -27,8 +27,13 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     `angle_mode="group"` is the reference's binning (2^tbits bins over each group's own angle
     range); `"uniform"` uses fixed bins over [-pi, pi) and writes the constants
     tmn = -pi, tscale = 2*pi/2^tbits into the metadata, so decode is unchanged.
+
+    `packed=True` (rbits + tbits <= 6) stores the 64 codes of a token as 48 bytes of packed 6-bit
+    codes ([B,Nk,Nb,128,48]) instead of one byte each; the decode entry points recognise the shape.
     """
     assert angle_mode in ("group", "uniform")
+    assert not packed or rbits + tbits <= 6, "packed 6-bit codes need rbits + tbits <= 6"
+    row = 48 if packed else PAIRS
     if not key_states.is_cuda:
         raise RuntimeError("polarquant_amd: the quantizer needs tensors on the GPU (no CPU fallback)")
     B, Nk, L, D2 = key_states.shape
@@ -40,17 +45,18 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
         key_states = key_states.contiguous()
     dev = key_states.device
     if out is None:
-        codes = torch.empty((B, Nk, Nb, GROUP, PAIRS), dtype=torch.uint8, device=dev)
+        codes = torch.empty((B, Nk, Nb, GROUP, row), dtype=torch.uint8, device=dev)
         meta = [torch.empty((B, Nk, Nb, 1, PAIRS), dtype=key_states.dtype, device=dev) for _ in range(4)]
         cap, off = Nb, 0
     else:
         codes, meta = out[0], list(out[1:])
         cap, off = codes.shape[2], group_offset
-        assert codes.is_contiguous() and all(m.is_contiguous() for m in meta)
+        assert codes.is_contiguous() and all(m.is_contiguous() for m in meta) and codes.shape[-1] == row
     strides = (ctypes.c_int64 * 4)(*key_states.stride())
     with torch.cuda.device(dev):
         rc = _ffi.lib().pq_quantize_groups(key_states.data_ptr(), ctypes.cast(strides, ctypes.c_void_p), dt, B, Nk, Nb,
-                                           rbits, tbits, (_ffi.PQ_WRAP_FP32 if wrap_fp32 else 0) | (_ffi.PQ_ANGLE_UNIFORM if angle_mode == "uniform" else 0),
+                                           rbits, tbits, (_ffi.PQ_WRAP_FP32 if wrap_fp32 else 0) | (_ffi.PQ_ANGLE_UNIFORM if angle_mode == "uniform" else 0)
+                                           | (_ffi.PQ_CODES_PACKED6 if packed else 0),
                                            codes.data_ptr(), *[m.data_ptr() for m in meta], cap, off,
                                            _stream_ptr(dev))
     _ffi.check(rc, "pq_quantize_groups")

@@ -124,7 +124,7 @@ def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], re
 
 
 # ----------------------------------------------------------------------------- GPU-resident workloads and timing
-def build_workload(idx, dev, dtype=torch.float16, keep_keys=False):
+def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False):
     """configs[idx] resident in HBM: polar key cache of L/128 groups per (sequence, KV head),
     fp16 V cache, one new token whose key sits in the fp16 residual buffer.  Ragged shapes
     (configs[2]) carry per-sequence group / residual counts; their caches are sized for the longest."""
@@ -134,7 +134,8 @@ def build_workload(idx, dev, dtype=torch.float16, keep_keys=False):
     B, N, Nk, L = sh.batch, sh.n_heads, sh.n_kv_heads, sh.context
     Nb = L // 128
     g = torch.Generator(device=dev).manual_seed(sh.seed)
-    codes = torch.empty(B, Nk, Nb, 128, 64, dtype=torch.uint8, device=dev)
+    # packed: 6-bit codes stored 48 bytes per token (needs rbits + tbits <= 6, i.e. configs[2])
+    codes = torch.empty(B, Nk, Nb, 128, 48 if packed else 64, dtype=torch.uint8, device=dev)
     meta = [torch.empty(B, Nk, Nb, 1, 64, dtype=dtype, device=dev) for _ in range(4)]
     inv_freq = 1.0 / (sh.rope_theta ** (torch.arange(0, 128, 2, dtype=torch.float32, device=dev) / 128))
     ang = torch.arange(L, dtype=torch.float32, device=dev)[:, None] * inv_freq[None, :]
@@ -145,7 +146,7 @@ def build_workload(idx, dev, dtype=torch.float16, keep_keys=False):
         k = torch.randn(1, Nk, L, 128, generator=g, device=dev, dtype=torch.float32)
         k[..., outl] *= 8.0
         k = (k * cos + torch.cat([-k[..., 64:], k[..., :64]], -1) * sin).to(dtype)
-        quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=(codes[b:b + 1], *[m[b:b + 1] for m in meta]))
+        quantize_and_pack_nbit(k, sh.rbits, sh.tbits, packed=packed, out=(codes[b:b + 1], *[m[b:b + 1] for m in meta]))
         if keep_keys:
             keys.append(k)
     v = torch.empty(B, Nk, L + 1, 128, dtype=dtype, device=dev)

@@ -42,7 +42,7 @@ def test_version_and_status_strings(lib):
 
 
 def test_validate_decode_scores(lib):
-    ok = [P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0]
+    ok = [P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 0]
     assert lib.pq_validate_decode_scores(*ok) == 0
 
     def bad(i, v):
@@ -55,7 +55,11 @@ def test_validate_decode_scores(lib):
     assert bad(13, 2) == -4                                          # dtype
     assert bad(1, P + 4) == -5 and bad(6, P + 2) == -5               # misaligned codes / out
     # the launching entry point runs the same checks before touching the device
-    assert lib.pq_decode_scores(*ok[:11], 5, 4, 0, None) == -3
+    assert lib.pq_decode_scores(*ok[:11], 5, 4, 0, 0, None) == -3
+    # packed 6-bit code rows: tbits == 3 and rbits <= 3 only; unknown flag bits are refused
+    assert lib.pq_validate_decode_scores(*ok[:11], 3, 3, 0, 4) == 0
+    assert lib.pq_validate_decode_scores(*ok[:11], 4, 4, 0, 4) == -3 and lib.pq_validate_decode_scores(*ok[:11], 4, 3, 0, 4) == -3
+    assert lib.pq_validate_decode_scores(*ok[:11], 3, 3, 0, 8) == -2
 
 
 def test_validate_quantize_groups(lib):
@@ -72,7 +76,10 @@ def test_validate_quantize_groups(lib):
     assert bad(6, 5) == -3 and bad(7, 0) == -3
     assert bad(2, 7) == -4
     assert bad(8, 1) == 0 and bad(8, 2) == 0 and bad(8, 3) == 0   # PQ_WRAP_FP32, PQ_ANGLE_UNIFORM
-    assert bad(8, 4) == -2                           # unknown flag bit
+    assert bad(8, 4) == -3                           # packed 6-bit codes need rbits + tbits <= 6
+    a = list(ok); a[6], a[7], a[8] = 3, 3, 4
+    assert lib.pq_validate_quantize_groups(*a) == 0
+    assert bad(8, 8) == -2                           # unknown flag bit
     assert bad(14, 1) == -6 and bad(15, 1) == -6     # capacity < offset + Nb
     assert bad(0, P + 2) == -5                       # key pointer not 8-byte aligned
     for i, s in enumerate([(8 * 256 * 128, 256 * 128, 128, 2), (8 * 256 * 128, 256 * 128, 64, 1),
@@ -90,8 +97,12 @@ def test_validate_decode_attn_and_plan(lib):
     B, N, Nk, ns = 2, 32, 8, 4
     wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
     assert wsb == B * N * ns * 132 * 4
-    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, 1024, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P]
+    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, 1024, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P, 0]
     assert lib.pq_validate_decode_attn(*ok) == 0
+    a = list(ok); a[21], a[22], a[29] = 3, 3, 4
+    assert lib.pq_validate_decode_attn(*a) == 0                      # packed 6-bit codes with 3/3 bits
+    a[21] = 4
+    assert lib.pq_validate_decode_attn(*a) == -3
 
     def bad(i, v):
         a = list(ok); a[i] = v
@@ -142,7 +153,7 @@ def test_validate_value_quantizer_and_v4_attention(lib):
 
     B, N, Nk, ns = 2, 32, 8, 4
     wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
-    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, P, P, P, 512, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P]
+    ok = [P, P, P, P, P, P, 4, 3, None, P, 128, 5, None, P, P, P, P, 512, None, 0, 0.088, B, N, Nk, 4, 4, 0, ns, 0, P, wsb, P, 0]
     assert lib.pq_validate_decode_attn_v4(*ok) == 0
 
     def bad4(i, v):

@@ -464,3 +464,20 @@ def test_snapkv_cache_bookkeeping(L):
         # decode continues at position L and appends to the 1152 cached tokens
         out, c2 = po.decode_step(wl.make_half((1, 4, 1, 128), g), k[:, :, :1], v[:, :, :1], cache)
         assert c2[-1] == L + 1 and c2[6].shape[2] == 1153 and c2[0].shape[2] == 1
+
+
+# ------------------------------------------------------------------ packed 6-bit code rows
+def test_packed6_layout_known_answer_and_round_trip():
+    """Code i of a row sits in bits [6i, 6i+6) of the 48-byte row (little-endian): checked on rows
+    with a single non-zero code against the bit position computed by hand, then as a round trip."""
+    for i, val in [(0, 63), (1, 1), (4, 33), (5, 63), (21, 42), (63, 63)]:
+        row = torch.zeros(64, dtype=torch.uint8)
+        row[i] = val
+        packed = po.pack_codes6(row)
+        assert packed.shape == (48,)
+        bits = sum(int(b) << (8 * j) for j, b in enumerate(packed.tolist()))
+        assert bits == val << (6 * i)
+    g = torch.Generator().manual_seed(3)
+    codes = torch.randint(0, 64, (2, 3, 5, 128, 64), generator=g, dtype=torch.uint8)
+    packed = po.pack_codes6(codes)
+    assert packed.shape == (2, 3, 5, 128, 48) and torch.equal(po.unpack_codes6(packed), codes)
