@@ -66,6 +66,11 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * sub-byte store it announces there.  Code tensors are then [B,Nk,capacity,128,48]. */
 #define PQ_CODES_PACKED6 4u
 
+/* Layout converter for code rows: pack != 0 turns `n_rows` byte-per-code rows (64 bytes each, every
+ * code < 64) into packed 6-bit rows (48 bytes each), pack == 0 the reverse.  For caches built by the
+ * reference (always byte-per-code) that are to be kept packed, and back.  No reference counterpart. */
+int pq_convert_codes6(const uint8_t *src, uint8_t *dst, size_t n_rows, int pack, void *stream);
+
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
 int pq_version(void);
 

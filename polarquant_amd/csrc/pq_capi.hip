@@ -294,6 +294,14 @@ int pq_silu_mul(const void* gate, const void* up, void* y, int rows, int cols, i
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
+int pq_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, int pack, void* stream) {
+    if (!src || !dst) return PQ_ERR_NULL_POINTER;
+    if (n_rows == 0 || n_rows > (size_t{1} << 40)) return PQ_ERR_BAD_SHAPE;
+    if (!aligned(src, pack ? 16 : 4) || !aligned(dst, pack ? 4 : 16)) return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_convert_codes6(src, dst, n_rows, pack != 0, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;

@@ -162,6 +162,42 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
     *reinterpret_cast<uint4*>(y + out) = make_uint4(yo[0], yo[1], yo[2], yo[3]);
 }
 
+// Layout converters between byte-per-code rows (64 B per token, the reference's store) and packed
+// 6-bit rows (48 B).  One thread converts a quarter row: 16 codes = 16 bytes <-> 12 bytes.
+__global__ __launch_bounds__(256) void pack_codes6_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n_quarters) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_quarters) return;
+    const uint4 v = *reinterpret_cast<const uint4*>(src + i * 16);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t x[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) x[c] = (w[c] & 0x3Fu) | ((w[c] >> 2) & 0xFC0u) | ((w[c] >> 4) & 0x3F000u) | ((w[c] >> 6) & 0xFC0000u);
+    uint32_t* o = reinterpret_cast<uint32_t*>(dst + i * 12);
+    o[0] = x[0] | (x[1] << 24);
+    o[1] = (x[1] >> 8) | (x[2] << 16);
+    o[2] = (x[2] >> 16) | (x[3] << 8);
+}
+
+__global__ __launch_bounds__(256) void unpack_codes6_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, size_t n_quarters) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n_quarters) return;
+    const uint32_t* p = reinterpret_cast<const uint32_t*>(src + i * 12);
+    const uint32_t a = p[0], b = p[1], c = p[2];
+    const uint32_t x[4] = {a & 0xFFFFFFu, (a >> 24) | ((b & 0xFFFFu) << 8), (b >> 16) | ((c & 0xFFu) << 16), c >> 8};
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) w[k] = (x[k] & 0x3Fu) | ((x[k] << 2) & 0x3F00u) | ((x[k] << 4) & 0x3F0000u) | ((x[k] << 6) & 0x3F000000u);
+    *reinterpret_cast<uint4*>(dst + i * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+int launch_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, bool pack, hipStream_t st) {
+    const size_t nq = n_rows * 4;
+    const unsigned blocks = static_cast<unsigned>((nq + 255) / 256);
+    if (pack) hipLaunchKernelGGL(pack_codes6_kernel, dim3(blocks), dim3(256), 0, st, src, dst, nq);
+    else hipLaunchKernelGGL(unpack_codes6_kernel, dim3(blocks), dim3(256), 0, st, src, dst, nq);
+    return static_cast<int>(hipGetLastError());
+}
+
 int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_tab, const void* sin_tab,
                        const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
                        void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int64_t max_pos, int dtype,

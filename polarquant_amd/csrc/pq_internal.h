@@ -27,6 +27,8 @@ int launch_rmsnorm(const void* x, const void* res, const void* w, void* y, void*
                    int dtype, hipStream_t st);
 int launch_silu_mul(const void* gate, const void* up, void* y, int rows, int cols, int64_t in_stride, int dtype, hipStream_t st);
 
+int launch_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, bool pack, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;

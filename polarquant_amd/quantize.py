@@ -64,3 +64,17 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
         return (codes, *meta)
     sl = slice(off, off + Nb)
     return (codes[:, :, sl], *[m[:, :, sl] for m in meta])
+
+
+def convert_codes6(indices: torch.Tensor, pack: bool) -> torch.Tensor:
+    """Byte-per-code rows [..., 64] (codes < 64) -> packed 6-bit rows [..., 48] (pack=True), or back."""
+    if not indices.is_cuda:
+        raise RuntimeError("polarquant_amd: the layout converter needs tensors on the GPU (no CPU fallback)")
+    src_row, dst_row = (PAIRS, 48) if pack else (48, PAIRS)
+    assert indices.dtype == torch.uint8 and indices.shape[-1] == src_row
+    src = indices.contiguous()
+    dst = torch.empty(src.shape[:-1] + (dst_row,), dtype=torch.uint8, device=src.device)
+    with torch.cuda.device(src.device):
+        rc = _ffi.lib().pq_convert_codes6(src.data_ptr(), dst.data_ptr(), src.numel() // src_row, int(pack), _stream_ptr(src.device))
+    _ffi.check(rc, "pq_convert_codes6")
+    return dst

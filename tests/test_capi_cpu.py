@@ -196,6 +196,12 @@ def test_fused_decode_ops_reject_bad_arguments(lib):
     assert lib.pq_silu_mul(P, P, P, 2, 64, 32, 0, None) == -6                      # rows would overlap
 
 
+def test_convert_codes6_rejects_bad_arguments(lib):
+    assert lib.pq_convert_codes6(None, P, 4, 1, None) == -1 and lib.pq_convert_codes6(P, None, 4, 0, None) == -1
+    assert lib.pq_convert_codes6(P, P, 0, 1, None) == -2
+    assert lib.pq_convert_codes6(P + 4, P, 4, 1, None) == -5 and lib.pq_convert_codes6(P, P + 4, 4, 0, None) == -5
+
+
 def test_python_wrappers_refuse_cpu_tensors():
     import torch
     from polarquant_amd.attention import polar_decode_attention

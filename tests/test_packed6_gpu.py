@@ -121,3 +121,13 @@ def test_attention_class_with_packed_codes_equals_the_plain_one(gpu):
         assert (ca[j] is None and cb[j] is None) or torch.equal(ca[j], cb[j])
     m = Qwen2PolarForCausalLM(PolarConfig(packed_codes=True, **kw))
     assert m.kv_cache_bytes_per_token() == 1 * 1 * (48 + 4 + 256)
+
+
+def test_layout_converters_round_trip(gpu):
+    from polarquant_amd.quantize import convert_codes6
+    g = torch.Generator().manual_seed(64)
+    codes = torch.randint(0, 64, (2, 3, 5, 128, 64), generator=g, dtype=torch.uint8)
+    packed = convert_codes6(codes.to(gpu), pack=True)
+    assert packed.shape == (2, 3, 5, 128, 48) and torch.equal(packed.cpu(), po.pack_codes6(codes))
+    back = convert_codes6(packed, pack=False)
+    assert torch.equal(back.cpu(), codes)
