@@ -135,7 +135,11 @@ int pq_validate_quantize_groups(const void *k, const int64_t *k_strides, int dty
  * ALL 2^32 (y, x) operand pairs of the dtype (NaNs skipped) and adds to
  * counters[0] the number of pairs whose rounded angle or radius differ (must stay
  * 0) and to counters[1] the number of pairs that needed the exact routine.
- * `counters`: device uint64[2], zeroed by the caller. Takes ~0.1 s. */
+ * Both quantizers also replace the fp32 division by a scale with a reciprocal and
+ * two fused multiply-adds; counters[2] receives the number of (dividend, scale)
+ * pairs of the dtype, over the whole range the quantizers can meet, whose
+ * quotient rounded to the dtype differs from the divided one (must stay 0).
+ * `counters`: device uint64[3], zeroed by the caller. Takes ~0.1 s. */
 int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
 
 /* ---------------------------------------------------------------------------

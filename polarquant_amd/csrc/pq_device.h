@@ -46,6 +46,34 @@ template <> __device__ __forceinline__ uint16_t f2lo<BF16>(float f) {
     return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
+// ---- division of two key-dtype values, rounded to the key dtype ----------------
+// Eager torch evaluates a / b on half / bfloat16 tensors as round_dtype(fp32 quotient).  The
+// IEEE fp32 division is ~10 instructions; the quantizers divide every element by a scale that
+// is shared by many elements, so they use instead
+//     q0 = d * inv,  r = fma(-q0, sc, d),  q1 = fma(r, inv, q0),      inv = v_rcp_f32(sc) (1 ulp)
+// q1 is a faithful fp32 quotient (the residual r is exact, so q1 is the rounding of a value
+// within 2^-46 of d / sc).  It may differ from the correctly rounded fp32 quotient in the last
+// bit, but never across a rounding boundary of the dtype: such a boundary t has at most 12
+// significant bits and sc 11 (9 and 8 for bfloat16), so t * sc is exact in fp32 arithmetic and
+// d / sc is either exactly t (then q1 == t as well) or more than 2 fp32 ulps away from it.
+// Hence round_dtype(q1) == round_dtype(RN32(d / sc)).  Conditions: sc finite, positive and far
+// from the ends of the fp32 range (fast_div_ok), d finite with d / sc far below overflow; callers
+// take the plain division otherwise.  pq_selftest_quantizer_math checks the identity on the
+// device for every operand pair of the dtype that meets them.
+__device__ __forceinline__ bool fast_div_ok(float sc) { return sc >= 0x1p-100f && sc <= 0x1p100f; }
+__device__ __forceinline__ float div_faithful(float d, float sc, float inv) {
+    const float q0 = d * inv;
+    const float r = __builtin_fmaf(-q0, sc, d);
+    return __builtin_fmaf(r, inv, q0);
+}
+
+// v of lane (l & ~15) | ((l + N) & 15): a rotation inside each row of 16 lanes, as a DPP
+// modifier of a move instead of a trip through the LDS crossbar
+template <int N>
+__device__ __forceinline__ uint32_t row_rotate(uint32_t v) {
+    return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x120 | N, 0xf, 0xf, true));
+}
+
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [0, N).  Unlike
 // "#pragma unroll" the indices are constants when the body is instantiated, so
 // register arrays indexed by them never fall back to scratch memory.

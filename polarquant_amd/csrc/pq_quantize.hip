@@ -33,6 +33,8 @@ __device__ __forceinline__ float rnd(float f) { return lo2f<T>(f2lo<T>(f)); }
 // special operands (zeros, infinities, NaNs, results below the dtype's normal
 // range), take the exact path.  That the two paths agree on EVERY pair of half /
 // bfloat16 operands is checked exhaustively on the device by pq_selftest_quantizer_math.
+template <typename T> struct IsHalf { static constexpr bool value = false; };
+template <> struct IsHalf<F16> { static constexpr bool value = true; };
 template <typename T> struct DT;
 template <> struct DT<F16> { static constexpr uint32_t kLowMask = 0x1fffu, kMid = 0x1000u; static constexpr float kMinNormal = 6.103515625e-05f; };
 template <> struct DT<BF16> { static constexpr uint32_t kLowMask = 0xffffu, kMid = 0x8000u; static constexpr float kMinNormal = 1.17549435e-38f; };
@@ -73,11 +75,14 @@ __device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out
     const float ss = __builtin_fmaf(x, x, y * y);          // x*x, y*y are exact for half/bf16 operands
     const float a = atan2_fast(y, x);
     const float r = __builtin_amdgcn_sqrtf(ss);
-    // zeros, infinities, NaNs, and magnitudes (bfloat16 only) at which the reciprocal or the
-    // hardware square root leave their accurate range
+    // Infinities, NaNs, and (bfloat16 only) magnitudes at which the reciprocal or the hardware
+    // square root leave their accurate range: one comparison for half, whose finite squares all lie
+    // inside (2^-80, 2^80).  Zeros need no test of their own: with one zero operand the estimate is
+    // exactly 0, pi/2 or pi like the exact routine's (0 then fails the kMinNormal test below), and
+    // x == y == 0 gives a NaN angle with radius 0, which fails that test as well.
     // (bitwise | on purpose: one straight-line predicate instead of a chain of exec-mask branches)
-    const int in_range = static_cast<int>(ss > 0x1p-80f) & static_cast<int>(ss < 0x1p80f);
-    const int special = (in_range ^ 1) | static_cast<int>(fminf(fabsf(x), fabsf(y)) == 0.0f);
+    int special = static_cast<int>(!(ss < 0x1p80f));
+    if constexpr (!IsHalf<T>::value) special |= static_cast<int>(!(ss > 0x1p-80f));
     *a_out = a;
     *r_out = r;
     return (special | static_cast<int>(fminf(fabsf(a), r) < DT<T>::kMinNormal) |
@@ -111,6 +116,13 @@ template <typename T>
 __device__ __forceinline__ uint32_t code_of(float v, float mn, float scale, float topf) {
     const float d = rnd<T>(v - mn);
     const float qf = floorf(rnd<T>(d / scale));
+    return static_cast<uint32_t>(__builtin_amdgcn_fmed3f(qf, 0.0f, topf));
+}
+// The same with div_faithful in place of the division; `inv` = v_rcp_f32(scale), scale accepted by fast_div_ok.
+template <typename T>
+__device__ __forceinline__ uint32_t code_of_fast(float v, float mn, float scale, float inv, float topf) {
+    const float d = rnd<T>(v - mn);
+    const float qf = floorf(rnd<T>(div_faithful(d, scale, inv)));
     return static_cast<uint32_t>(__builtin_amdgcn_fmed3f(qf, 0.0f, topf));
 }
 __device__ __forceinline__ float clamp_bound(float scale, int top) { return scale > 0.0f ? static_cast<float>(top) : 0.0f; }
@@ -159,7 +171,7 @@ __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const An
     float phi = rnd<T>(a);
     uint32_t aw;
     if constexpr (UNIFORM) {
-        aw = code_of<T>(phi, am.tmn, am.tscale, static_cast<float>(am.ttop));
+        aw = code_of_fast<T>(phi, am.tmn, am.tscale, __builtin_amdgcn_rcpf(am.tscale), static_cast<float>(am.ttop));
     } else {
         if (phi < 0.0f) phi = rnd<T>(phi + am.two_pi);             // :144
         aw = f2lo<T>(phi);
@@ -277,18 +289,16 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         rtop[i] = clamp_bound(rs[i], (1 << rbits) - 1);
     }
     uint8_t* cb = codes + plane * (kGroup * (PK6 ? kPackedRowBytes : kPairs));
+    // scales of 0 (degenerate pairs), infinities and the far ends of the bfloat16 range take the division
+    bool fast = true;
+    float tinv[4], rinv[4];
 #pragma unroll
-    for (int it = 0; it < kTokPerThread; it++) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t v = pr[it * 4 + i][tid];
-            const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
-            const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
-            const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop[i]);    // :148
-            const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop[i]);      // :153
-            w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
-        }
+    for (int i = 0; i < 4; i++) {
+        fast = fast && fast_div_ok(ts[i]) && fast_div_ok(rs[i]);
+        tinv[i] = __builtin_amdgcn_rcpf(ts[i]);
+        rinv[i] = __builtin_amdgcn_rcpf(rs[i]);
+    }
+    auto store_codes = [&](int it, uint32_t w) {
         if constexpr (PK6) {
             // 4 codes -> 24 bits; the 4 lanes that share 12 bytes of the row assemble its 3 words:
             // lane 4k+0 writes x0 | x1 << 24, lane 4k+1 x1 >> 8 | x2 << 16, lane 4k+2 x2 >> 16 | x3 << 8
@@ -300,6 +310,38 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
                 *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPackedRowBytes + 12 * (pq4 >> 2) + 4 * k) = word;
         } else {
             *reinterpret_cast<uint32_t*>(cb + (it * 16 + tl) * kPairs + 4 * pq4) = w;
+        }
+    };
+    // PK6 exchanges words between lanes, so the whole wavefront takes one side together
+    if (__builtin_expect(PK6 ? __all(fast) : fast, 1)) {
+#pragma unroll
+        for (int it = 0; it < kTokPerThread; it++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t v = pr[it * 4 + i][tid];
+                const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
+                const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
+                const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of_fast<T>(phi, tm[i], ts[i], tinv[i], ttop[i]);    // :148
+                const uint32_t rh = code_of_fast<T>(r, rm[i], rs[i], rinv[i], rtop[i]);      // :153
+                w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
+            }
+            store_codes(it, w);
+        }
+    } else {
+#pragma unroll
+        for (int it = 0; it < kTokPerThread; it++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t v = pr[it * 4 + i][tid];
+                const float phi = lo2f<T>(static_cast<uint16_t>(v & 0xffffu));
+                const float r = lo2f<T>(static_cast<uint16_t>(v >> 16));
+                const uint32_t th = UNIFORM ? (v & 0xffffu) : code_of<T>(phi, tm[i], ts[i], ttop[i]);    // :148
+                const uint32_t rh = code_of<T>(r, rm[i], rs[i], rtop[i]);      // :153
+                w |= (((rh << tbits) + th) & 0xffu) << (8 * i);             // :155
+            }
+            store_codes(it, w);
         }
     }
 }
@@ -325,9 +367,35 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* misma
     if (slow) atomicAdd(slow_lanes, static_cast<unsigned long long>(slow));
 }
 
+// Exhaustive check of div_faithful: block == bit pattern of the dividend d, thread t covers the
+// divisor patterns t, t+256, ...  Pairs the quantizers can meet: divisor accepted by fast_div_ok,
+// 0 <= d <= 1024 * sc (d is a distance from the group minimum and sc the group's range over at
+// most 2^8 bins).  Quotients below 1/4 may differ in denormal digits; floor() and rint() of both
+// are 0 there, which is all the quantizers take from them.
+template <typename T>
+__global__ __launch_bounds__(256) void selftest_div_kernel(unsigned long long* mismatches) {
+    const float d = lo2f<T>(static_cast<uint16_t>(blockIdx.x));
+    unsigned int bad = 0;
+    if (d >= 0.0f && d < INFINITY) {
+        for (uint32_t sb = threadIdx.x; sb < 65536u; sb += 256u) {
+            const float sc = lo2f<T>(static_cast<uint16_t>(sb));
+            if (!fast_div_ok(sc) || !(d <= 1024.0f * sc)) continue;
+            const float exact = rnd<T>(d / sc);
+            const float fast = rnd<T>(div_faithful(d, sc, __builtin_amdgcn_rcpf(sc)));
+            bad += (exact != fast) && !(exact < 0.25f && fast < 0.25f);
+        }
+    }
+    if (bad) atomicAdd(mismatches, static_cast<unsigned long long>(bad));
+}
+
 int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st) {
-    if (dtype == 0) hipLaunchKernelGGL(selftest_kernel<F16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
-    else hipLaunchKernelGGL(selftest_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+    if (dtype == 0) {
+        hipLaunchKernelGGL(selftest_kernel<F16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+        hipLaunchKernelGGL(selftest_div_kernel<F16>, dim3(65536), dim3(256), 0, st, counters + 2);
+    } else {
+        hipLaunchKernelGGL(selftest_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+        hipLaunchKernelGGL(selftest_div_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters + 2);
+    }
     return static_cast<int>(hipGetLastError());
 }
 

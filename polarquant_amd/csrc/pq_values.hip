@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
     if (live) w = *reinterpret_cast<const uint4*>(v + b * sb + h * sh + static_cast<int64_t>(t) * st + 8 * n);
     if constexpr (IsF16<T>::value) {
         // half precision: the eager ops ARE half-precision instructions here (v_pk_min/max_f16,
-        // v_sub_f16, the compiler's correctly rounded half division, v_med3_f16, v_rndne_f16)
+        // v_sub_f16, v_med3_f16, v_rndne_f16); the division is div_faithful
         typedef _Float16 half2v __attribute__((ext_vector_type(2)));
         const half2v p0 = __builtin_bit_cast(half2v, w.x), p1 = __builtin_bit_cast(half2v, w.y);
         const half2v p2 = __builtin_bit_cast(half2v, w.z), p3 = __builtin_bit_cast(half2v, w.w);
@@ -47,23 +47,40 @@ __global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
         // (min, -max) in one register: both reduce with a packed min
         half2v red = {live ? (mn2.x < mn2.y ? mn2.x : mn2.y) : static_cast<_Float16>(INFINITY),
                       live ? -(mx2.x > mx2.y ? mx2.x : mx2.y) : static_cast<_Float16>(INFINITY)};
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) {
-            const int other = __shfl_xor(__builtin_bit_cast(int, red), o);
-            red = __builtin_elementwise_min(red, __builtin_bit_cast(half2v, other));
+        {
+            uint32_t rw = __builtin_bit_cast(uint32_t, red);
+            static_for<4>([&](auto s) {
+                const uint32_t other = row_rotate<(1 << decltype(s)::value)>(rw);
+                rw = __builtin_bit_cast(uint32_t, __builtin_elementwise_min(__builtin_bit_cast(half2v, rw), __builtin_bit_cast(half2v, other)));
+            });
+            red = __builtin_bit_cast(half2v, rw);
         }
         if (!live) return;
         const _Float16 lo = red.x, hi = -red.y;
         const _Float16 sc = static_cast<_Float16>(hi - lo) / static_cast<_Float16>(15.0f);
         const half2v ps[4] = {p0, p1, p2, p3};
+        const float scf = static_cast<float>(sc);
         uint32_t word = 0;
+        if (__builtin_expect(fast_div_ok(scf), 1)) {
+            const float inv = __builtin_amdgcn_rcpf(scf);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const _Float16 x = (i & 1) ? ps[i >> 1].y : ps[i >> 1].x;
-            _Float16 q = static_cast<_Float16>(x - lo) / sc;
-            q = __builtin_amdgcn_fmed3h(q, static_cast<_Float16>(0.0f), static_cast<_Float16>(15.0f));   // NaN (0/0) -> 0
-            q = __builtin_rintf16(q);                      // round half to even
-            word |= static_cast<uint32_t>(static_cast<unsigned short>(q)) << (4 * i);
+            for (int i = 0; i < 8; i++) {
+                const _Float16 x = (i & 1) ? ps[i >> 1].y : ps[i >> 1].x;
+                _Float16 q = static_cast<_Float16>(div_faithful(static_cast<float>(static_cast<_Float16>(x - lo)), scf, inv));
+                q = __builtin_amdgcn_fmed3h(q, static_cast<_Float16>(0.0f), static_cast<_Float16>(15.0f));
+                q = __builtin_rintf16(q);                      // round half to even
+                word |= static_cast<uint32_t>(static_cast<unsigned short>(q)) << (4 * i);
+            }
+        } else {
+            // constant rows (0/0), scales that underflow to 0 (x/0), infinities
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const _Float16 x = (i & 1) ? ps[i >> 1].y : ps[i >> 1].x;
+                _Float16 q = static_cast<_Float16>(x - lo) / sc;
+                q = __builtin_amdgcn_fmed3h(q, static_cast<_Float16>(0.0f), static_cast<_Float16>(15.0f));   // NaN (0/0) -> 0
+                q = __builtin_rintf16(q);
+                word |= static_cast<uint32_t>(static_cast<unsigned short>(q)) << (4 * i);
+            }
         }
         codes[row * 16 + n] = static_cast<int32_t>(word);
         if (n == 0) { scale[row] = __builtin_bit_cast(uint16_t, sc); mn[row] = __builtin_bit_cast(uint16_t, lo); }
@@ -80,20 +97,30 @@ __global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
 #pragma unroll
             for (int i = 0; i < 8; i++) { lo = fminf(lo, x[i]); hi = fmaxf(hi, x[i]); }
         }
-#pragma unroll
-        for (int o = 1; o < 16; o <<= 1) {
-            lo = fminf(lo, __shfl_xor(lo, o));
-            hi = fmaxf(hi, __shfl_xor(hi, o));
-        }
+        static_for<4>([&](auto s) {
+            lo = fminf(lo, __uint_as_float(row_rotate<(1 << decltype(s)::value)>(__float_as_uint(lo))));
+            hi = fmaxf(hi, __uint_as_float(row_rotate<(1 << decltype(s)::value)>(__float_as_uint(hi))));
+        });
         if (!live) return;
         const float sc = rnd_v<T>(rnd_v<T>(hi - lo) / 15.0f);
         uint32_t word = 0;
+        if (__builtin_expect(fast_div_ok(sc), 1)) {
+            const float inv = __builtin_amdgcn_rcpf(sc);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            float q = rnd_v<T>(rnd_v<T>(x[i] - lo) / sc);
-            q = __builtin_amdgcn_fmed3f(q, 0.0f, 15.0f);   // NaN (0/0 on a constant row) comes out as the minimum, 0
-            q = __builtin_rintf(q);                        // round half to even
-            word |= static_cast<uint32_t>(q) << (4 * i);
+            for (int i = 0; i < 8; i++) {
+                float q = rnd_v<T>(div_faithful(rnd_v<T>(x[i] - lo), sc, inv));
+                q = __builtin_amdgcn_fmed3f(q, 0.0f, 15.0f);
+                q = __builtin_rintf(q);                        // round half to even
+                word |= static_cast<uint32_t>(q) << (4 * i);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float q = rnd_v<T>(rnd_v<T>(x[i] - lo) / sc);
+                q = __builtin_amdgcn_fmed3f(q, 0.0f, 15.0f);   // NaN (0/0 on a constant row) comes out as the minimum, 0
+                q = __builtin_rintf(q);
+                word |= static_cast<uint32_t>(q) << (4 * i);
+            }
         }
         codes[row * 16 + n] = static_cast<int32_t>(word);
         if (n == 0) { scale[row] = f2lo<T>(sc); mn[row] = f2lo<T>(lo); }

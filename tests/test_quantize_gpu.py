@@ -144,10 +144,12 @@ def test_quantize_wrap_fp32_flag(gpu):
 def test_quantizer_math_selftest_exhaustive(gpu, dtype_code, name):
     """The cheap-estimate-with-guard path against the exact path on all 2^32 operand pairs of the dtype."""
     from polarquant_amd import _ffi
-    counters = torch.zeros(2, dtype=torch.int64, device=gpu)
+    counters = torch.zeros(3, dtype=torch.int64, device=gpu)
     rc = _ffi.lib().pq_selftest_quantizer_math(dtype_code, counters.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
-    bad, slow = counters.tolist()
-    print("%s: %d mismatching pairs, %.3f%% of pairs take the exact path" % (name, bad, 100.0 * slow / 2 ** 32), flush=True)
+    bad, slow, bad_div = counters.tolist()
+    print("%s: %d mismatching pairs, %.3f%% of pairs take the exact path, %d mismatching quotients"
+          % (name, bad, 100.0 * slow / 2 ** 32, bad_div), flush=True)
     assert bad == 0
+    assert bad_div == 0     # reciprocal + two fused multiply-adds against the fp32 division, every (dividend, scale) pair
