@@ -24,18 +24,11 @@ template <> struct IsF16<F16> { static constexpr bool value = true; };
 constexpr int kVThreads = 256;
 constexpr int kRowsPerBlock = kVThreads / 16;
 
+constexpr int kRowsPerLane = 2;   // two independent 16-byte loads in flight per lane
+
 template <typename T>
-__global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
-    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t st, int Nk, int n_tok,
-    int32_t* __restrict__ codes, uint16_t* __restrict__ scale, uint16_t* __restrict__ mn, int64_t cap, int64_t off) {
-    const int n = threadIdx.x & 15;
-    const int t = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 4);
-    const int bh = blockIdx.y;
-    const bool live = t < n_tok;                       // whole 16-lane row groups are live or not
-    const int b = bh / Nk, h = bh - b * Nk;
-    const int64_t row = static_cast<int64_t>(bh) * cap + off + t;
-    uint4 w = make_uint4(0, 0, 0, 0);
-    if (live) w = *reinterpret_cast<const uint4*>(v + b * sb + h * sh + static_cast<int64_t>(t) * st + 8 * n);
+__device__ __forceinline__ void quantize_row(uint4 w, bool live, int n, int64_t row,
+                                             int32_t* __restrict__ codes, uint16_t* __restrict__ scale, uint16_t* __restrict__ mn) {
     if constexpr (IsF16<T>::value) {
         // half precision: the eager ops ARE half-precision instructions here (v_pk_min/max_f16,
         // v_sub_f16, v_med3_f16, v_rndne_f16); the division is div_faithful
@@ -127,9 +120,30 @@ __global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
     }
 }
 
+template <typename T>
+__global__ __launch_bounds__(kVThreads) void quantize_values_kernel(
+    const uint16_t* __restrict__ v, int64_t sb, int64_t sh, int64_t st, int Nk, int n_tok,
+    int32_t* __restrict__ codes, uint16_t* __restrict__ scale, uint16_t* __restrict__ mn, int64_t cap, int64_t off) {
+    const int n = threadIdx.x & 15;
+    const int bh = blockIdx.y;
+    const int b = bh / Nk, h = bh - b * Nk;
+    const uint16_t* vb = v + b * sb + h * sh + 8 * n;
+    uint4 w[kRowsPerLane];
+    int t[kRowsPerLane];
+#pragma unroll
+    for (int u = 0; u < kRowsPerLane; u++) {
+        t[u] = (blockIdx.x * kRowsPerLane + u) * kRowsPerBlock + (threadIdx.x >> 4);
+        w[u] = make_uint4(0, 0, 0, 0);
+        if (t[u] < n_tok) w[u] = *reinterpret_cast<const uint4*>(vb + static_cast<int64_t>(t[u]) * st);   // whole 16-lane rows are live or not
+    }
+#pragma unroll
+    for (int u = 0; u < kRowsPerLane; u++)
+        quantize_row<T>(w[u], t[u] < n_tok, n, static_cast<int64_t>(bh) * cap + off + t[u], codes, scale, mn);
+}
+
 int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int B, int Nk, int T,
                            int32_t* codes, void* scale, void* mn, int64_t cap, int64_t off, hipStream_t st) {
-    dim3 grid((T + kRowsPerBlock - 1) / kRowsPerBlock, B * Nk), block(kVThreads);
+    dim3 grid((T + kRowsPerBlock * kRowsPerLane - 1) / (kRowsPerBlock * kRowsPerLane), B * Nk), block(kVThreads);
     if (dtype == 0)
         hipLaunchKernelGGL(quantize_values_kernel<F16>, grid, block, 0, st, (const uint16_t*)v, strides[0], strides[1],
                            strides[2], Nk, T, codes, (uint16_t*)scale, (uint16_t*)mn, cap, off);
