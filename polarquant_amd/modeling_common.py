@@ -108,10 +108,42 @@ def repeat_kv_quant(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
     return hidden_states[:, :, None].expand(b, h, n_rep, nb, s, d).reshape(b, h * n_rep, nb, s, d)
 
 
+def rope_parameters(config):
+    """(theta, scaling dict or None) of a PolarConfig or of a HF config of either generation:
+    transformers < 5 keeps `rope_theta` / `rope_scaling` as attributes, 5.x one `rope_parameters` dict."""
+    theta = getattr(config, "rope_theta", None)
+    scaling = getattr(config, "rope_scaling", None)
+    rp = getattr(config, "rope_parameters", None)
+    if isinstance(rp, dict):
+        theta = rp.get("rope_theta", theta)
+        scaling = rp
+    if isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type", "default")) == "default":
+        scaling = None
+    return (10000.0 if theta is None else float(theta)), scaling
+
+
 class RotaryEmbedding(nn.Module):
-    def __init__(self, head_dim: int, base: float):
+    """cos / sin tables as HF's LlamaRotaryEmbedding gives them, which is what the reference's forward receives as
+    `position_embeddings` (models/modeling_llama_polar.py:56-59).  Frequency scalings: none, "linear" and "llama3"
+    (Llama-3.1's published wavelength-dependent rescaling); any other type is refused."""
+
+    def __init__(self, head_dim: int, base: float, scaling: Optional[dict] = None):
         super().__init__()
         inv_freq = 1.0 / (base ** (torch.arange(0, head_dim, 2, dtype=torch.float32) / head_dim))
+        kind = "default" if not scaling else scaling.get("rope_type", scaling.get("type", "default"))
+        if kind == "linear":
+            inv_freq = inv_freq / float(scaling["factor"])
+        elif kind == "llama3":
+            factor, lo, hi = float(scaling["factor"]), float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
+            old_len = float(scaling["original_max_position_embeddings"])
+            wavelen = 2 * math.pi / inv_freq
+            scaled = torch.where(wavelen > old_len / lo, inv_freq / factor, inv_freq)
+            smooth = (old_len / wavelen - lo) / (hi - lo)
+            blended = (1 - smooth) * scaled / factor + smooth * scaled
+            medium = ~(wavelen < old_len / hi) & ~(wavelen > old_len / lo)
+            inv_freq = torch.where(medium, blended, scaled)
+        elif kind != "default":
+            raise NotImplementedError("polarquant_amd: rope scaling type %r is not implemented" % (kind,))
         self.register_buffer("inv_freq", inv_freq, persistent=False)
 
     @torch.no_grad()
@@ -595,7 +627,7 @@ class PolarModel(nn.Module):
         self.layers = nn.ModuleList([self.layer_class(config, i) for i in range(config.num_hidden_layers)])
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
         head_dim = _cfg(config, "head_dim", None) or config.hidden_size // config.num_attention_heads
-        self.rotary_emb = RotaryEmbedding(head_dim, _cfg(config, "rope_theta", 10000.0))
+        self.rotary_emb = RotaryEmbedding(head_dim, *rope_parameters(config))
 
     def forward(self, input_ids=None, attention_mask=None, past_key_values=None):
         bsz, q_len = input_ids.shape
