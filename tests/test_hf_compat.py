@@ -106,3 +106,30 @@ def test_shell_computes_what_hf_computes_before_any_key_is_quantized(gpu, family
             cache = out.past_key_values
             _logits_close(out.logits[:, -1], ref[:, L + s], 2e-2)
         assert cache[0][-1] == L + steps and cache[0][1] is None       # no group was quantized
+
+
+@pytest.mark.gpu
+def test_left_padded_batch_matches_hf_at_the_real_tokens(gpu):
+    """Two layers, so that whatever the padded positions produce in layer 0 meets the mask in layer 1."""
+    from polarquant_amd.modeling_llama_polar import LlamaPolarForCausalLM
+    torch.manual_seed(12)
+    cfg = _llama_config()
+    hf = transformers.LlamaForCausalLM(cfg).eval()
+    mine = LlamaPolarForCausalLM(cfg)
+    mine.load_state_dict(hf.state_dict(), strict=True)
+    mine = mine.half().to(gpu).eval()
+    B, L, steps, pad = 2, 70, 5, 9
+    ids = torch.randint(0, 1000, (B, L + steps))
+    mask = torch.ones(B, L + steps, dtype=torch.int64)
+    mask[1, :pad] = 0
+    with torch.no_grad():
+        ref = hf(ids, attention_mask=mask).logits
+        out = mine(ids[:, :L].to(gpu), mask[:, :L].to(gpu), None)
+        assert torch.isfinite(out.logits[0]).all() and torch.isfinite(out.logits[1, pad:]).all()
+        _logits_close(out.logits[0], ref[0, :L], 2e-2)
+        _logits_close(out.logits[1, pad:], ref[1, pad:L], 2e-2)
+        cache = out.past_key_values
+        for s in range(steps):
+            out = mine(ids[:, L + s:L + s + 1].to(gpu), mask[:, :L + s + 1].to(gpu), cache)
+            cache = out.past_key_values
+            _logits_close(out.logits[:, -1], ref[:, L + s], 2e-2)
