@@ -682,20 +682,22 @@ class PolarForCausalLM(nn.Module):
 # ----------------------------------------------------------------------------- generation (reference :565-666)
 def top_k_top_p_filtering(logits, top_k: int = 0, top_p: float = 1.0, filter_value: float = -float("Inf"),
                           min_tokens_to_keep: int = 1):
+    """Top-k, then nucleus filtering of [rows, vocab] logits, in place (models/modeling_llama_polar.py:565-588).
+    Nucleus rule as the reference applies it: in descending order, a token is dropped when the probability mass up
+    to and including its predecessor exceeds `top_p`, so the token that crosses the threshold survives; with
+    `min_tokens_to_keep` > 1 the predecessors' verdicts of the first `min_tokens_to_keep` places are cleared first."""
     if top_k > 0:
-        top_k = min(max(top_k, min_tokens_to_keep), logits.size(-1))
-        indices_to_remove = logits < torch.topk(logits, top_k)[0][..., -1, None]
-        logits[indices_to_remove] = filter_value
+        k = min(max(top_k, min_tokens_to_keep), logits.size(-1))
+        kth_largest = logits.topk(k, dim=-1).values[..., -1:]
+        logits.masked_fill_(logits < kth_largest, filter_value)
     if top_p < 1.0:
-        sorted_logits, sorted_indices = torch.sort(logits, descending=True)
-        cumulative_probs = torch.cumsum(F.softmax(sorted_logits, dim=-1), dim=-1)
-        sorted_indices_to_remove = cumulative_probs > top_p
+        order = logits.argsort(dim=-1, descending=True)
+        over = logits.gather(-1, order).softmax(-1).cumsum(-1) > top_p
         if min_tokens_to_keep > 1:
-            sorted_indices_to_remove[..., :min_tokens_to_keep] = 0
-        sorted_indices_to_remove[..., 1:] = sorted_indices_to_remove[..., :-1].clone()
-        sorted_indices_to_remove[..., 0] = 0
-        indices_to_remove = sorted_indices_to_remove.scatter(1, sorted_indices, sorted_indices_to_remove)
-        logits[indices_to_remove] = filter_value
+            over[..., :min_tokens_to_keep] = False
+        drop_sorted = torch.zeros_like(over)
+        drop_sorted[..., 1:] = over[..., :-1]
+        logits.masked_fill_(torch.zeros_like(over).scatter_(-1, order, drop_sorted), filter_value)
     return logits
 
 
@@ -716,30 +718,26 @@ class GenerationConfig:
 
 
 def generate(model, input_ids, attention_mask, generation_config, do_sample=False, max_new_tokens=8):
-    current_input_ids = input_ids
-    batch_size = input_ids.size(0)
-    device = model.device
-    generate_ids = torch.zeros([batch_size, max_new_tokens], dtype=torch.long, device=device)
-    eos_sequence = torch.zeros([batch_size, 1], dtype=torch.bool, device=device)
-    eos = generation_config.eos_token_id
-    stop_tensor = torch.tensor(eos if isinstance(eos, (list, tuple)) else [eos], dtype=torch.long, device=device)
-    next_decoder_cache = None
+    """The reference's decoding loop (models/modeling_llama_polar.py:622-666): prefill, then one token per step,
+    the mask grown by a column of ones; stops early once every sequence has produced a stop token (sequences that
+    stopped earlier keep producing tokens until then, as in the reference).  -> LongTensor [B, <= max_new_tokens]."""
+    dev = model.device
+    n_seq = input_ids.size(0)
+    stop_ids = generation_config.eos_token_id
+    stop_ids = torch.as_tensor(stop_ids if isinstance(stop_ids, (list, tuple)) else [stop_ids], dtype=torch.long, device=dev)
+    produced = torch.zeros((n_seq, max_new_tokens), dtype=torch.long, device=dev)
+    finished = torch.zeros((n_seq, 1), dtype=torch.bool, device=dev)
+    tokens, cache, n_out = input_ids, None, 0
     with torch.no_grad():
-        step = 0
-        while True:
-            if step >= max_new_tokens:
-                break
-            outputs = model(input_ids=current_input_ids, attention_mask=attention_mask,
-                            past_key_values=next_decoder_cache, num_logits_to_keep=1)
-            output_ids = sample(outputs.logits, generation_config, do_sample=do_sample)
-            next_decoder_cache = outputs.past_key_values
-            generate_ids[:, step:step + 1] = output_ids
-            current_input_ids = output_ids
+        while n_out < max_new_tokens:
+            step_out = model(input_ids=tokens, attention_mask=attention_mask, past_key_values=cache, num_logits_to_keep=1)
+            cache = step_out.past_key_values
+            tokens = sample(step_out.logits, generation_config, do_sample=do_sample)
+            produced[:, n_out:n_out + 1] = tokens
+            n_out += 1
             if attention_mask is not None:
-                attention_mask = torch.cat([attention_mask, torch.ones_like(output_ids)], dim=-1)
-            eos_sequence = eos_sequence | torch.isin(current_input_ids, stop_tensor)
-            if eos_sequence.sum().item() == batch_size:
+                attention_mask = torch.cat([attention_mask, torch.ones_like(tokens)], dim=-1)
+            finished |= torch.isin(tokens, stop_ids)
+            if bool(finished.all()):
                 break
-            step += 1
-    step = min(step + 1, max_new_tokens)
-    return generate_ids[:, :step]
+    return produced[:, :n_out]

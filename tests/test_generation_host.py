@@ -1,0 +1,105 @@
+"""Host logic of the decoding loop (models/modeling_llama_polar.py:565-666 in the reference): top-k / nucleus
+filtering against known answers and a plain-loop restatement, and the stopping rule of generate() against a
+scripted stand-in model.  No GPU."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from polarquant_amd.modeling_common import GenerationConfig, generate, sample, top_k_top_p_filtering
+
+
+def _kept(logits):
+    return [sorted(torch.nonzero(torch.isfinite(r)).flatten().tolist()) for r in logits]
+
+
+def test_nucleus_keeps_the_token_that_crosses_the_threshold():
+    probs = torch.tensor([[0.05, 0.5, 0.15, 0.3]])
+    assert _kept(top_k_top_p_filtering(probs.log(), top_k=0, top_p=0.7)) == [[1, 3]]        # 0.5, then 0.3 crosses 0.7
+    assert _kept(top_k_top_p_filtering(probs.log(), top_k=0, top_p=0.81)) == [[1, 2, 3]]    # 0.8 does not exceed 0.81
+    assert _kept(top_k_top_p_filtering(probs.log(), top_k=0, top_p=0.4)) == [[1]]
+    assert _kept(top_k_top_p_filtering(probs.log(), top_k=0, top_p=1.0)) == [[0, 1, 2, 3]]
+
+
+def test_top_k_keeps_ties_with_the_kth_largest_and_clamps_k():
+    logits = torch.tensor([[1.0, 3.0, 2.0, 2.0, 0.0]])
+    assert _kept(top_k_top_p_filtering(logits.clone(), top_k=2)) == [[1, 2, 3]]      # both 2.0 are "not smaller than the 2nd"
+    assert _kept(top_k_top_p_filtering(logits.clone(), top_k=1)) == [[1]]
+    assert _kept(top_k_top_p_filtering(logits.clone(), top_k=50)) == [[0, 1, 2, 3, 4]]
+    assert _kept(top_k_top_p_filtering(logits.clone(), top_k=1, min_tokens_to_keep=3)) == [[1, 2, 3]]
+
+
+def _loop_restatement(row, top_k, top_p, min_keep):
+    keep = set(range(len(row)))
+    if top_k > 0:
+        k = min(max(top_k, min_keep), len(row))
+        kth = sorted(row, reverse=True)[k - 1]
+        keep = {i for i in keep if not row[i] < kth}
+    if top_p < 1.0:
+        vals = [row[i] if i in keep else -math.inf for i in range(len(row))]
+        order = sorted(range(len(row)), key=lambda i: -vals[i])
+        m = max(vals)
+        z = sum(math.exp(v - m) for v in vals)
+        cum, over = 0.0, []
+        for i in order:
+            cum += math.exp(vals[i] - m) / z
+            over.append(cum > top_p)
+        if min_keep > 1:
+            for j in range(min_keep):
+                over[j] = False
+        for pos, i in enumerate(order):
+            if pos > 0 and over[pos - 1]:
+                keep.discard(i)
+    return sorted(keep)
+
+
+@pytest.mark.parametrize("top_k,top_p,min_keep", [(0, 0.9, 1), (5, 0.5, 1), (3, 1.0, 1), (8, 0.3, 4), (0, 0.05, 2)])
+def test_filtering_against_a_plain_loop(top_k, top_p, min_keep):
+    g = torch.Generator().manual_seed(top_k * 100 + int(top_p * 10))
+    logits = torch.randn(6, 17, generator=g, dtype=torch.float64) * 2
+    want = [_loop_restatement(r.tolist(), top_k, top_p, min_keep) for r in logits]
+    got = top_k_top_p_filtering(logits.clone(), top_k=top_k, top_p=top_p, min_tokens_to_keep=min_keep)
+    assert _kept(got) == want
+    assert torch.equal(got[torch.isfinite(got)], logits[torch.isfinite(got)])       # survivors keep their values
+
+
+def test_sample_greedy_and_filtered():
+    logits = torch.tensor([[[0.0, 5.0, 1.0]], [[2.0, 0.0, -1.0]]])
+    assert sample(logits, GenerationConfig(), do_sample=False).tolist() == [[1], [0]]
+    torch.manual_seed(0)
+    cfg = GenerationConfig(top_k=1)
+    for _ in range(5):      # top_k = 1 leaves one candidate: sampling is then greedy
+        assert sample(logits.clone(), cfg, do_sample=True).tolist() == [[1], [0]]
+
+
+class _Scripted:
+    """Stand-in model: sequence b produces script[b][step]; records what generate() passes in."""
+    device = torch.device("cpu")
+
+    def __init__(self, script, vocab=10):
+        self.script, self.vocab, self.calls = script, vocab, []
+
+    def __call__(self, input_ids, attention_mask, past_key_values, num_logits_to_keep):
+        step = 0 if past_key_values is None else past_key_values
+        self.calls.append((tuple(input_ids.shape), None if attention_mask is None else tuple(attention_mask.shape), num_logits_to_keep))
+        logits = torch.zeros(len(self.script), 1, self.vocab)
+        for b, row in enumerate(self.script):
+            logits[b, 0, row[step]] = 1.0
+        return SimpleNamespace(logits=logits, past_key_values=step + 1)
+
+
+def test_generate_stops_when_every_sequence_has_stopped_and_keeps_the_stop_token():
+    model = _Scripted([[3, 9, 4, 4, 4, 4], [5, 6, 7, 9, 1, 1]])
+    out = generate(model, torch.zeros(2, 4, dtype=torch.long), torch.ones(2, 4, dtype=torch.long),
+                   GenerationConfig(eos_token_id=[9]), max_new_tokens=6)
+    # sequence 0 stops at step 1 and keeps producing; sequence 1 stops at step 3: four columns come back
+    assert out.tolist() == [[3, 9, 4, 4], [5, 6, 7, 9]]
+    assert model.calls[0] == ((2, 4), (2, 4), 1) and model.calls[1] == ((2, 1), (2, 5), 1) and model.calls[3][1] == (2, 7)
+
+
+def test_generate_runs_to_the_limit_without_a_stop_token_and_accepts_a_scalar_eos():
+    model = _Scripted([[1, 2, 3, 4]])
+    out = generate(model, torch.zeros(1, 2, dtype=torch.long), None, GenerationConfig(eos_token_id=7), max_new_tokens=3)
+    assert out.tolist() == [[1, 2, 3]] and len(model.calls) == 3 and model.calls[2][1] is None
+    assert generate(model, torch.zeros(1, 2, dtype=torch.long), None, GenerationConfig(), max_new_tokens=0).shape == (1, 0)
