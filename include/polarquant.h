@@ -66,6 +66,20 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * sub-byte store it announces there.  Code tensors are then [B,Nk,capacity,128,48]. */
 #define PQ_CODES_PACKED6 4u
 
+/* Linear layer of a decode step: y[M, N] = x[M, K] . w[N, K]^T (+ bias[N]), M <= 16 rows (one new
+ * token per sequence), fp32 accumulation, one rounding to the dtype.  Replaces the q/k/v, o and MLP
+ * projections (`nn.Linear`) the decode step calls around the attention
+ * (models/modeling_llama_polar.py:47-52, :131, and the decoder layer's MLP, :456-486): at this M they
+ * are streams of the weight matrix through HBM, which the kernel is laid out for.
+ *   x [M, K] rows `x_row_stride` elements apart, w [N, K] dense row-major (the nn.Linear weight),
+ *   y [M, N] rows `y_row_stride` apart; N % 16 == 0, K % 32 == 0, x and w 16-byte aligned.
+ *   w_up != NULL: the gated MLP input in one call, y = silu(x.w^T) * (x.w_up^T) with the eager
+ *   modules' roundings (both products and silu rounded to the dtype first); no bias then. */
+int pq_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const void *w_up, const void *bias,
+                      void *y, int64_t y_row_stride, int M, int N, int K, int dtype, void *stream);
+int pq_validate_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const void *w_up, const void *bias,
+                               const void *y, int64_t y_row_stride, int M, int N, int K, int dtype);
+
 /* Layout converter for code rows: pack != 0 turns `n_rows` byte-per-code rows (64 bytes each, every
  * code < 64) into packed 6-bit rows (48 bytes each), pack == 0 the reverse.  For caches built by the
  * reference (always byte-per-code) that are to be kept packed, and back.  No reference counterpart. */

@@ -302,6 +302,28 @@ int pq_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, int pack,
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
+int pq_validate_linear_small_m(const void* x, int64_t x_row_stride, const void* w, const void* w_up, const void* bias,
+                               const void* y, int64_t y_row_stride, int M, int N, int K, int dtype) {
+    if (!x || !w || !y) return PQ_ERR_NULL_POINTER;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (M < 1 || M > 16 || N < 16 || (N % 16) != 0 || K < 32 || (K % 32) != 0) return PQ_ERR_BAD_SHAPE;
+    if (static_cast<long long>(N) * K > (1LL << 40)) return PQ_ERR_BAD_SHAPE;
+    if (x_row_stride < K || (x_row_stride % 8) != 0 || y_row_stride < N || (y_row_stride % 4) != 0) return PQ_ERR_BAD_STRIDE;
+    if (w_up && bias) return PQ_ERR_BAD_SHAPE;       // the gated form has no bias
+    if (!aligned(x, 16) || !aligned(w, 16) || (w_up && !aligned(w_up, 16)) || !aligned(y, 8) || (bias && !aligned(bias, 2)))
+        return PQ_ERR_MISALIGNED;
+    return PQ_OK;
+}
+
+int pq_linear_small_m(const void* x, int64_t x_row_stride, const void* w, const void* w_up, const void* bias,
+                      void* y, int64_t y_row_stride, int M, int N, int K, int dtype, void* stream) {
+    const int rc = pq_validate_linear_small_m(x, x_row_stride, w, w_up, bias, y, y_row_stride, M, N, K, dtype);
+    if (rc != PQ_OK) return rc;
+    const int err = pq::launch_small_m_linear(x, x_row_stride, w, w_up, bias, y, y_row_stride, M, N, K, dtype,
+                                              static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;

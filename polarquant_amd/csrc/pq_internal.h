@@ -29,6 +29,9 @@ int launch_silu_mul(const void* gate, const void* up, void* y, int rows, int col
 
 int launch_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, bool pack, hipStream_t st);
 
+int launch_small_m_linear(const void* x, int64_t x_stride, const void* w, const void* w_up, const void* bias, void* y,
+                          int64_t y_stride, int M, int N, int K, int dtype, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;

@@ -80,3 +80,28 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
                                     _stream_ptr(gate.device))
     _ffi.check(rc, "pq_silu_mul")
     return y
+
+
+def linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                   up_weight: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`F.linear(x, weight, bias)` for at most 16 rows (x [..., K] with up to 16 leading elements, unit
+    element stride, one row stride), streamed through the weight-streaming kernel.  With `up_weight`:
+    the gated MLP input `silu(x @ weight.T) * (x @ up_weight.T)` in one launch (no bias)."""
+    _gpu(x)
+    K = x.shape[-1]
+    N = weight.shape[0]
+    x2 = x.reshape(-1, K)
+    M = x2.shape[0]
+    assert weight.is_contiguous() and weight.shape == (N, K) and weight.dtype == x.dtype and x2.stride(1) == 1
+    if up_weight is not None:
+        assert up_weight.is_contiguous() and up_weight.shape == weight.shape and up_weight.dtype == x.dtype
+    if bias is not None:
+        assert bias.is_contiguous() and bias.numel() == N and bias.dtype == x.dtype
+    y = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _ffi.lib().pq_linear_small_m(x2.data_ptr(), x2.stride(0) if M > 1 else K, weight.data_ptr(),
+                                          None if up_weight is None else up_weight.data_ptr(),
+                                          None if bias is None else bias.data_ptr(), y.data_ptr(), N, M, N, K,
+                                          _dtype_code(x), _stream_ptr(x.device))
+    _ffi.check(rc, "pq_linear_small_m")
+    return y

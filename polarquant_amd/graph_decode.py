@@ -28,11 +28,15 @@ from .modeling_common import GROUP, apply_rotary_pos_emb
 
 
 class PolarGraphDecoder:
-    def __init__(self, model, max_len: int, use_graph: bool = True, fused_ops: bool = True):
+    def __init__(self, model, max_len: int, use_graph: bool = True, fused_ops: bool = True, small_m_gemm: bool = True):
         """fused_ops: run RoPE + cache append, the norms and the MLP activation as one HIP launch each
         (polarquant_amd.decode_ops) instead of the eager modules' chains of elementwise launches.  The
-        rotation is bit-identical to the eager ops; the norms and SiLU agree to the dtype's last bit."""
+        rotation is bit-identical to the eager ops; the norms and SiLU agree to the dtype's last bit.
+        small_m_gemm (with fused_ops, batch <= 16): o_proj, gate/up (with the SiLU product in its epilogue) and
+        down_proj through the weight-streaming kernel `decode_ops.linear_small_m` instead of the BLAS library;
+        fp32 accumulation in a different order, so logits agree to rounding."""
         self.fused_ops = fused_ops
+        self.small_m_gemm = small_m_gemm
         self.model = model
         self.cfg = model.config
         self.max_len = int(max_len)
@@ -121,7 +125,7 @@ class PolarGraphDecoder:
     def _step_body_fused(self):
         """The decode step with one launch per elementwise stage: 2 norms (each with the residual add
         folded in), RoPE + append, SiLU * up, plus the GEMMs and the attention, per layer."""
-        from .decode_ops import rmsnorm, rope_append, silu_mul
+        from .decode_ops import linear_small_m, rmsnorm, rope_append, silu_mul
         model, B = self.model, self.B
         layers = model.model.layers
         x = model.model.embed_tokens(self.ids).contiguous()                 # residual stream [B,1,H], updated in place
@@ -135,11 +139,21 @@ class PolarGraphDecoder:
             q = rope_append(q_lin, k_lin, v_lin, self.cos_table, self.sin_table, self.pos, ar.kres, self.resid_idx,
                             v_dst, v_row, att.num_heads, att.num_key_value_heads)
             o = self._attend(att, ar, q)
-            a = att.o_proj(o.reshape(B, 1, -1))
+            own = self.small_m_gemm and B <= 16 and all(
+                lin.weight.is_contiguous() and lin.weight.shape[0] % 16 == 0 and lin.weight.shape[1] % 32 == 0
+                for lin in (att.o_proj, mlp.gate_proj, mlp.up_proj, mlp.down_proj))
             pn = layer.post_attention_layernorm
-            h = rmsnorm(x, pn.weight, pn.variance_epsilon, residual=a, sum_out=x)
-            # (gate | up as one GEMM was measured too: no faster than the two, so they stay separate)
-            m = mlp.down_proj(silu_mul(mlp.gate_proj(h), mlp.up_proj(h)))
+            if own and mlp.gate_proj.bias is None and mlp.up_proj.bias is None:
+                # (the fused q|k|v projection stays with the library: equal time at that shape)
+                a = linear_small_m(o.reshape(B, 1, -1), att.o_proj.weight, att.o_proj.bias)
+                h = rmsnorm(x, pn.weight, pn.variance_epsilon, residual=a, sum_out=x)
+                act = linear_small_m(h, mlp.gate_proj.weight, up_weight=mlp.up_proj.weight)
+                m = linear_small_m(act, mlp.down_proj.weight, mlp.down_proj.bias)
+            else:
+                a = att.o_proj(o.reshape(B, 1, -1))
+                h = rmsnorm(x, pn.weight, pn.variance_epsilon, residual=a, sum_out=x)
+                # (gate | up as one library GEMM was measured too: no faster than the two, so they stay separate)
+                m = mlp.down_proj(silu_mul(mlp.gate_proj(h), mlp.up_proj(h)))
             nn_ = layers[li + 1].input_layernorm if li + 1 < len(layers) else model.model.norm
             h = rmsnorm(x, nn_.weight, nn_.variance_epsilon, residual=m, sum_out=x)
         logits = model.lm_head(h)

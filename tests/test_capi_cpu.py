@@ -196,6 +196,25 @@ def test_fused_decode_ops_reject_bad_arguments(lib):
     assert lib.pq_silu_mul(P, P, P, 2, 64, 32, 0, None) == -6                      # rows would overlap
 
 
+def test_linear_small_m_rejects_bad_arguments(lib):
+    ok = [P, 4096, P, None, None, P, 4096, 8, 4096, 4096, 1]
+    assert lib.pq_validate_linear_small_m(*ok) == 0
+    def bad(i, v):
+        a = list(ok)
+        a[i] = v
+        return lib.pq_validate_linear_small_m(*a)
+    assert bad(0, None) == -1 and bad(2, None) == -1 and bad(5, None) == -1
+    assert bad(10, 2) == -4                                             # dtype
+    assert bad(7, 0) == -2 and bad(7, 17) == -2                         # rows
+    assert bad(8, 4100) == -2 and bad(9, 4100) == -2 and bad(9, 16) == -2   # N % 16, K % 32
+    assert bad(1, 4000) == -6 and bad(1, 4100) == -6 and bad(6, 4000) == -6 and bad(6, 4098) == -6   # strides
+    assert bad(0, P + 8) == -5 and bad(2, P + 2) == -5 and bad(5, P + 4) == -5 and bad(3, P + 8) == -5
+    gated_with_bias = list(ok)
+    gated_with_bias[3], gated_with_bias[4] = P, P
+    assert lib.pq_validate_linear_small_m(*gated_with_bias) == -2
+    assert lib.pq_linear_small_m(None, 4096, P, None, None, P, 4096, 8, 4096, 4096, 1, None) == -1
+
+
 def test_convert_codes6_rejects_bad_arguments(lib):
     assert lib.pq_convert_codes6(None, P, 4, 1, None) == -1 and lib.pq_convert_codes6(P, None, 4, 0, None) == -1
     assert lib.pq_convert_codes6(P, P, 0, 1, None) == -2
