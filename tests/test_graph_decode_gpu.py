@@ -47,9 +47,10 @@ def test_graph_decoder_matches_eager_model(gpu, cls, cfg, dtype):
     dec_g = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=True)
     dec_e = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=False)
     dec_u = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=False, fused_ops=False)
+    dec_l = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=False, small_m_gemm=False)   # library GEMMs
     with torch.no_grad():
         ref = model(input_ids=ids, attention_mask=None, past_key_values=None, num_logits_to_keep=1)
-        for d in (dec_g, dec_e, dec_u):
+        for d in (dec_g, dec_e, dec_u, dec_l):
             assert torch.equal(d.prefill(ids), ref.logits)
         cache = ref.past_key_values
         tok = ref.logits.argmax(-1)
@@ -58,11 +59,12 @@ def test_graph_decoder_matches_eager_model(gpu, cls, cfg, dtype):
             cache = ref.past_key_values
             got_u = dec_u.step(tok).clone()
             got_e = dec_e.step(tok).clone()
+            got_l = dec_l.step(tok).clone()
             got_g = dec_g.step(tok).clone()
             torch.cuda.synchronize()
             assert torch.equal(got_g, got_e), "graph replay %d differs from the eager step" % s
             rl = ref.logits.float()
-            for got in (got_u, got_e):
+            for got in (got_u, got_e, got_l):
                 err = (got.float() - rl).abs().max().item()
                 assert err <= 2e-2 * max(1.0, rl.abs().max().item()), (s, err)
                 # the token the static step would pick is (nearly) the model's best
