@@ -147,8 +147,10 @@ int pq_validate_quantize_groups(const void *k, const int64_t *k_strides, int dty
  * The kernel takes a cheap arctangent / square root first and the exact,
  * eager-torch-identical routines only near a rounding boundary; this runs both on
  * ALL 2^32 (y, x) operand pairs of the dtype (NaNs skipped) and adds to
- * counters[0] the number of pairs whose rounded angle or radius differ (must stay
- * 0) and to counters[1] the number of pairs that needed the exact routine.
+ * counters[0] the number of pairs whose rounded angle or radius differ, plus the
+ * pairs whose exact radius is not the correctly rounded square root (checked in
+ * double precision against the midpoints to its two neighbours); must stay 0.
+ * counters[1] receives the number of pairs that needed the exact routine.
  * Both quantizers also replace the fp32 division by a scale with a reciprocal and
  * two fused multiply-adds; counters[2] receives the number of (dividend, scale)
  * pairs of the dtype, over the whole range the quantizers can meet, whose

@@ -90,13 +90,19 @@ __device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out
             static_cast<int>(near_rounding_boundary<T>(r, kSqrtGuardUlps))) != 0;
 }
 
+// Correctly rounded fp32 square root.  NOT __fsqrt_rn: HIP defines that as the native (1 ulp)
+// instruction unless OCML_BASIC_ROUNDED_OPERATIONS is set; sqrtf() is expanded by the compiler to
+// the correctly rounded sequence (the default of -fhip-fp32-correctly-rounded-divide-sqrt), and the
+// device self-test checks every result against its two neighbours' midpoints in double precision.
+__device__ __forceinline__ float sqrt_rn(float s) { return __builtin_sqrtf(s); }
+
 // -> (angle in [-pi, pi], radius), both rounded to the key dtype
 template <typename T>
 __device__ __forceinline__ void angle_radius(float x, float y, float* phi, float* rad) {
     float a, r;
     if (__builtin_expect(angle_radius_fast<T>(x, y, &a, &r), 0)) {
         a = math::atan2f_sleef_u10(y, x);
-        r = __fsqrt_rn(__builtin_fmaf(x, x, y * y));
+        r = sqrt_rn(__builtin_fmaf(x, x, y * y));
     }
     *phi = rnd<T>(a);
     *rad = rnd<T>(r);
@@ -105,7 +111,7 @@ __device__ __forceinline__ void angle_radius(float x, float y, float* phi, float
 template <typename T>
 __device__ __forceinline__ void angle_radius_exact(float x, float y, float* phi, float* rad) {
     *phi = rnd<T>(math::atan2f_sleef_u10(y, x));
-    *rad = rnd<T>(__fsqrt_rn(__builtin_fmaf(x, x, y * y)));
+    *rad = rnd<T>(sqrt_rn(__builtin_fmaf(x, x, y * y)));
 }
 
 // floor(dtype((v - mn) / scale)) clamped to [0, top] (:148, :153).  `topf` is the clamp bound as a
@@ -360,6 +366,14 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* misma
         angle_radius<T>(x, y, &p0, &r0);
         angle_radius_exact<T>(x, y, &p1, &r1);
         bad += (f2lo<T>(p0) != f2lo<T>(p1)) || (f2lo<T>(r0) != f2lo<T>(r1));
+        // the exact radius: s lies between the squares of the midpoints to the two neighbours of sqrt_rn(s)
+        const float s = __builtin_fmaf(x, x, y * y);
+        if (s > 0.0f && s < INFINITY) {
+            const float rr = sqrt_rn(s);
+            const double lo = 0.5 * (static_cast<double>(rr) + static_cast<double>(__uint_as_float(__float_as_uint(rr) - 1u)));
+            const double hi = 0.5 * (static_cast<double>(rr) + static_cast<double>(__uint_as_float(__float_as_uint(rr) + 1u)));
+            bad += !(lo * lo <= static_cast<double>(s) && static_cast<double>(s) <= hi * hi);
+        }
         const float a = atan2_fast(y, x), r = __builtin_amdgcn_sqrtf(__builtin_fmaf(x, x, y * y));
         slow += near_rounding_boundary<T>(a, kAtanGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
     }

@@ -153,3 +153,18 @@ def test_quantizer_math_selftest_exhaustive(gpu, dtype_code, name):
           % (name, bad, 100.0 * slow / 2 ** 32, bad_div), flush=True)
     assert bad == 0
     assert bad_div == 0     # reciprocal + two fused multiply-adds against the fp32 division, every (dividend, scale) pair
+
+
+def test_radius_on_a_double_rounding_tie(gpu):
+    """x = 0xa2cd, y = 0x15b1 (half words): the correctly rounded fp32 square root of x^2 + y^2 lies one ulp above
+    a midpoint between two half values, a 1-ulp-low square root lies exactly on it and rounds (to even) the other
+    way.  Eager torch gives the upper neighbour; the kernel's exact path must use a correctly rounded root."""
+    bits = torch.tensor([0xa2cd - 65536, 0x15b1], dtype=torch.int16).view(torch.float16)
+    g = torch.Generator().manual_seed(77)
+    k = (torch.randn(1, 1, 128, 128, generator=g) * 0.5 + 2.0).half()       # every other radius is far larger
+    k[0, 0, 5, 0], k[0, 0, 5, 64] = bits[0], bits[1]
+    ref = po.quantize_and_pack_nbit(k, 4, 4)
+    assert ref[2][0, 0, 0, 0, 0].item() == 0.01335906982421875              # the minimum radius of pair 0
+    got = quantize_and_pack_nbit(k.to(gpu), 4, 4)
+    flips = count_flips(got, ref)
+    assert all(v == 0 for v in flips.values()), flips
