@@ -318,7 +318,9 @@ class PolarGroupAttention(nn.Module):
         if self.capture is not None:
             self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
 
-        if q_len == 1:   # decoding time (:61-101)
+        # decoding time (:61-101).  A one-token prompt (no cache yet) is a prefill here; the reference takes its
+        # decode branch on q_len alone and fails unpacking the missing cache.
+        if q_len == 1 and past_key_value is not None:
             arena = self._arena_of(past_key_value, query_states.dtype, query_states.device)
             arena.reserve(arena.kv_len + 1)
             arena.kres[:, :, arena.n_resid] = key_states[:, :, 0]          # :77
@@ -454,7 +456,7 @@ class PolarMixedGroupAttention(PolarGroupAttention):
         if self.capture is not None:
             self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
 
-        if q_len == 1:   # decoding time (:185-257)
+        if q_len == 1 and past_key_value is not None:   # decoding time (:185-257); a one-token prompt is a prefill
             arena = self._arena_of(past_key_value, query_states.dtype, query_states.device)
             arena.reserve(arena.kv_len + 1)
             arena.kres[:, :, arena.n_resid] = key_states[:, :, 0]          # :201

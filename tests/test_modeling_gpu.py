@@ -28,7 +28,7 @@ def _rope(cfg, start, n, dtype, dev):
 
 
 @pytest.mark.parametrize("cls,n_heads,n_kv,rb,tb", [(LlamaPolarGroupAttention, 4, 2, 4, 4), (Qwen2PolarGroupAttention, 7, 1, 3, 3)])
-@pytest.mark.parametrize("L", [5, 200, 256])
+@pytest.mark.parametrize("L", [1, 5, 200, 256])      # 1: a one-token prompt is a prefill here (the reference fails on it)
 def test_attention_forward_matches_reference_restatement(gpu, cls, n_heads, n_kv, rb, tb, L):
     """Prefill then decode across a residual flush.  The post-RoPE q/k/v of every call are captured
     on the GPU and replayed through the oracle's forward: cache contents must be bit-identical
@@ -172,7 +172,7 @@ def test_decode_with_bf16_model(gpu):
     assert cache[1].dtype == torch.uint8 and cache[2].dtype == torch.bfloat16
 
 
-@pytest.mark.parametrize("L", [5, 200, 256])
+@pytest.mark.parametrize("L", [1, 5, 200, 256])
 def test_mixed_attention_forward_matches_reference_restatement(gpu, L):
     """LlamaPolarMixedGroupAttention (polar keys + 4-bit values): prefill, then decode across a
     flush of the shared residual window.  Captured post-RoPE q/k/v are replayed through the oracle's
