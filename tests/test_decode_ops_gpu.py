@@ -53,7 +53,7 @@ def test_rope_append_is_bit_identical_to_the_eager_ops(gpu, dtype, N, Nk):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("hidden", [512, 4096, 3584])
+@pytest.mark.parametrize("hidden", [512, 4096, 3584, 16384])
 def test_rmsnorm_matches_module(gpu, dtype, hidden):
     torch.manual_seed(hidden)
     mod = RMSNorm(hidden, 1e-5).to(dtype).to(gpu)
