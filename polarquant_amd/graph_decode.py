@@ -48,7 +48,9 @@ class PolarGraphDecoder:
 
     # ------------------------------------------------------------------ prompt
     @torch.no_grad()
-    def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
+    def prefill(self, input_ids: torch.Tensor, attention_mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """attention_mask [B, L] of {0, 1}: left padding of the prompt, as the reference's loop takes it
+        (models/modeling_llama_polar.py:622-656); the new tokens are always attended to."""
         model, cfg = self.model, self.cfg
         dev = input_ids.device
         B, L = input_ids.shape
@@ -56,7 +58,7 @@ class PolarGraphDecoder:
         old = getattr(cfg, "cache_capacity", 0)
         cfg.cache_capacity = self.max_len          # arenas never grow: their addresses are baked into the graph
         try:
-            out = model(input_ids=input_ids, attention_mask=None, past_key_values=None, num_logits_to_keep=1)
+            out = model(input_ids=input_ids, attention_mask=attention_mask, past_key_values=None, num_logits_to_keep=1)
         finally:
             cfg.cache_capacity = old
         self.arenas = [c.arena for c in out.past_key_values]
@@ -70,6 +72,12 @@ class PolarGraphDecoder:
         self.n_groups_dev = torch.full((B,), a0.n_groups, dtype=torch.int32, device=dev)
         self.n_resid_dev = torch.full((B,), self.n_resid + 1, dtype=torch.int32, device=dev)  # count INCLUDING the new key
         self.ids = torch.zeros((B, 1), dtype=torch.long, device=dev)
+        # static mask over the whole capacity: the prompt's padding, ones for every later position (the
+        # kernels read only the columns of tokens that exist, so nothing has to be updated per step)
+        self.mask8 = None
+        if attention_mask is not None:
+            self.mask8 = torch.ones((B, self.max_len), dtype=torch.uint8, device=dev)
+            self.mask8[:, :L] = (attention_mask != 0).to(torch.uint8)
         inv_freq = model.model.rotary_emb.inv_freq.float().to(dev)       # same table the eager step multiplies by
         ang = torch.arange(self.max_len, dtype=torch.float32, device=dev)[:, None] * inv_freq[None, :]
         emb = torch.cat([ang, ang], dim=-1)
@@ -117,7 +125,8 @@ class PolarGraphDecoder:
     # ------------------------------------------------------------------ one token
     def _attend(self, att, ar, q):
         common = dict(rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
-                      n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits)
+                      n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits,
+                      attention_mask=self.mask8)
         if self.mixed:
             return polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0, **common)
         return polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, **common)
@@ -184,12 +193,12 @@ class PolarGraphDecoder:
                 o = polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0,
                                               rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
                                               n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev,
-                                              n_splits=self.n_splits)
+                                              n_splits=self.n_splits, attention_mask=self.mask8)
             else:
                 ar.v.index_copy_(2, self.pos, v)
                 o = polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, rbits=att.rbits, tbits=att.tbits,
                                            sm_scale=1.0 / math.sqrt(att.head_dim), n_groups_per_seq=self.n_groups_dev,
-                                           n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits)
+                                           n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits, attention_mask=self.mask8)
             x = x + att.o_proj(o.reshape(B, 1, -1))
             x = x + layer.mlp(layer.post_attention_layernorm(x))
         logits = model.lm_head(model.model.norm(x))

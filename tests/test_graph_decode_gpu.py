@@ -79,6 +79,42 @@ def test_graph_decoder_matches_eager_model(gpu, cls, cfg, dtype):
         assert dec_g.graph is not None and dec_e.graph is None
 
 
+@pytest.mark.parametrize("mixed", [False, True])
+def test_graph_decoder_with_left_padded_prompt(gpu, mixed):
+    """The prompt's padding mask is carried as a static mask over the whole capacity: graph replay, eager
+    static step and the drop-in model (which grows its mask by one column per token) agree across a flush."""
+    torch.manual_seed(21)
+    cfg = _tiny(8, 2, vbits=4) if mixed else _tiny()
+    model = LlamaPolarForCausalLM(cfg).half().to(gpu).eval()
+    B, L, new = 3, 120, 20                        # flush at 128 tokens
+    ids = torch.randint(0, cfg.vocab_size, (B, L), device=gpu)
+    mask = torch.ones(B, L, dtype=torch.int64, device=gpu)
+    mask[1, :7] = 0
+    mask[2, :50] = 0
+    dec_g = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=True)
+    dec_e = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=False)
+    with torch.no_grad():
+        ref = model(input_ids=ids, attention_mask=mask, past_key_values=None, num_logits_to_keep=1)
+        for d in (dec_g, dec_e):
+            assert torch.equal(d.prefill(ids, mask), ref.logits)
+        cache, tok = ref.past_key_values, ref.logits.argmax(-1)
+        for s in range(new):
+            mask = torch.cat([mask, torch.ones_like(tok)], dim=-1)
+            ref = model(input_ids=tok, attention_mask=mask, past_key_values=cache, num_logits_to_keep=1)
+            cache = ref.past_key_values
+            got_e, got_g = dec_e.step(tok).clone(), dec_g.step(tok).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(got_g, got_e), s
+            rl = ref.logits.float()
+            err = (got_g.float() - rl).abs().max().item()
+            assert err <= 2e-2 * max(1.0, rl.abs().max().item()), (s, err)
+            tok = ref.logits.argmax(-1)
+        # the mask matters: without it the padded sequences' logits move
+        dec_n = PolarGraphDecoder(model, max_len=L + new + 8, use_graph=False)
+        dec_n.prefill(ids, None)
+        assert not torch.allclose(dec_n.step(tok)[2].float(), dec_e.step(tok)[2].float(), atol=1e-3)
+
+
 def test_graph_decoder_rejects_overflow(gpu):
     torch.manual_seed(12)
     cfg = _tiny(layers=1)
