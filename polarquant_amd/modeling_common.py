@@ -671,6 +671,17 @@ class PolarForCausalLM(nn.Module):
         logits = self.lm_head(hidden_states[:, -num_logits_to_keep:, :])
         return CausalLMOutputWithPast(logits=logits, past_key_values=past_key_values)
 
+    def prepare_inputs_for_generation(self, input_ids, past_key_values=None, attention_mask=None, **kwargs):
+        """The hook HF's `generate` calls (models/modeling_llama_polar.py:549-560): batch 1 only, the last token
+        once a cache exists."""
+        if input_ids.size(0) != 1:
+            raise NotImplementedError
+        return {"input_ids": input_ids[:, -1:] if past_key_values is not None else input_ids,
+                "attention_mask": attention_mask, "past_key_values": past_key_values}
+
+    def _prepare_cache_for_generation(self, *args, **kwargs):
+        return None                      # the cache is this model's own tuple, never an HF cache object (:562-563)
+
     def kv_cache_bytes_per_token(self) -> int:
         """Bytes one cached token costs across all layers: 1 code byte per pair, 4 metadata
         halves per (group, pair) amortised over 128 tokens, fp16 V (or 4-bit V with config.vbits == 4)."""

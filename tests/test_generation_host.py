@@ -103,3 +103,16 @@ def test_generate_runs_to_the_limit_without_a_stop_token_and_accepts_a_scalar_eo
     out = generate(model, torch.zeros(1, 2, dtype=torch.long), None, GenerationConfig(eos_token_id=7), max_new_tokens=3)
     assert out.tolist() == [[1, 2, 3]] and len(model.calls) == 3 and model.calls[2][1] is None
     assert generate(model, torch.zeros(1, 2, dtype=torch.long), None, GenerationConfig(), max_new_tokens=0).shape == (1, 0)
+
+
+def test_hf_generation_hook_is_batch_one_and_feeds_the_last_token():
+    from polarquant_amd.modeling_common import PolarForCausalLM
+    hook = PolarForCausalLM.prepare_inputs_for_generation
+    ids = torch.arange(6).view(1, 6)
+    first = hook(None, ids, None, torch.ones(1, 6))
+    assert first["input_ids"] is ids and first["past_key_values"] is None
+    later = hook(None, ids, past_key_values=("cache",), attention_mask=None)
+    assert later["input_ids"].tolist() == [[5]] and later["past_key_values"] == ("cache",)
+    with pytest.raises(NotImplementedError):
+        hook(None, torch.zeros(2, 3, dtype=torch.long))
+    assert PolarForCausalLM._prepare_cache_for_generation(None, 1, 2, 3) is None
