@@ -606,17 +606,14 @@ class PolarDecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
     def forward(self, hidden_states, attention_mask=None, past_key_value=None, position_embeddings=None, **kwargs):
-        residual = hidden_states
-        hidden_states = self.input_layernorm(hidden_states)
-        hidden_states, present_key_value = self.self_attn(
-            hidden_states=hidden_states, attention_mask=attention_mask, past_key_value=past_key_value,
-            position_embeddings=position_embeddings, **kwargs)
-        hidden_states = residual + hidden_states
-        residual = hidden_states
-        hidden_states = self.post_attention_layernorm(hidden_states)
-        hidden_states = self.mlp(hidden_states)
-        hidden_states = residual + hidden_states
-        return (hidden_states, present_key_value)
+        """-> (hidden_states, present_key_value): pre-norm attention and MLP blocks, each added to its input
+        (models/modeling_llama_polar.py:456-486)."""
+        x = hidden_states
+        attn_out, present = self.self_attn(hidden_states=self.input_layernorm(x), attention_mask=attention_mask,
+                                           past_key_value=past_key_value, position_embeddings=position_embeddings, **kwargs)
+        x = x + attn_out
+        x = x + self.mlp(self.post_attention_layernorm(x))
+        return x, present
 
 
 class PolarModel(nn.Module):
@@ -632,21 +629,19 @@ class PolarModel(nn.Module):
         self.rotary_emb = RotaryEmbedding(head_dim, *rope_parameters(config))
 
     def forward(self, input_ids=None, attention_mask=None, past_key_values=None):
-        bsz, q_len = input_ids.shape
-        next_decoder_cache = ()
-        inputs_embeds = self.embed_tokens(input_ids)
-        past_seen_tokens = 0 if past_key_values is None else past_key_values[0][-1]          # reference :501
-        cache_position = torch.arange(past_seen_tokens, past_seen_tokens + q_len, device=inputs_embeds.device)
-        hidden_states = inputs_embeds
-        position_embeddings = self.rotary_emb(hidden_states, cache_position.unsqueeze(0))
-        for layer_idx, decoder_layer in enumerate(self.layers):
-            hidden_states, past_key_value = decoder_layer(
-                hidden_states, attention_mask=attention_mask,
-                past_key_value=past_key_values[layer_idx] if past_key_values is not None else None,
-                position_embeddings=position_embeddings)
-            next_decoder_cache += (past_key_value,)
-        hidden_states = self.norm(hidden_states)
-        return hidden_states, next_decoder_cache
+        """-> (normed hidden states, tuple of per-layer cache tuples).  Positions continue from the last slot of
+        the first layer's cache tuple, the count of tokens seen so far (models/modeling_llama_polar.py:494-521);
+        the 2-D padding mask is handed to the layers as it is."""
+        n_seen = 0 if past_key_values is None else past_key_values[0][-1]
+        x = self.embed_tokens(input_ids)
+        positions = torch.arange(n_seen, n_seen + input_ids.shape[1], device=x.device).unsqueeze(0)
+        rope = self.rotary_emb(x, positions)
+        presents = []
+        for i, layer in enumerate(self.layers):
+            x, present = layer(x, attention_mask=attention_mask, position_embeddings=rope,
+                               past_key_value=None if past_key_values is None else past_key_values[i])
+            presents.append(present)
+        return self.norm(x), tuple(presents)
 
 
 class PolarForCausalLM(nn.Module):
