@@ -138,3 +138,37 @@ def test_random_quantizer_case(gpu, seed):
     for name, a, b in zip(["scale", "mn"], vgot[1:], vref[1:]):
         a, b = a.cpu().float(), b.float()
         assert bool(((a == b) | (a.isnan() & b.isnan())).all()), name
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))
+def test_random_scores_case(gpu, seed):
+    """The score op on random heads / bit widths / group counts, with quantized keys or (as the reference's
+    micro-benchmark does) arbitrary codes and randn metadata, byte-per-code or packed 6-bit rows."""
+    from polarquant_amd.kernel4group import attention_decode_forward_triton_impl
+    rnd = random.Random(9000 + seed)
+    N, Nk = rnd.choice(HEADS)
+    rb, tb = rnd.choice(BITS)
+    B, Nb = rnd.randint(1, 3), rnd.randint(1, 6)
+    dtype = torch.bfloat16 if seed % 4 == 3 else torch.float16
+    synthetic = rnd.random() < 0.4
+    packed = (rb, tb) == (3, 3) and rnd.random() < 0.6
+    print("case", dict(seed=seed, N=N, Nk=Nk, bits=(rb, tb), B=B, Nb=Nb, dtype=str(dtype), synthetic=synthetic, packed=packed), flush=True)
+    g = torch.Generator().manual_seed(seed)
+    q = wl.make_half((B, N, 1, 128), g, dtype)
+    if synthetic:
+        codes = torch.randint(0, 1 << (rb + tb), (B, Nk, Nb, 128, 64), generator=g, dtype=torch.uint8)
+        meta = [torch.randn(B, Nk, Nb, 1, 64, generator=g).to(dtype) for _ in range(4)]
+        if rnd.random() < 0.5:
+            meta[0][0, 0, 0, 0, :5] = 0
+            meta[2][0, 0, 0, 0, 5:9] = 0
+    else:
+        quant = po.quantize_and_pack_nbit(wl.make_keys(B, Nk, Nb * 128, 5e5, g, dtype), rb, tb)
+        codes, meta = quant[0], list(quant[1:])
+    ref = po.decode_scores(q, codes, *meta, rbits=rb, tbits=tb, dtype=torch.float64)
+    dev_codes = po.pack_codes6(codes) if packed else codes
+    got = attention_decode_forward_triton_impl(q.to(gpu), dev_codes.to(gpu), *[m.to(gpu) for m in meta], rbits=rb, tbits=tb)
+    assert got.shape == (B, N, 1, Nb * 128) and got.dtype == torch.float32
+    got = got.double().cpu()
+    # the per-pair table is built in fp32: error relative to the largest magnitude a row can reach
+    bound = ref.abs().amax(-1, keepdim=True).clamp_min(1e-30)
+    assert float(((got - ref).abs() / bound).max()) < 2e-5
