@@ -75,10 +75,14 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     assert gate.dim() <= 2 or all(gate.stride(i) == gate.stride(i + 1) * gate.shape[i + 1] for i in range(gate.dim() - 2)), \
         "rows must be evenly spaced"
     y = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    esz = gate.element_size()
     with torch.cuda.device(gate.device):
-        rc = _ffi.lib().pq_silu_mul(gate.data_ptr(), up.data_ptr(), y.data_ptr(), rows, cols, stride, _dtype_code(gate),
-                                    _stream_ptr(gate.device))
-    _ffi.check(rc, "pq_silu_mul")
+        for r0 in range(0, rows, 65535):          # one launch covers at most 65535 rows (a prompt has more)
+            n = min(65535, rows - r0)
+            rc = _ffi.lib().pq_silu_mul(gate.data_ptr() + r0 * stride * esz, up.data_ptr() + r0 * stride * esz,
+                                        y.data_ptr() + r0 * cols * esz, n, cols, stride, _dtype_code(gate),
+                                        _stream_ptr(gate.device))
+            _ffi.check(rc, "pq_silu_mul")
     return y
 
 

@@ -5,7 +5,7 @@ Reports prefill seconds, decode tokens/s and KV-cache bytes per token.  Mirrors 
 reference's throughput script (benchmark/benchmark_throughput.py:15-113): one timed prefill,
 then the timed greedy loop with EOS made unreachable.
 
-    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32] [--graph] [--values4]
+    python -m polarquant_amd.e2e_bench [--batch 8] [--prompt 16384] [--new 256] [--layers 32] [--graph] [--values4] [--fused-prefill]
 
 --graph replays the decode step from a captured HIP graph (polarquant_amd/graph_decode.py)
 instead of driving ~40 launches per layer from Python.
@@ -47,6 +47,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--graph", action="store_true")
     ap.add_argument("--values4", action="store_true", help="4-bit values as well (the reference's Mixed variant)")
+    ap.add_argument("--fused-prefill", action="store_true", help="with --graph: fused norm / SiLU kernels in the prompt pass too")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = PolarConfig.llama3_8b(num_hidden_layers=args.layers, cache_capacity=args.prompt + args.new + 128,
@@ -58,7 +59,7 @@ def main():
     with torch.no_grad():
         if args.graph:
             from .graph_decode import PolarGraphDecoder
-            dec = PolarGraphDecoder(model, max_len=args.prompt + args.new + 128)
+            dec = PolarGraphDecoder(model, max_len=args.prompt + args.new + 128, fused_prefill=args.fused_prefill)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             logits = dec.prefill(ids)

@@ -115,6 +115,43 @@ def test_graph_decoder_with_left_padded_prompt(gpu, mixed):
         assert not torch.allclose(dec_n.step(tok)[2].float(), dec_e.step(tok)[2].float(), atol=1e-3)
 
 
+def test_fused_prompt_pass_agrees_with_the_eager_model_to_rounding(gpu):
+    """fused_prefill: norms and SiLU * up of the prompt pass through the fused kernels (more rows than one
+    launch of the activation kernel takes are split).  Logits of the prompt and of later steps agree with the
+    eager model to rounding; the cache bookkeeping is the same."""
+    torch.manual_seed(23)
+    cfg = _tiny()
+    model = LlamaPolarForCausalLM(cfg).half().to(gpu).eval()
+    B, L, new = 2, 300, 12
+    ids = torch.randint(0, cfg.vocab_size, (B, L), device=gpu)
+    dec = PolarGraphDecoder(model, max_len=L + new + 8, fused_prefill=True)
+    with torch.no_grad():
+        ref = model(input_ids=ids, attention_mask=None, past_key_values=None, num_logits_to_keep=1)
+        got = dec.prefill(ids)
+        rl = ref.logits.float()
+        assert (got.float() - rl).abs().max().item() <= 2e-2 * max(1.0, rl.abs().max().item())
+        cache, tok = ref.past_key_values, ref.logits.argmax(-1)
+        assert dec.kv_len == L and dec.arenas[0].n_groups == cache[0][1].shape[2] == 2
+        for s in range(new):
+            ref = model(input_ids=tok, attention_mask=None, past_key_values=cache, num_logits_to_keep=1)
+            cache = ref.past_key_values
+            got = dec.step(tok)
+            rl = ref.logits.float()
+            assert (got.float() - rl).abs().max().item() <= 2e-2 * max(1.0, rl.abs().max().item()), s
+            tok = ref.logits.argmax(-1)
+
+
+def test_silu_mul_splits_more_rows_than_one_launch_takes(gpu):
+    from polarquant_amd.decode_ops import silu_mul
+    g = torch.Generator().manual_seed(3)
+    gate = torch.randn(70000, 64, generator=g).half().to(gpu)
+    up = torch.randn(70000, 64, generator=g).half().to(gpu)
+    y = silu_mul(gate, up)
+    ref = (torch.nn.functional.silu(gate.float()).half().float() * up.float()).half()
+    assert (y.float() - ref.float()).abs().max().item() <= 2e-3 * ref.float().abs().max().item()
+    assert torch.equal(y[65535:], silu_mul(gate[65535:].contiguous(), up[65535:].contiguous()))
+
+
 def test_graph_decoder_rejects_overflow(gpu):
     torch.manual_seed(12)
     cfg = _tiny(layers=1)
