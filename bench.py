@@ -198,6 +198,21 @@ def main():
     ms = time_events(step, args.steps, args.warmup)
     k_ms = kernel_duration_ms(partials_only, args.steps)
 
+    # what a plain read-once kernel is delivered on this GPU: the V tensors of the two input sets
+    # (1 GiB each) streamed alternately, one wavefront per SIMD and two per SIMD, best of the two
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream_gbps = 0.0
+    for n_waves in (1024, 2048):
+        got = [0]
+
+        def stream_once():
+            v = sets[turn[0] & 1]["v"]
+            turn[0] += 1
+            got[0] = lib.pq_stream_read(v.data_ptr(), v.numel() * 2, n_waves, sink.data_ptr(), _stream_ptr(dev))
+            assert got[0] > 0
+        s_ms = time_events(stream_once, 20, 4)
+        stream_gbps = max(stream_gbps, got[0] / (s_ms * 1e-3) / 1e9)
+
     alg_bytes = wl.algorithmic_bytes(Nk, N, [w["n_groups"] * 128] * B, [w["n_resid"]] * B, sh.rbits, sh.tbits)
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     result = {
@@ -213,7 +228,9 @@ def main():
         "pct_of_hbm_peak": round(100 * alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "kernel": "attn_kernel<F16,4,4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES},
+                     "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "plain_stream_read_gbps": round(stream_gbps, 1),
+                     "frac_of_plain_stream_read": round(achieved / stream_gbps, 4)},
     }
     # the same step with the values of the quantized groups in 4 bits (the reference's Mixed variant)
     if not args.no_values4:

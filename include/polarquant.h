@@ -80,6 +80,14 @@ int pq_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const 
 int pq_validate_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const void *w_up, const void *bias,
                                const void *y, int64_t y_row_stride, int M, int N, int K, int dtype);
 
+/* Measurement aid (no reference counterpart): a plain streaming read of `bytes` bytes at `src` by
+ * `n_wavefronts` wavefronts, each reading one contiguous slice with 16 KiB in flight, with the
+ * non-temporal loads the decode kernels use.  Time it to learn what a read-once kernel can be
+ * delivered on the GPU at hand.  Returns the number of bytes the launch reads (slices are whole
+ * multiples of 16 KiB, so slightly fewer than `bytes`), 0 on a bad argument or a failed launch.
+ * `sink`: 4 writable bytes on the device (practically never written). */
+size_t pq_stream_read(const void *src, size_t bytes, int n_wavefronts, uint32_t *sink, void *stream);
+
 /* Layout converter for code rows: pack != 0 turns `n_rows` byte-per-code rows (64 bytes each, every
  * code < 64) into packed 6-bit rows (48 bytes each), pack == 0 the reverse.  For caches built by the
  * reference (always byte-per-code) that are to be kept packed, and back.  No reference counterpart. */

@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libpolarquant_hip.so")
-SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_attn.hip"]
+SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_stream.hip", "pq_attn.hip"]
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]

@@ -324,6 +324,16 @@ int pq_linear_small_m(const void* x, int64_t x_row_stride, const void* w, const 
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
+size_t pq_stream_read(const void* src, size_t bytes, int n_wavefronts, uint32_t* sink, void* stream) {
+    if (!src || !sink || n_wavefronts <= 0 || n_wavefronts > (1 << 20) || !aligned(src, 16) || !aligned(sink, 4)) return 0;
+    const size_t chunk = 16 * 1024;                       // what one wavefront requests per trip
+    size_t per_wave = bytes / static_cast<size_t>(n_wavefronts) / chunk * chunk;
+    if (per_wave > (size_t{1} << 31) - chunk) per_wave = ((size_t{1} << 31) - chunk) / chunk * chunk;
+    if (per_wave == 0) return 0;
+    if (pq::launch_stream_read(src, per_wave, n_wavefronts, sink, static_cast<hipStream_t>(stream)) != 0) return 0;
+    return per_wave * static_cast<size_t>(n_wavefronts);
+}
+
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;

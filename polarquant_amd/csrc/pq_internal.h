@@ -32,6 +32,8 @@ int launch_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, bool 
 int launch_small_m_linear(const void* x, int64_t x_stride, const void* w, const void* w_up, const void* bias, void* y,
                           int64_t y_stride, int M, int N, int K, int dtype, hipStream_t st);
 
+int launch_stream_read(const void* src, size_t bytes_per_wave, int n_waves, uint32_t* sink, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;

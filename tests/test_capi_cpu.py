@@ -215,6 +215,12 @@ def test_linear_small_m_rejects_bad_arguments(lib):
     assert lib.pq_linear_small_m(None, 4096, P, None, None, P, 4096, 8, 4096, 4096, 1, None) == -1
 
 
+def test_stream_read_rejects_bad_arguments(lib):
+    assert lib.pq_stream_read(None, 1 << 30, 1024, P, None) == 0 and lib.pq_stream_read(P, 1 << 30, 1024, None, None) == 0
+    assert lib.pq_stream_read(P, 1 << 30, 0, P, None) == 0 and lib.pq_stream_read(P + 8, 1 << 30, 1024, P, None) == 0
+    assert lib.pq_stream_read(P, 1000, 1024, P, None) == 0          # less than one 16 KiB trip per wavefront
+
+
 def test_convert_codes6_rejects_bad_arguments(lib):
     assert lib.pq_convert_codes6(None, P, 4, 1, None) == -1 and lib.pq_convert_codes6(P, None, 4, 0, None) == -1
     assert lib.pq_convert_codes6(P, P, 0, 1, None) == -2
