@@ -709,6 +709,17 @@ def top_k_top_p_filtering(logits, top_k: int = 0, top_p: float = 1.0, filter_val
     return logits
 
 
+def return_top_p_filtered_indices(logits, top_p):
+    """Boolean mask over the vocabulary of [batch, positions, vocab] logits: True for the tokens nucleus filtering
+    keeps, i.e. the most probable ones up to and including the one whose cumulative probability first exceeds
+    `top_p` (models/modeling_llama_polar.py:592-606; no caller in the reference)."""
+    order = logits.argsort(dim=-1, descending=True)
+    over = logits.gather(-1, order).softmax(-1).cumsum(-1) > top_p
+    keep_sorted = torch.ones_like(over)
+    keep_sorted[..., 1:] = ~over[..., :-1]
+    return torch.zeros_like(over).scatter_(-1, order, keep_sorted)
+
+
 def sample(logits, generation_config, do_sample=False):
     if do_sample:
         logits_ = top_k_top_p_filtering(logits.view(-1, logits.size(-1)) / generation_config.temperature,

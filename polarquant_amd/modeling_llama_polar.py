@@ -4,7 +4,7 @@ LlamaPolarModel, LlamaPolarForCausalLM, generate, sample, top_k_top_p_filtering.
 from .kernel4group import attention_decode_forward_triton_impl  # noqa: F401  (re-exported, as the reference imports it here)
 from .modeling_common import (  # noqa: F401
     CausalLMOutputWithPast, GenerationConfig, PolarCache, PolarConfig, PolarDecoderLayer, PolarForCausalLM,
-    PolarGroupAttention, PolarMixedGroupAttention, PolarModel, PolarSnapKVAttention, apply_rotary_pos_emb, generate, repeat_kv, repeat_kv_quant, sample,
+    PolarGroupAttention, PolarMixedGroupAttention, PolarModel, PolarSnapKVAttention, apply_rotary_pos_emb, generate, repeat_kv, repeat_kv_quant, return_top_p_filtered_indices, sample,
     top_k_top_p_filtering)
 
 

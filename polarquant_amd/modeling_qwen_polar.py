@@ -6,7 +6,7 @@ Qwen's ratios (7, 6, 5) natively."""
 from .kernel4group import attention_decode_forward_triton_impl  # noqa: F401
 from .modeling_common import (  # noqa: F401
     CausalLMOutputWithPast, GenerationConfig, PolarCache, PolarConfig, PolarDecoderLayer, PolarForCausalLM,
-    PolarGroupAttention, PolarModel, apply_rotary_pos_emb, generate, repeat_kv, repeat_kv_quant, sample,
+    PolarGroupAttention, PolarModel, apply_rotary_pos_emb, generate, repeat_kv, repeat_kv_quant, return_top_p_filtered_indices, sample,
     top_k_top_p_filtering)
 
 

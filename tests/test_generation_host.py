@@ -116,3 +116,15 @@ def test_hf_generation_hook_is_batch_one_and_feeds_the_last_token():
     with pytest.raises(NotImplementedError):
         hook(None, torch.zeros(2, 3, dtype=torch.long))
     assert PolarForCausalLM._prepare_cache_for_generation(None, 1, 2, 3) is None
+
+
+def test_top_p_keep_mask_matches_the_filter():
+    from polarquant_amd.modeling_common import return_top_p_filtered_indices
+    probs = torch.tensor([[[0.05, 0.5, 0.15, 0.3], [0.25, 0.25, 0.4, 0.1]]])
+    keep = return_top_p_filtered_indices(probs.log(), 0.7)
+    assert keep.dtype == torch.bool and keep.tolist() == [[[False, True, False, True], [True, True, True, False]]]
+    g = torch.Generator().manual_seed(4)
+    logits = torch.randn(2, 3, 19, generator=g, dtype=torch.float64)
+    keep = return_top_p_filtered_indices(logits, 0.6)
+    filtered = top_k_top_p_filtering(logits.reshape(-1, 19).clone(), top_k=0, top_p=0.6).reshape(2, 3, 19)
+    assert torch.equal(keep, torch.isfinite(filtered))
