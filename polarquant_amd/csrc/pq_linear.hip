@@ -132,27 +132,164 @@ __global__ __launch_bounds__(kWave * KSPLIT) void small_m_linear_kernel(
                    static_cast<uint32_t>(out[2]) | (static_cast<uint32_t>(out[3]) << 16));
 }
 
-// Four wavefronts per workgroup and short stages measured best at the decode shapes of Llama-3-8B
-// (K-split 4 / 8 / 16 and stages of 2 / 4 / 8 loads were swept); K / KSPLIT must stay a whole
-// number of 32-wide steps.
+// M <= 8: each 16 x 16 MFMA tile is used as two 8 x 8 tiles on its diagonal.  Tile rows 0-7 are 8 rows
+// of W over the first 32 of a 64-wide k-step, tile rows 8-15 the SAME 8 rows over the second 32; tile
+// columns 0-7 are the rows of x over the first 32, columns 8-15 over the second 32.  Then
+// y[m][n] = C[n][m] + C[n + 8][m + 8] and the off-diagonal quarters are ignored.  No lane loads a
+// duplicate row of x, a wavefront load of W covers 8 rows x 128 contiguous bytes (whole cache lines,
+// which is what lets the weight stream carry the non-temporal hint: with half lines the hint drops a
+// line before its second half is asked for), and the workgroup's 16 rows of W are two such tiles that
+// share one x operand: per 64-wide step two W loads and one x load instead of four and four.
+template <bool GATED, int kStage>
+struct Stage8T {
+    u32x4_l w[2][kStage], x[kStage], u[GATED ? 2 : 1][GATED ? kStage : 1];
+};
+
+template <typename T, int KSPLIT, bool GATED, int kStage>
+__global__ __launch_bounds__(kWave * KSPLIT) void small_m8_linear_kernel(
+    const uint16_t* __restrict__ x, int64_t x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ w_up,
+    const uint16_t* __restrict__ bias, uint16_t* __restrict__ y, int64_t y_stride, int M, int K) {
+    __shared__ float part[KSPLIT][GATED ? 4 : 2][4][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int row = r & 7, chunk = (r >> 3) * 4 + g;       // W row inside an 8-row tile == x row; 16-byte piece of the step
+    const int n0 = blockIdx.x * 16;
+    const int klen = K / KSPLIT, steps = klen / 64;
+    const int m = row < M ? row : 0;                       // tile columns >= M repeat row 0 and are never stored
+    const size_t koff = static_cast<size_t>(wv) * klen + 8 * chunk;
+    const uint16_t* wp = w + static_cast<size_t>(n0 + row) * K + koff;
+    const uint16_t* up = GATED ? w_up + static_cast<size_t>(n0 + row) * K + koff : nullptr;
+    const uint16_t* xp = x + static_cast<size_t>(m) * x_stride + koff;
+    const size_t half_tile = static_cast<size_t>(8) * K;   // rows n0 + 8 .. n0 + 15
+
+    floatx4_l acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}}, acu[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    auto ldw = [](const uint16_t* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4_l*>(p)); };
+    auto load = [&](Stage8T<GATED, kStage>& st, int s0) {          // branch-free, see small_m_linear_kernel
+        static_for<kStage>([&](auto U) {
+            constexpr int u = decltype(U)::value;
+            st.w[0][u] = ldw(wp + (s0 + u) * 64);
+            st.w[1][u] = ldw(wp + half_tile + (s0 + u) * 64);
+            if constexpr (GATED) {
+                st.u[0][u] = ldw(up + (s0 + u) * 64);
+                st.u[1][u] = ldw(up + half_tile + (s0 + u) * 64);
+            }
+            st.x[u] = *reinterpret_cast<const u32x4_l*>(xp + (s0 + u) * 64);
+        });
+    };
+    auto compute = [&](const Stage8T<GATED, kStage>& st) {
+        static_for<kStage>([&](auto U) {
+            constexpr int u = decltype(U)::value;
+            acc[0] = mfma32<T>(st.w[0][u], st.x[u], acc[0]);
+            acc[1] = mfma32<T>(st.w[1][u], st.x[u], acc[1]);
+            if constexpr (GATED) {
+                acu[0] = mfma32<T>(st.u[0][u], st.x[u], acu[0]);
+                acu[1] = mfma32<T>(st.u[1][u], st.x[u], acu[1]);
+            }
+        });
+    };
+    const int full = steps / kStage;
+    if (full > 0) {
+        Stage8T<GATED, kStage> sa, sb;
+        load(sa, 0);
+        int st = 0;
+        while (st + 2 < full) {
+            load(sb, (st + 1) * kStage);
+            compute(sa);
+            load(sa, (st + 2) * kStage);
+            compute(sb);
+            st += 2;
+        }
+        if (full - st == 2) {
+            load(sb, (st + 1) * kStage);
+            compute(sa);
+            compute(sb);
+        } else {
+            compute(sa);
+        }
+    }
+    for (int s1 = full * kStage; s1 < steps; s1++) {
+        const u32x4_l xv1 = *reinterpret_cast<const u32x4_l*>(xp + s1 * 64);
+        acc[0] = mfma32<T>(ldw(wp + s1 * 64), xv1, acc[0]);
+        acc[1] = mfma32<T>(ldw(wp + half_tile + s1 * 64), xv1, acc[1]);
+        if constexpr (GATED) {
+            acu[0] = mfma32<T>(ldw(up + s1 * 64), xv1, acu[0]);
+            acu[1] = mfma32<T>(ldw(up + half_tile + s1 * 64), xv1, acu[1]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        part[wv][0][i][lane] = acc[0][i];
+        part[wv][1][i][lane] = acc[1][i];
+        if constexpr (GATED) { part[wv][2][i][lane] = acu[0][i]; part[wv][3][i][lane] = acu[1][i]; }
+    }
+    __syncthreads();
+    // lane (r < 8, g < 2) owns outputs y[r][n0 + 8h + 4g + i] (h: which 8-row tile), each the sum of the tile's
+    // entry (row 4g + i, column r) and its diagonal partner (row + 8, column + 8), which lane + 40 holds
+    if (wv != 0 || r >= 8 || r >= M || g >= 2) return;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint16_t out[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float s = 0.0f, t = 0.0f;
+#pragma unroll
+            for (int k = 0; k < KSPLIT; k++) {
+                s += part[k][h][i][lane] + part[k][h][i][lane + 40];
+                if constexpr (GATED) t += part[k][2 + h][i][lane] + part[k][2 + h][i][lane + 40];
+            }
+            if constexpr (GATED) {
+                const float gv = rnd_l<T>(s), uv = rnd_l<T>(t);
+                const float a = rnd_l<T>(gv / (1.0f + __expf(-gv)));
+                out[i] = f2lo<T>(a * uv);
+            } else {
+                if (bias) s += lo2f<T>(bias[n0 + 8 * h + 4 * g + i]);
+                out[i] = f2lo<T>(s);
+            }
+        }
+        *reinterpret_cast<uint2*>(y + static_cast<size_t>(r) * y_stride + n0 + 8 * h + 4 * g) =
+            make_uint2(static_cast<uint32_t>(out[0]) | (static_cast<uint32_t>(out[1]) << 16),
+                       static_cast<uint32_t>(out[2]) | (static_cast<uint32_t>(out[3]) << 16));
+    }
+}
+
+// Launch shapes measured at the decode shapes of Llama-3-8B (K-split 4 / 8 / 16 and stages of 1 / 2 / 4 / 8
+// loads were swept): the 16-row kernel runs four wavefronts per workgroup with stages of 4 (2 when gated); the
+// M <= 8 kernel four wavefronts with stages of 1, or eight with stages of 2 when K >= 8192 (down_proj).
+// K / KSPLIT must stay a whole number of k-steps.
 int launch_small_m_linear(const void* x, int64_t x_stride, const void* w, const void* w_up, const void* bias, void* y,
                           int64_t y_stride, int M, int N, int K, int dtype, hipStream_t st) {
-    int ks = 4;
-    while (ks > 1 && (K % (32 * ks)) != 0) ks >>= 1;
-    dim3 grid(N / 16), block(kWave * ks);
-#define PQ_LAUNCH_L(T, KS, G, S)                                                                                     \
-    hipLaunchKernelGGL((small_m_linear_kernel<T, KS, G, S>), grid, block, 0, st, (const uint16_t*)x, x_stride,     \
-                       (const uint16_t*)w, (const uint16_t*)w_up, (const uint16_t*)bias, (uint16_t*)y, y_stride, M, K)
-#define PQ_LAUNCH_LK(T, G, S)                                                                                        \
-    do {                                                                                                             \
-        if (ks == 4) PQ_LAUNCH_L(T, 4, G, S);                                                                        \
-        else if (ks == 2) PQ_LAUNCH_L(T, 2, G, S);                                                                   \
-        else PQ_LAUNCH_L(T, 1, G, S);                                                                                \
-    } while (0)
     const bool gated = w_up != nullptr;
-    if (dtype == 0) { if (gated) PQ_LAUNCH_LK(F16, true, 2); else PQ_LAUNCH_LK(F16, false, 4); }
-    else            { if (gated) PQ_LAUNCH_LK(BF16, true, 2); else PQ_LAUNCH_LK(BF16, false, 4); }
-#undef PQ_LAUNCH_LK
+    const bool m8 = M <= 8 && (K % 64) == 0;
+    const int kstep = m8 ? 64 : 32;
+    int ks = (m8 && K >= 8192) ? 8 : 4;
+    while (ks > 1 && (K % (kstep * ks)) != 0) ks >>= 1;
+    dim3 grid(N / 16), block(kWave * ks);
+#define PQ_LAUNCH_L(KERNEL, T, KS, G, S)                                                                             \
+    hipLaunchKernelGGL((KERNEL<T, KS, G, S>), grid, block, 0, st, (const uint16_t*)x, x_stride,                      \
+                       (const uint16_t*)w, (const uint16_t*)w_up, (const uint16_t*)bias, (uint16_t*)y, y_stride, M, K)
+#define PQ_LAUNCH_M8(T, G)                                                                                           \
+    do {                                                                                                             \
+        if (ks == 8) PQ_LAUNCH_L(small_m8_linear_kernel, T, 8, G, 2);                                                \
+        else if (ks == 4) PQ_LAUNCH_L(small_m8_linear_kernel, T, 4, G, 1);                                           \
+        else if (ks == 2) PQ_LAUNCH_L(small_m8_linear_kernel, T, 2, G, 1);                                           \
+        else PQ_LAUNCH_L(small_m8_linear_kernel, T, 1, G, 1);                                                        \
+    } while (0)
+#define PQ_LAUNCH_M16(T, G, S)                                                                                       \
+    do {                                                                                                             \
+        if (ks == 4) PQ_LAUNCH_L(small_m_linear_kernel, T, 4, G, S);                                                 \
+        else if (ks == 2) PQ_LAUNCH_L(small_m_linear_kernel, T, 2, G, S);                                            \
+        else PQ_LAUNCH_L(small_m_linear_kernel, T, 1, G, S);                                                         \
+    } while (0)
+#define PQ_LAUNCH_LM(T)                                                                                              \
+    do {                                                                                                             \
+        if (m8) { if (gated) PQ_LAUNCH_M8(T, true); else PQ_LAUNCH_M8(T, false); }                                   \
+        else    { if (gated) PQ_LAUNCH_M16(T, true, 2); else PQ_LAUNCH_M16(T, false, 4); }                           \
+    } while (0)
+    if (dtype == 0) PQ_LAUNCH_LM(F16);
+    else PQ_LAUNCH_LM(BF16);
+#undef PQ_LAUNCH_LM
+#undef PQ_LAUNCH_M16
+#undef PQ_LAUNCH_M8
 #undef PQ_LAUNCH_L
     return static_cast<int>(hipGetLastError());
 }

@@ -176,18 +176,20 @@ class PolarGraphDecoder:
         for li, (layer, ar) in enumerate(zip(layers, self.arenas)):
             att, mlp = layer.self_attn, layer.mlp
             nq, nkv = att.num_heads * att.head_dim, att.num_key_value_heads * att.head_dim
-            qkv = torch.nn.functional.linear(h, att._wqkv, att._bqkv)           # [B,1,(N+2Nk)*128]
+            own = self.small_m_gemm and B <= 16 and all(
+                w_.is_contiguous() and w_.shape[0] % 16 == 0 and w_.shape[1] % 32 == 0
+                for w_ in (att._wqkv, att.o_proj.weight, mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
+            if own:
+                qkv = linear_small_m(h, att._wqkv, att._bqkv)                   # [B,1,(N+2Nk)*128]
+            else:
+                qkv = torch.nn.functional.linear(h, att._wqkv, att._bqkv)
             q_lin, k_lin, v_lin = qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:]
             v_dst, v_row = (ar.vres, self.resid_idx) if self.mixed else (ar.v, self.pos)
             q = rope_append(q_lin, k_lin, v_lin, self.cos_table, self.sin_table, self.pos, ar.kres, self.resid_idx,
                             v_dst, v_row, att.num_heads, att.num_key_value_heads)
             o = self._attend(att, ar, q)
-            own = self.small_m_gemm and B <= 16 and all(
-                lin.weight.is_contiguous() and lin.weight.shape[0] % 16 == 0 and lin.weight.shape[1] % 32 == 0
-                for lin in (att.o_proj, mlp.gate_proj, mlp.up_proj, mlp.down_proj))
             pn = layer.post_attention_layernorm
             if own and mlp.gate_proj.bias is None and mlp.up_proj.bias is None:
-                # (the fused q|k|v projection stays with the library: equal time at that shape)
                 a = linear_small_m(o.reshape(B, 1, -1), att.o_proj.weight, att.o_proj.bias)
                 h = rmsnorm(x, pn.weight, pn.variance_epsilon, residual=a, sum_out=x)
                 act = linear_small_m(h, mlp.gate_proj.weight, up_weight=mlp.up_proj.weight)

@@ -20,7 +20,7 @@ def _check(y, ref, dtype, ulps=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K,bias", [(8, 6144, 4096, False), (1, 4096, 4096, False), (16, 4096, 14336, False),
+@pytest.mark.parametrize("M,N,K,bias", [(8, 6144, 4096, False), (1, 4096, 4096, False), (16, 4096, 14336, False), (8, 4096, 14336, False), (9, 256, 4096, True), (4, 64, 160, False),
                                         (5, 1024, 3584, True), (8, 64, 96, True), (3, 18944, 3584, False), (8, 4608, 3584, True)])
 def test_linear_matches_fp32_matmul(gpu, dtype, M, N, K, bias):
     print("case", dtype, M, N, K, bias, flush=True)
