@@ -3,7 +3,9 @@
 // (models/modeling_llama_polar.py:47-52, :131 and the decoder layer's MLP, :456-486).
 //
 // At M <= 16 the product is a stream of the weight matrix through HBM, 2*M flops per weight
-// byte: the kernel is laid out for the stream, not for the matrix cores.  A workgroup owns
+// byte: the kernels are laid out for the stream, not for the matrix cores.  Two of them:
+// small_m_linear_kernel (any M <= 16, described here) and small_m8_linear_kernel (M <= 8, further
+// down: whole-line loads, half the x operand traffic).  A workgroup owns
 // 16 output columns (16 rows of W) and splits K over its KSPLIT wavefronts; each wavefront
 // keeps two stages of kStage 16-byte loads per lane in flight (ping-pong) and feeds them to
 // v_mfma_f32_16x16x32 with the W rows as the A operand and x (rows >= M unused) as the B operand:
