@@ -31,9 +31,12 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def _compile(src: str) -> str:
-    obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+TIMERS_LIB = os.path.join(HERE, "libpolarquant_hip_timers.so")
+
+
+def _compile(src: str, defines=(), tag: str = "") -> str:
+    obj = os.path.join(OBJ, os.path.splitext(src)[0] + tag + ".o")
+    cmd = [_hipcc()] + FLAGS + ["-D" + d for d in defines] + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -43,21 +46,25 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, phase_timers: bool = False) -> str:
+    """The library the package loads; or, with phase_timers, a second library (same ABI, not loaded by default)
+    whose attention kernel times its phases with the wall clock and prints them: a measuring build for
+    `python -m polarquant_amd.phase_timing`, a few percent slower than the real one."""
     os.makedirs(OBJ, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    lib, defines, tag = (TIMERS_LIB, ("PQ_ATTN_PHASE_TIMERS",), ".timers") if phase_timers else (LIB, (), "")
     with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
-    tmp = LIB + ".tmp"
+        objs = list(ex.map(lambda s_: _compile(s_, defines, tag), srcs))
+    tmp = lib + ".tmp"
     r = subprocess.run([_hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs,
                        capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
-    os.replace(tmp, LIB)
+    os.replace(tmp, lib)
     if verbose:
-        print("built", LIB)
-    return LIB
+        print("built", lib)
+    return lib
 
 
 if __name__ == "__main__":
-    build()
+    build(phase_timers="--phase-timers" in sys.argv[1:])

@@ -28,6 +28,27 @@
 #include "pq_device.h"
 #include "pq_internal.h"
 
+// Measuring build only (-DPQ_ATTN_PHASE_TIMERS, `python -m polarquant_amd.build --phase-timers`): wall-clock
+// (100 MHz) time of each phase of the group loop, summed per wavefront and printed by a few of them.
+#ifdef PQ_ATTN_PHASE_TIMERS
+#define PQ_T_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}, pt_mark_ = 0; const long long pt_begin_ = wall_clock64()
+#define PQ_T_MARK() pt_mark_ = wall_clock64()
+#define PQ_T_ADD(i) do { const long long pt_now_ = wall_clock64(); pt_[i] += pt_now_ - pt_mark_; pt_mark_ = pt_now_; } while (0)
+#define PQ_T_KEEP(x) asm volatile("" ::"v"(x))
+#define PQ_T_REPORT(n_groups)                                                                                        \
+    do {                                                                                                             \
+        if (threadIdx.x == 0 && blockIdx.x % 97 == 0)                                                                \
+            printf("pq_phase block %d groups %d total %lld table %lld value_issue %lld code_wait %lld code_issue %lld score %lld softmax_pv %lld\n", \
+                   static_cast<int>(blockIdx.x), n_groups, wall_clock64() - pt_begin_, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]); \
+    } while (0)
+#else
+#define PQ_T_DECL
+#define PQ_T_MARK()
+#define PQ_T_ADD(i)
+#define PQ_T_KEEP(x)
+#define PQ_T_REPORT(n_groups)
+#endif
+
 namespace pq {
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -407,12 +428,15 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                 }
             };
             load_values(0, static_cast<uint32_t>(2 * g0) * kWave, true);
+            PQ_T_DECL;
             for (int grp = g0; grp < g1; grp++) {
+                PQ_T_MARK();
                 asm volatile("" ::: "memory");
                 const float cdv = build_lut<T, TB, REPP>(lut, lane, qx, qy, mrs, mrm, mts, mtm);
                 float cds[kPairs];
                 broadcast_cd(cdv, cds);
                 asm volatile("" ::: "memory");
+                PQ_T_ADD(0);
                 if (grp + 1 < g1) {
                     const int o = (grp + 1) * kPairs;
                     mrs = prs[o]; mrm = prm[o]; mts = pts[o]; mtm = ptm[o];
@@ -422,7 +446,9 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     const int tt = 2 * grp + half;
                     const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
                     // past the last tile of this slice the loads run off the buffer's end and return zeros
+                    PQ_T_MARK();
                     load_values(half ^ 1, tok0 + kWave, half == 0 || grp + 1 < g1);
+                    PQ_T_ADD(1);
                     uint32_t cw[16];
                     if constexpr (PK6) {
                         uint32_t pk[12];
@@ -437,15 +463,21 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                             cw[4 * i] = cnext[i].x; cw[4 * i + 1] = cnext[i].y; cw[4 * i + 2] = cnext[i].z; cw[4 * i + 3] = cnext[i].w;
                         }
                     }
+                    PQ_T_KEEP(cw[0]);
+                    PQ_T_KEEP(cw[15]);
+                    PQ_T_ADD(2);
                     if (half == 0 || grp + 1 < g1) {
 #pragma unroll
                         for (int i = 0; i < kRowLoads; i++)
                             cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(tt + 1) * (kWave * kRowB) + 16 * i);
                     }
+                    PQ_T_ADD(3);
                     float s[REPP];
 #pragma unroll
                     for (int j = 0; j < REPP; j++) s[j] = 0.0f;
                     score_token<TB, REPP>(lut, cw, cds, s);
+                    PQ_T_KEEP(s[0]);
+                    PQ_T_ADD(4);
                     const bool keep = has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(tok0), 0) != 0) : true;
 #pragma unroll
                     for (int j = 0; j < REPP; j++) s[j] = keep ? s[j] * scale_log2 : -INFINITY;
@@ -454,8 +486,11 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                     } else {
                         softmax_pv_tile<T, REPP>(st, s, vv[half].r, pbuf, lane);
                     }
+                    PQ_T_KEEP(st.acc[0][0]);
+                    PQ_T_ADD(5);
                 }
             }
+            PQ_T_REPORT(g1 - g0);
             if constexpr (V4) finish_v4<REPP>(st, lane);
         }
     }

@@ -1,0 +1,91 @@
+"""Where a wavefront of the fused decode-attention kernel spends its time, phase by phase.
+
+Needs the measuring build of the library (`python -m polarquant_amd.build --phase-timers`), whose attention
+kernel brackets its phases with the 100 MHz wall clock and lets every 97th wavefront print its sums.  The
+instrumentation costs a few percent, so totals are a little above the real kernel's; the split is what matters.
+
+    python -m polarquant_amd.phase_timing [--config 1] [--values4]
+
+Phases of one 128-token group: table = build of the per-group angle table in LDS; value_issue = issue of the
+next tile's value loads (16 buffer loads; the time is spent in the issue itself when the compute unit's miss
+queue is full); code_wait = arrival of this tile's codes; code_issue = issue of the next tile's code loads;
+score = the 64-code table walk; softmax_pv = mask, softmax update and the P.V MFMAs (including the arrival of
+the value tile requested a tile earlier).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import re
+import sys
+import tempfile
+
+import torch
+
+from . import _ffi
+from .build import TIMERS_LIB
+
+PHASES = ("table", "value_issue", "code_wait", "code_issue", "score", "softmax_pv")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--config", type=int, default=1)
+    ap.add_argument("--values4", action="store_true")
+    args = ap.parse_args()
+    if not os.path.exists(TIMERS_LIB):
+        sys.exit("phase_timing: build the measuring library first: python -m polarquant_amd.build --phase-timers")
+    _ffi.LIB_PATH = TIMERS_LIB
+    from . import workloads as wl
+    from .attention import polar_decode_attention, polar_decode_attention_v4
+    from .values import quantize_values
+    dev = torch.device("cuda:0")
+    w = wl.build_workload(args.config, dev)
+    sh = w["shape"]
+    kw = dict(rbits=sh.rbits, tbits=sh.tbits)
+    if w.get("groups_per_seq") is not None:
+        kw.update(n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=int(w["groups_per_seq"].sum()))
+    if args.values4:
+        L = w["n_groups"] * 128
+        vq = quantize_values(w["v"][:, :, :L])
+        vres = torch.zeros(w["v"].shape[0], w["v"].shape[1], 128, 128, dtype=w["v"].dtype, device=dev)
+        vres[:, :, :1] = w["v"][:, :, L:L + 1]
+        kw.pop("total_groups", None)
+        call = lambda: polar_decode_attention_v4(w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], **kw)
+    else:
+        call = lambda: polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], **kw)
+    torch.cuda.synchronize()
+    sys.stdout.flush()
+    # the kernel prints from the device: collect the process's stdout of one launch in a file
+    with tempfile.TemporaryFile(mode="w+b") as tmp:
+        saved = os.dup(1)
+        os.dup2(tmp.fileno(), 1)
+        try:
+            call()
+            torch.cuda.synchronize()
+        finally:
+            os.dup2(saved, 1)
+            os.close(saved)
+        tmp.seek(0)
+        text = tmp.read().decode(errors="replace")
+    rows = []
+    for line in text.splitlines():
+        m = re.match(r"pq_phase block (\d+) groups (\d+) total (\d+) " + " ".join(p + r" (\d+)" for p in PHASES), line)
+        if m:
+            rows.append([int(v) for v in m.groups()])
+    rows = [r for r in rows if r[1] > 0]
+    if not rows:
+        sys.exit("phase_timing: no wavefront reported (is this the measuring build?)")
+    groups = sum(r[1] for r in rows)
+    per_group = {"total": sum(r[2] for r in rows) / groups * 0.01}
+    for i, p in enumerate(PHASES):
+        per_group[p] = sum(r[3 + i] for r in rows) / groups * 0.01
+    per_group["other"] = per_group["total"] - sum(per_group[p] for p in PHASES)
+    print(json.dumps({"config": args.config, "values4": bool(args.values4), "wavefronts_reporting": len(rows),
+                      "groups_per_wavefront": round(groups / len(rows), 2),
+                      "us_per_group": {k: round(v, 3) for k, v in per_group.items()}}))
+
+
+if __name__ == "__main__":
+    main()
