@@ -80,6 +80,21 @@ int pq_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const 
 int pq_validate_linear_small_m(const void *x, int64_t x_row_stride, const void *w, const void *w_up, const void *bias,
                                const void *y, int64_t y_row_stride, int M, int N, int K, int dtype);
 
+/* The q, k, v projections of a decode step as ONE product with the concatenated weight
+ * w_qkv [(N + 2 Nk) * 128, K] (q heads, then k heads, then v heads; optional bias of the same length),
+ * with RoPE and the two cache appends in its epilogue: pq_linear_small_m followed by pq_rope_append in
+ * one launch, bit-identical to that pair (models/modeling_llama_polar.py:47-59,77,98).  M <= 8 rows
+ * (sequences), K % 64 == 0.  cos / sin tables, pos, q_out, k_dst / k_row, v_dst / v_row: as for
+ * pq_rope_append, with B = M. */
+int pq_qkv_rope_append(const void *x, int64_t x_row_stride, const void *w_qkv, const void *bias, int M, int K, int dtype,
+                       const void *cos_table, const void *sin_table, int64_t table_rows, const int64_t *pos, void *q_out,
+                       void *k_dst, int64_t k_rows, const int64_t *k_row, void *v_dst, int64_t v_rows,
+                       const int64_t *v_row, int N, int Nk, void *stream);
+int pq_validate_qkv_rope_append(const void *x, int64_t x_row_stride, const void *w_qkv, const void *bias, int M, int K,
+                                int dtype, const void *cos_table, const void *sin_table, int64_t table_rows,
+                                const int64_t *pos, const void *q_out, const void *k_dst, int64_t k_rows,
+                                const int64_t *k_row, const void *v_dst, int64_t v_rows, const int64_t *v_row, int N, int Nk);
+
 /* Measurement aid (no reference counterpart): a plain streaming read of `bytes` bytes at `src` by
  * `n_wavefronts` wavefronts, each reading one contiguous slice with 16 KiB in flight, with the
  * non-temporal loads the decode kernels use.  Time it to learn what a read-once kernel can be

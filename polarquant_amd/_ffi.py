@@ -63,6 +63,10 @@ SIGNATURES = {
     "pq_silu_mul": (c_int, [c_void_p] * 3 + [c_int, c_int, c_int64, c_int, c_void_p]),
     "pq_linear_small_m": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "pq_validate_linear_small_m": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int]),
+    "pq_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
+                                   c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
+    "pq_validate_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
+                                            c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int]),
     "pq_stream_read": (c_size_t, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
     "pq_convert_codes6": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),

@@ -334,6 +334,35 @@ size_t pq_stream_read(const void* src, size_t bytes, int n_wavefronts, uint32_t*
     return per_wave * static_cast<size_t>(n_wavefronts);
 }
 
+int pq_validate_qkv_rope_append(const void* x, int64_t x_row_stride, const void* w_qkv, const void* bias, int M, int K,
+                                int dtype, const void* cos_table, const void* sin_table, int64_t table_rows,
+                                const int64_t* pos, const void* q_out, const void* k_dst, int64_t k_rows,
+                                const int64_t* k_row, const void* v_dst, int64_t v_rows, const int64_t* v_row, int N, int Nk) {
+    if (!x || !w_qkv || !cos_table || !sin_table || !pos || !q_out || !k_dst || !k_row || !v_dst || !v_row)
+        return PQ_ERR_NULL_POINTER;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (M < 1 || M > 8 || K < 64 || (K % 64) != 0 || N < 1 || Nk < 1 || N + 2 * Nk > 8191) return PQ_ERR_BAD_SHAPE;
+    if (x_row_stride < K || (x_row_stride % 8) != 0 || table_rows <= 0 || k_rows <= 0 || v_rows <= 0) return PQ_ERR_BAD_STRIDE;
+    if (!aligned(x, 16) || !aligned(w_qkv, 16) || !aligned(q_out, 8) || !aligned(k_dst, 8) || !aligned(v_dst, 8) ||
+        !aligned(cos_table, 2) || !aligned(sin_table, 2) || (bias && !aligned(bias, 2)) || !aligned(pos, 8) ||
+        !aligned(k_row, 8) || !aligned(v_row, 8))
+        return PQ_ERR_MISALIGNED;
+    return PQ_OK;
+}
+
+int pq_qkv_rope_append(const void* x, int64_t x_row_stride, const void* w_qkv, const void* bias, int M, int K, int dtype,
+                       const void* cos_table, const void* sin_table, int64_t table_rows, const int64_t* pos, void* q_out,
+                       void* k_dst, int64_t k_rows, const int64_t* k_row, void* v_dst, int64_t v_rows,
+                       const int64_t* v_row, int N, int Nk, void* stream) {
+    const int rc = pq_validate_qkv_rope_append(x, x_row_stride, w_qkv, bias, M, K, dtype, cos_table, sin_table, table_rows,
+                                               pos, q_out, k_dst, k_rows, k_row, v_dst, v_rows, v_row, N, Nk);
+    if (rc != PQ_OK) return rc;
+    const int err = pq::launch_qkv_rope_append(x, x_row_stride, w_qkv, bias, M, K, dtype, cos_table, sin_table, table_rows,
+                                               pos, q_out, k_dst, k_rows, k_row, v_dst, v_rows, v_row, N, Nk,
+                                               static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 // ---- 4-bit values (Mixed variant) ------------------------------------------------------------
 int pq_decode_attn_v4_plan(int B, int N, int Nk, int max_groups, int n_cus) {
     if (B <= 0 || Nk <= 0 || N <= 0 || max_groups <= 0) return 1;

@@ -34,6 +34,11 @@ int launch_small_m_linear(const void* x, int64_t x_stride, const void* w, const 
 
 int launch_stream_read(const void* src, size_t bytes_per_wave, int n_waves, uint32_t* sink, hipStream_t st);
 
+int launch_qkv_rope_append(const void* x, int64_t x_stride, const void* w, const void* bias, int M, int K, int dtype,
+                           const void* cos_tab, const void* sin_tab, int64_t max_pos, const int64_t* pos, void* q_out,
+                           void* k_dst, int64_t k_rows, const int64_t* k_row, void* v_dst, int64_t v_rows,
+                           const int64_t* v_row, int N, int Nk, hipStream_t st);
+
 struct AttnArgs {
     const void* q;
     const uint8_t* codes;

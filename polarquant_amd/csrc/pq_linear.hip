@@ -254,6 +254,169 @@ __global__ __launch_bounds__(kWave * KSPLIT) void small_m8_linear_kernel(
     }
 }
 
+// The fused q|k|v projection of a decode step with RoPE and the cache appends in its epilogue (M <= 8):
+// small_m8_linear_kernel's loop on the concatenated [(N + 2 Nk) * 128, K] weight, with the workgroup's two
+// 8-row tiles 64 rows apart instead of adjacent, i.e. dims d..d+7 and d+64..d+71 of one head: the two halves of
+// 8 rotation pairs.  The epilogue rounds both to the dtype (the projection's output), rotates q and k heads
+// exactly as rope_append_kernel does (every product and sum rounded to the dtype), and writes the query to
+// q_out [M, N, 128], the key to row *k_row of k_dst [M, Nk, k_rows, 128] and the value (unrotated) to row
+// *v_row of v_dst [M, Nk, v_rows, 128].  One launch instead of two, no [M, (N + 2 Nk) * 128] round trip.
+struct RopeAppendArgs {
+    const uint16_t* cos_tab;
+    const uint16_t* sin_tab;
+    const int64_t* pos;
+    uint16_t* q_out;
+    uint16_t* k_dst;
+    const int64_t* k_row;
+    uint16_t* v_dst;
+    const int64_t* v_row;
+    int64_t max_pos, k_rows, v_rows;
+    int N, Nk;
+};
+
+template <typename T, int KSPLIT, int kStage>
+__global__ __launch_bounds__(kWave * KSPLIT) void qkv_rope_append_kernel(
+    const uint16_t* __restrict__ x, int64_t x_stride, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
+    int M, int K, RopeAppendArgs ra) {
+    __shared__ float part[KSPLIT][2][4][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wv = threadIdx.x / kWave;
+    const int r = lane & 15, g = lane >> 4;
+    const int row = r & 7, chunk = (r >> 3) * 4 + g;
+    const int head = blockIdx.x >> 3, c8 = (blockIdx.x & 7) * 8;       // dims c8 .. c8+7 and 64 + c8 .. of this head
+    const int n0 = head * kHeadDim + c8;
+    const int klen = K / KSPLIT, steps = klen / 64;
+    const int m = row < M ? row : 0;
+    const size_t koff = static_cast<size_t>(wv) * klen + 8 * chunk;
+    const uint16_t* wp = w + static_cast<size_t>(n0 + row) * K + koff;
+    const uint16_t* xp = x + static_cast<size_t>(m) * x_stride + koff;
+    const size_t half_tile = static_cast<size_t>(kPairs) * K;           // rows n0 + 64 .. n0 + 71
+
+    floatx4_l acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    auto ldw = [](const uint16_t* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4_l*>(p)); };
+    auto load = [&](Stage8T<false, kStage>& st, int s0) {
+        static_for<kStage>([&](auto U) {
+            constexpr int u = decltype(U)::value;
+            st.w[0][u] = ldw(wp + (s0 + u) * 64);
+            st.w[1][u] = ldw(wp + half_tile + (s0 + u) * 64);
+            st.x[u] = *reinterpret_cast<const u32x4_l*>(xp + (s0 + u) * 64);
+        });
+    };
+    auto compute = [&](const Stage8T<false, kStage>& st) {
+        static_for<kStage>([&](auto U) {
+            constexpr int u = decltype(U)::value;
+            acc[0] = mfma32<T>(st.w[0][u], st.x[u], acc[0]);
+            acc[1] = mfma32<T>(st.w[1][u], st.x[u], acc[1]);
+        });
+    };
+    const int full = steps / kStage;
+    if (full > 0) {
+        Stage8T<false, kStage> sa, sb;
+        load(sa, 0);
+        int st = 0;
+        while (st + 2 < full) {
+            load(sb, (st + 1) * kStage);
+            compute(sa);
+            load(sa, (st + 2) * kStage);
+            compute(sb);
+            st += 2;
+        }
+        if (full - st == 2) {
+            load(sb, (st + 1) * kStage);
+            compute(sa);
+            compute(sb);
+        } else {
+            compute(sa);
+        }
+    }
+    for (int s1 = full * kStage; s1 < steps; s1++) {
+        const u32x4_l xv1 = *reinterpret_cast<const u32x4_l*>(xp + s1 * 64);
+        acc[0] = mfma32<T>(ldw(wp + s1 * 64), xv1, acc[0]);
+        acc[1] = mfma32<T>(ldw(wp + half_tile + s1 * 64), xv1, acc[1]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        part[wv][0][i][lane] = acc[0][i];
+        part[wv][1][i][lane] = acc[1][i];
+    }
+    __syncthreads();
+    if (wv != 0 || r >= 8 || r >= M || g >= 2) return;
+    // lane (r, g): batch row r, dims d = c8 + 4g + i (first half) and d + 64 (second half), i < 4
+    const int N = ra.N, Nk = ra.Nk;
+    const bool is_q = head < N, is_k = !is_q && head < N + Nk;
+    int64_t p = *ra.pos;
+    p = p < 0 ? 0 : (p >= ra.max_pos ? ra.max_pos - 1 : p);
+    uint16_t o1[4], o2[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KSPLIT; k++) {
+            s1 += part[k][0][i][lane] + part[k][0][i][lane + 40];
+            s2 += part[k][1][i][lane] + part[k][1][i][lane + 40];
+        }
+        const int d = c8 + 4 * g + i;
+        if (bias) { s1 += lo2f<T>(bias[n0 + 4 * g + i]); s2 += lo2f<T>(bias[n0 + kPairs + 4 * g + i]); }
+        const float x1 = rnd_l<T>(s1), x2 = rnd_l<T>(s2);           // the projection's output in the dtype
+        if (is_q || is_k) {
+            const float c1 = lo2f<T>(ra.cos_tab[p * kHeadDim + d]), c2 = lo2f<T>(ra.cos_tab[p * kHeadDim + kPairs + d]);
+            const float n1 = lo2f<T>(ra.sin_tab[p * kHeadDim + d]), n2 = lo2f<T>(ra.sin_tab[p * kHeadDim + kPairs + d]);
+            // (x * cos) + (rotate_half(x) * sin), rotate_half(x) = cat(-x2, x1)
+            o1[i] = f2lo<T>(rnd_l<T>(x1 * c1) + rnd_l<T>(-x2 * n1));
+            o2[i] = f2lo<T>(rnd_l<T>(x2 * c2) + rnd_l<T>(x1 * n2));
+        } else {
+            o1[i] = f2lo<T>(x1);
+            o2[i] = f2lo<T>(x2);
+        }
+    }
+    uint16_t* dst;
+    if (is_q) {
+        dst = ra.q_out + (static_cast<size_t>(r) * N + head) * kHeadDim;
+    } else if (is_k) {
+        int64_t kr = *ra.k_row;
+        kr = kr < 0 ? 0 : (kr >= ra.k_rows ? ra.k_rows - 1 : kr);
+        dst = ra.k_dst + ((static_cast<size_t>(r) * Nk + (head - N)) * ra.k_rows + kr) * kHeadDim;
+    } else {
+        int64_t vr = *ra.v_row;
+        vr = vr < 0 ? 0 : (vr >= ra.v_rows ? ra.v_rows - 1 : vr);
+        dst = ra.v_dst + ((static_cast<size_t>(r) * Nk + (head - N - Nk)) * ra.v_rows + vr) * kHeadDim;
+    }
+    dst += c8 + 4 * g;
+    *reinterpret_cast<uint2*>(dst) = make_uint2(static_cast<uint32_t>(o1[0]) | (static_cast<uint32_t>(o1[1]) << 16),
+                                                static_cast<uint32_t>(o1[2]) | (static_cast<uint32_t>(o1[3]) << 16));
+    *reinterpret_cast<uint2*>(dst + kPairs) = make_uint2(static_cast<uint32_t>(o2[0]) | (static_cast<uint32_t>(o2[1]) << 16),
+                                                         static_cast<uint32_t>(o2[2]) | (static_cast<uint32_t>(o2[3]) << 16));
+}
+
+int launch_qkv_rope_append(const void* x, int64_t x_stride, const void* w, const void* bias, int M, int K, int dtype,
+                           const void* cos_tab, const void* sin_tab, int64_t max_pos, const int64_t* pos, void* q_out,
+                           void* k_dst, int64_t k_rows, const int64_t* k_row, void* v_dst, int64_t v_rows,
+                           const int64_t* v_row, int N, int Nk, hipStream_t st) {
+    RopeAppendArgs ra;
+    ra.cos_tab = static_cast<const uint16_t*>(cos_tab); ra.sin_tab = static_cast<const uint16_t*>(sin_tab);
+    ra.pos = pos; ra.q_out = static_cast<uint16_t*>(q_out); ra.k_dst = static_cast<uint16_t*>(k_dst); ra.k_row = k_row;
+    ra.v_dst = static_cast<uint16_t*>(v_dst); ra.v_row = v_row; ra.max_pos = max_pos; ra.k_rows = k_rows; ra.v_rows = v_rows;
+    ra.N = N; ra.Nk = Nk;
+    // the split of K, and with it the order of the partial sums, is launch_small_m_linear's for M <= 8
+    int ks = K >= 8192 ? 8 : 4;
+    while (ks > 1 && (K % (64 * ks)) != 0) ks >>= 1;
+    dim3 grid((N + 2 * Nk) * 8), block(kWave * ks);
+#define PQ_LAUNCH_R(T, KS, S)                                                                                        \
+    hipLaunchKernelGGL((qkv_rope_append_kernel<T, KS, S>), grid, block, 0, st, (const uint16_t*)x, x_stride,        \
+                       (const uint16_t*)w, (const uint16_t*)bias, M, K, ra)
+#define PQ_LAUNCH_RK(T)                                                                                              \
+    do {                                                                                                             \
+        if (ks == 8) PQ_LAUNCH_R(T, 8, 2);                                                                           \
+        else if (ks == 4) PQ_LAUNCH_R(T, 4, 1);                                                                      \
+        else if (ks == 2) PQ_LAUNCH_R(T, 2, 1);                                                                      \
+        else PQ_LAUNCH_R(T, 1, 1);                                                                                   \
+    } while (0)
+    if (dtype == 0) PQ_LAUNCH_RK(F16);
+    else PQ_LAUNCH_RK(BF16);
+#undef PQ_LAUNCH_RK
+#undef PQ_LAUNCH_R
+    return static_cast<int>(hipGetLastError());
+}
+
 // Launch shapes measured at the decode shapes of Llama-3-8B (K-split 4 / 8 / 16 and stages of 1 / 2 / 4 / 8
 // loads were swept): the 16-row kernel runs four wavefronts per workgroup with stages of 4 (2 when gated); the
 // M <= 8 kernel four wavefronts with stages of 1, or eight with stages of 2 when K >= 8192 (down_proj).

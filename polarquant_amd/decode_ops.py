@@ -109,3 +109,30 @@ def linear_small_m(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
                                           _dtype_code(x), _stream_ptr(x.device))
     _ffi.check(rc, "pq_linear_small_m")
     return y
+
+
+def qkv_rope_append(x: torch.Tensor, w_qkv: torch.Tensor, b_qkv: Optional[torch.Tensor], cos_table: torch.Tensor,
+                    sin_table: torch.Tensor, pos: torch.Tensor, k_dst: torch.Tensor, k_row: torch.Tensor,
+                    v_dst: torch.Tensor, v_row: torch.Tensor, n_heads: int, n_kv_heads: int) -> torch.Tensor:
+    """`linear_small_m(x, w_qkv, b_qkv)` followed by `rope_append(...)` in one launch, bit-identical to the pair:
+    x [B <= 8, 1, K]; w_qkv [(N + 2 Nk) * 128, K] (q, k, v heads in that order); returns the rotated query
+    [B, N, 1, 128], writes the rotated key into k_dst[:, :, k_row] and the value into v_dst[:, :, v_row]."""
+    _gpu(x)
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    B = x2.shape[0]
+    assert w_qkv.is_contiguous() and w_qkv.shape == ((n_heads + 2 * n_kv_heads) * 128, K) and w_qkv.dtype == x.dtype
+    assert x2.stride(1) == 1 and (b_qkv is None or (b_qkv.is_contiguous() and b_qkv.numel() == w_qkv.shape[0] and b_qkv.dtype == x.dtype))
+    assert k_dst.is_contiguous() and v_dst.is_contiguous() and cos_table.is_contiguous() and sin_table.is_contiguous()
+    assert pos.dtype == k_row.dtype == v_row.dtype == torch.int64
+    assert k_dst.shape[:2] == (B, n_kv_heads) == v_dst.shape[:2] and k_dst.shape[3] == 128 == v_dst.shape[3]
+    q_out = torch.empty((B, n_heads, 1, 128), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _ffi.lib().pq_qkv_rope_append(x2.data_ptr(), x2.stride(0) if B > 1 else K, w_qkv.data_ptr(),
+                                           None if b_qkv is None else b_qkv.data_ptr(), B, K, _dtype_code(x),
+                                           cos_table.data_ptr(), sin_table.data_ptr(), cos_table.shape[0], pos.data_ptr(),
+                                           q_out.data_ptr(), k_dst.data_ptr(), k_dst.shape[2], k_row.data_ptr(),
+                                           v_dst.data_ptr(), v_dst.shape[2], v_row.data_ptr(), n_heads, n_kv_heads,
+                                           _stream_ptr(x.device))
+    _ffi.check(rc, "pq_qkv_rope_append")
+    return q_out

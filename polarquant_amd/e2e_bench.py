@@ -48,6 +48,7 @@ def main():
     ap.add_argument("--graph", action="store_true")
     ap.add_argument("--values4", action="store_true", help="4-bit values as well (the reference's Mixed variant)")
     ap.add_argument("--fused-prefill", action="store_true", help="with --graph: fused norm / SiLU kernels in the prompt pass too")
+    ap.add_argument("--separate-rope", action="store_true", help="with --graph: q|k|v projection and RoPE + append as two launches")
     args = ap.parse_args()
     dev = torch.device("cuda:0")
     cfg = PolarConfig.llama3_8b(num_hidden_layers=args.layers, cache_capacity=args.prompt + args.new + 128,
@@ -59,7 +60,8 @@ def main():
     with torch.no_grad():
         if args.graph:
             from .graph_decode import PolarGraphDecoder
-            dec = PolarGraphDecoder(model, max_len=args.prompt + args.new + 128, fused_prefill=args.fused_prefill)
+            dec = PolarGraphDecoder(model, max_len=args.prompt + args.new + 128, fused_prefill=args.fused_prefill,
+                                    fused_qkv_rope=not args.separate_rope)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             logits = dec.prefill(ids)

@@ -29,19 +29,22 @@ from .modeling_common import GROUP, apply_rotary_pos_emb
 
 class PolarGraphDecoder:
     def __init__(self, model, max_len: int, use_graph: bool = True, fused_ops: bool = True, small_m_gemm: bool = True,
-                 fused_prefill: bool = False):
+                 fused_prefill: bool = False, fused_qkv_rope: bool = True):
         """fused_ops: run RoPE + cache append, the norms and the MLP activation as one HIP launch each
         (polarquant_amd.decode_ops) instead of the eager modules' chains of elementwise launches.  The
         rotation is bit-identical to the eager ops; the norms and SiLU agree to the dtype's last bit.
         small_m_gemm (with fused_ops, batch <= 16): o_proj, gate/up (with the SiLU product in its epilogue) and
         down_proj through the weight-streaming kernel `decode_ops.linear_small_m` instead of the BLAS library;
         fp32 accumulation in a different order, so logits agree to rounding.
+        fused_qkv_rope (with small_m_gemm, batch <= 8): the q|k|v projection, the rotation and the two cache
+        appends as one launch, `decode_ops.qkv_rope_append`, bit-identical to the projection followed by the rotation.
         fused_prefill: the prompt pass runs the norms and the MLP activation through the same fused kernels
         instead of the eager modules' elementwise chains (about a sixth of the prompt time); the cache it
         builds and the logits then agree with the eager model to rounding instead of bit for bit."""
         self.fused_ops = fused_ops
         self.small_m_gemm = small_m_gemm
         self.fused_prefill = fused_prefill
+        self.fused_qkv_rope = fused_qkv_rope
         self.model = model
         self.cfg = model.config
         self.max_len = int(max_len)
@@ -168,7 +171,7 @@ class PolarGraphDecoder:
     def _step_body_fused(self):
         """The decode step with one launch per elementwise stage: 2 norms (each with the residual add
         folded in), RoPE + append, SiLU * up, plus the GEMMs and the attention, per layer."""
-        from .decode_ops import linear_small_m, rmsnorm, rope_append, silu_mul
+        from .decode_ops import linear_small_m, qkv_rope_append, rmsnorm, rope_append, silu_mul
         model, B = self.model, self.B
         layers = model.model.layers
         x = model.model.embed_tokens(self.ids).contiguous()                 # residual stream [B,1,H], updated in place
@@ -179,14 +182,19 @@ class PolarGraphDecoder:
             own = self.small_m_gemm and B <= 16 and all(
                 w_.is_contiguous() and w_.shape[0] % 16 == 0 and w_.shape[1] % 32 == 0
                 for w_ in (att._wqkv, att.o_proj.weight, mlp.gate_proj.weight, mlp.up_proj.weight, mlp.down_proj.weight))
-            if own:
-                qkv = linear_small_m(h, att._wqkv, att._bqkv)                   # [B,1,(N+2Nk)*128]
-            else:
-                qkv = torch.nn.functional.linear(h, att._wqkv, att._bqkv)
-            q_lin, k_lin, v_lin = qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:]
             v_dst, v_row = (ar.vres, self.resid_idx) if self.mixed else (ar.v, self.pos)
-            q = rope_append(q_lin, k_lin, v_lin, self.cos_table, self.sin_table, self.pos, ar.kres, self.resid_idx,
-                            v_dst, v_row, att.num_heads, att.num_key_value_heads)
+            if own and self.fused_qkv_rope and B <= 8 and att._wqkv.shape[1] % 64 == 0:
+                # projection, rotation and both appends in one launch (bit-identical to the two below)
+                q = qkv_rope_append(h, att._wqkv, att._bqkv, self.cos_table, self.sin_table, self.pos, ar.kres,
+                                    self.resid_idx, v_dst, v_row, att.num_heads, att.num_key_value_heads)
+            else:
+                if own:
+                    qkv = linear_small_m(h, att._wqkv, att._bqkv)               # [B,1,(N+2Nk)*128]
+                else:
+                    qkv = torch.nn.functional.linear(h, att._wqkv, att._bqkv)
+                q_lin, k_lin, v_lin = qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:]
+                q = rope_append(q_lin, k_lin, v_lin, self.cos_table, self.sin_table, self.pos, ar.kres, self.resid_idx,
+                                v_dst, v_row, att.num_heads, att.num_key_value_heads)
             o = self._attend(att, ar, q)
             pn = layer.post_attention_layernorm
             if own and mlp.gate_proj.bias is None and mlp.up_proj.bias is None:

@@ -215,6 +215,24 @@ def test_linear_small_m_rejects_bad_arguments(lib):
     assert lib.pq_linear_small_m(None, 4096, P, None, None, P, 4096, 8, 4096, 4096, 1, None) == -1
 
 
+def test_qkv_rope_append_rejects_bad_arguments(lib):
+    #     x  stride  w  bias  M  K     dt cos sin rows pos q  k  krows krow v  vrows vrow N   Nk
+    ok = [P, 4096, P, None, 8, 4096, 0, P, P, 4096, P, P, P, 128, P, P, 4096, P, 32, 8]
+    assert lib.pq_validate_qkv_rope_append(*ok) == 0
+    def bad(i, v):
+        a = list(ok)
+        a[i] = v
+        return lib.pq_validate_qkv_rope_append(*a)
+    for i in (0, 2, 7, 8, 10, 11, 12, 14, 15, 17):
+        assert bad(i, None) == -1, i
+    assert bad(6, 3) == -4
+    assert bad(4, 0) == -2 and bad(4, 9) == -2 and bad(5, 4128) == -2 and bad(5, 0) == -2     # rows, K % 64
+    assert bad(18, 0) == -2 and bad(19, 0) == -2
+    assert bad(1, 4000) == -6 and bad(1, 4100) == -6 and bad(9, 0) == -6 and bad(13, 0) == -6 and bad(16, -1) == -6
+    assert bad(0, P + 8) == -5 and bad(2, P + 2) == -5 and bad(11, P + 4) == -5 and bad(10, P + 4) == -5 and bad(3, P + 1) == -5
+    assert lib.pq_qkv_rope_append(*(ok[:2] + [None] + ok[3:] + [None])) == -1
+
+
 def test_stream_read_rejects_bad_arguments(lib):
     assert lib.pq_stream_read(None, 1 << 30, 1024, P, None) == 0 and lib.pq_stream_read(P, 1 << 30, 1024, None, None) == 0
     assert lib.pq_stream_read(P, 1 << 30, 0, P, None) == 0 and lib.pq_stream_read(P + 8, 1 << 30, 1024, P, None) == 0

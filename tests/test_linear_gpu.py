@@ -73,3 +73,39 @@ def test_linear_rejects_what_the_kernel_does_not_cover(gpu):
         linear_small_m(x[:4], w[:24].contiguous())              # N not a multiple of 16
     with pytest.raises(RuntimeError):
         linear_small_m(x[:4].cpu(), w.cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,N,Nk,K,bias", [(8, 32, 8, 4096, False), (3, 4, 2, 512, True), (1, 7, 1, 896, True),
+                                            (5, 8, 8, 8192, False), (8, 2, 1, 192, False)])
+def test_qkv_rope_append_equals_projection_then_rotation(gpu, dtype, B, N, Nk, K, bias):
+    """One launch against the two it replaces: the rotated query, the key row and the value row are the same bits;
+    rows of the caches other than the written ones are untouched."""
+    from polarquant_amd.decode_ops import linear_small_m, qkv_rope_append, rope_append
+    g = torch.Generator().manual_seed(B * 1000 + N + K)
+    x = torch.randn(B, 1, K, generator=g).to(dtype).to(gpu)
+    w = (torch.randn((N + 2 * Nk) * 128, K, generator=g) / K ** 0.5).to(dtype).to(gpu)
+    b = torch.randn((N + 2 * Nk) * 128, generator=g).to(dtype).to(gpu) if bias else None
+    max_pos, k_rows, v_rows = 300, 128, 300
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * (1e4 ** (-torch.arange(0, 128, 2).float() / 128))[None]
+    emb = torch.cat([ang, ang], -1)
+    cos, sin = emb.cos().to(dtype).to(gpu), emb.sin().to(dtype).to(gpu)
+    pos = torch.tensor([257], device=gpu)
+    k_row = torch.tensor([77], device=gpu)
+    fill = torch.randn(B, Nk, k_rows, 128, generator=g).to(dtype).to(gpu)
+    fillv = torch.randn(B, Nk, v_rows, 128, generator=g).to(dtype).to(gpu)
+    k1, v1, k2, v2 = fill.clone(), fillv.clone(), fill.clone(), fillv.clone()
+    qkv = linear_small_m(x, w, b)
+    nq, nkv = N * 128, Nk * 128
+    q_ref = rope_append(qkv[..., :nq], qkv[..., nq:nq + nkv], qkv[..., nq + nkv:], cos, sin, pos, k1, k_row, v1, pos, N, Nk)
+    q_got = qkv_rope_append(x, w, b, cos, sin, pos, k2, k_row, v2, pos, N, Nk)
+    torch.cuda.synchronize()
+    assert q_got.shape == q_ref.shape and torch.equal(q_got, q_ref)
+    assert torch.equal(k2, k1) and torch.equal(v2, v1)
+    assert not torch.equal(k2[:, :, 77], fill[:, :, 77]) and torch.equal(k2[:, :, :77], fill[:, :, :77])
+    # a strided x (rows of a wider tensor)
+    wide = torch.zeros(B, 1, K + 64, dtype=dtype, device=gpu)
+    wide[..., :K] = x
+    k3, v3 = fill.clone(), fillv.clone()
+    assert torch.equal(qkv_rope_append(wide[..., :K], w, b, cos, sin, pos, k3, k_row, v3, pos, N, Nk), q_ref)
+    assert torch.equal(k3, k1) and torch.equal(v3, v1)
