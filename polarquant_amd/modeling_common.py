@@ -736,10 +736,13 @@ class GenerationConfig:
     temperature: float = 1.0
 
 
-def generate(model, input_ids, attention_mask, generation_config, do_sample=False, max_new_tokens=8):
+def generate(model, input_ids, attention_mask, generation_config, do_sample=False, max_new_tokens=8, graph_decoder=False):
     """The reference's decoding loop (models/modeling_llama_polar.py:622-666): prefill, then one token per step,
     the mask grown by a column of ones; stops early once every sequence has produced a stop token (sequences that
-    stopped earlier keep producing tokens until then, as in the reference).  -> LongTensor [B, <= max_new_tokens]."""
+    stopped earlier keep producing tokens until then, as in the reference).  -> LongTensor [B, <= max_new_tokens].
+    graph_decoder (not in the reference): the steps after the prompt replay a captured HIP graph on static state
+    (`graph_decode.PolarGraphDecoder`) instead of driving the modules launch by launch; logits agree with the
+    eager step to rounding, so a near-tie between two tokens may resolve differently."""
     dev = model.device
     n_seq = input_ids.size(0)
     stop_ids = generation_config.eos_token_id
@@ -747,14 +750,21 @@ def generate(model, input_ids, attention_mask, generation_config, do_sample=Fals
     produced = torch.zeros((n_seq, max_new_tokens), dtype=torch.long, device=dev)
     finished = torch.zeros((n_seq, 1), dtype=torch.bool, device=dev)
     tokens, cache, n_out = input_ids, None, 0
+    decoder = None
+    if graph_decoder:
+        from .graph_decode import PolarGraphDecoder
+        decoder = PolarGraphDecoder(model, max_len=input_ids.size(1) + max_new_tokens + 1)
     with torch.no_grad():
         while n_out < max_new_tokens:
-            step_out = model(input_ids=tokens, attention_mask=attention_mask, past_key_values=cache, num_logits_to_keep=1)
-            cache = step_out.past_key_values
-            tokens = sample(step_out.logits, generation_config, do_sample=do_sample)
+            if decoder is None:
+                step_out = model(input_ids=tokens, attention_mask=attention_mask, past_key_values=cache, num_logits_to_keep=1)
+                cache, logits = step_out.past_key_values, step_out.logits
+            else:
+                logits = decoder.prefill(tokens, attention_mask) if n_out == 0 else decoder.step(tokens)
+            tokens = sample(logits, generation_config, do_sample=do_sample)
             produced[:, n_out:n_out + 1] = tokens
             n_out += 1
-            if attention_mask is not None:
+            if attention_mask is not None and decoder is None:
                 attention_mask = torch.cat([attention_mask, torch.ones_like(tokens)], dim=-1)
             finished |= torch.isin(tokens, stop_ids)
             if bool(finished.all()):

@@ -152,6 +152,50 @@ def test_silu_mul_splits_more_rows_than_one_launch_takes(gpu):
     assert torch.equal(y[65535:], silu_mul(gate[65535:].contiguous(), up[65535:].contiguous()))
 
 
+def test_generate_with_the_graph_decoder(gpu):
+    """`generate(..., graph_decoder=True)`: the reference's loop with the steps replayed from the graph.  Same tokens
+    as driving the decoder by hand; against the eager loop the tokens agree until a near-tie (checked: every token
+    picked is within rounding of the eager model's best at that step); stops when every sequence has hit a stop id."""
+    from polarquant_amd.modeling_common import GenerationConfig, generate
+    torch.manual_seed(31)
+    cfg = _tiny()
+    model = LlamaPolarForCausalLM(cfg).half().to(gpu).eval()
+    B, L, new = 2, 125, 12                         # flush at 128 tokens
+    ids = torch.randint(0, cfg.vocab_size, (B, L), device=gpu)
+    mask = torch.ones(B, L, dtype=torch.int64, device=gpu)
+    mask[1, :9] = 0
+    gc = GenerationConfig(eos_token_id=[999999])
+    got = generate(model, ids, mask, gc, max_new_tokens=new, graph_decoder=True)
+    assert got.shape == (B, new)
+    dec = PolarGraphDecoder(model, max_len=L + new + 1)
+    with torch.no_grad():
+        tok = dec.prefill(ids, mask).argmax(-1)
+        by_hand = [tok]
+        for _ in range(new - 1):
+            tok = dec.step(tok).argmax(-1)
+            by_hand.append(tok)
+    assert torch.equal(got, torch.cat(by_hand, dim=-1))
+    # the eager model, fed the graph decoder's tokens, would have picked (nearly) the same at every step
+    with torch.no_grad():
+        m, cache, tok = mask, None, ids
+        for s in range(new):
+            out = model(input_ids=tok, attention_mask=m, past_key_values=cache, num_logits_to_keep=1)
+            cache, rl = out.past_key_values, out.logits.float()
+            tok = got[:, s:s + 1]
+            pick = rl.gather(-1, tok.unsqueeze(-1)).squeeze(-1)
+            assert bool((rl.max(-1).values - pick <= 4e-2 * max(1.0, rl.abs().max().item())).all()), s
+            m = torch.cat([m, torch.ones_like(tok)], dim=-1)
+    # stop ids: every sequence's first token is a stop id -> one token comes back
+    first = got[:, 0].tolist()
+    short = generate(model, ids, mask, GenerationConfig(eos_token_id=first), max_new_tokens=new, graph_decoder=True)
+    assert short.shape == (B, 1) and torch.equal(short, got[:, :1])
+    # sampling draws from the same filtered distribution: valid ids, right shape
+    torch.manual_seed(5)
+    smp = generate(model, ids, None, GenerationConfig(eos_token_id=[999999], top_k=5), do_sample=True, max_new_tokens=4,
+                   graph_decoder=True)
+    assert smp.shape == (B, 4) and int(smp.min()) >= 0 and int(smp.max()) < cfg.vocab_size
+
+
 def test_graph_decoder_rejects_overflow(gpu):
     torch.manual_seed(12)
     cfg = _tiny(layers=1)
