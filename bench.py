@@ -213,6 +213,20 @@ def main():
         s_ms = time_events(stream_once, 20, 4)
         stream_gbps = max(stream_gbps, got[0] / (s_ms * 1e-3) / 1e9)
 
+    # the attention kernel's own HBM reads without its arithmetic: same grid, loads, order and prefetch depth
+    n_tok = w["n_groups"] * 128
+    replica = [0]
+
+    def replica_once():
+        x = sets[turn[0] & 1]
+        turn[0] += 1
+        replica[0] = lib.pq_attn_load_replica(x["codes"].data_ptr(), x["v"].data_ptr(), B * Nk, x["codes"].shape[2] * 128,
+                                              x["v"].shape[2], n_tok, n_splits, sink.data_ptr(), _stream_ptr(dev))
+        assert replica[0] > 0
+    replica_once()
+    replica_once()
+    r_ms = kernel_duration_ms(replica_once, 20)
+
     alg_bytes = wl.algorithmic_bytes(Nk, N, [w["n_groups"] * 128] * B, [w["n_resid"]] * B, sh.rbits, sh.tbits)
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     result = {
@@ -230,7 +244,9 @@ def main():
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES,
                      "plain_stream_read_gbps": round(stream_gbps, 1),
-                     "frac_of_plain_stream_read": round(achieved / stream_gbps, 4)},
+                     "frac_of_plain_stream_read": round(achieved / stream_gbps, 4),
+                     "load_only_replica_us": round(r_ms * 1e3, 2),
+                     "load_only_replica_gbps": round(replica[0] / (r_ms * 1e-3) / 1e9, 1)},
     }
     # the same step with the values of the quantized groups in 4 bits (the reference's Mixed variant)
     if not args.no_values4:

@@ -103,6 +103,16 @@ int pq_validate_qkv_rope_append(const void *x, int64_t x_row_stride, const void 
  * `sink`: 4 writable bytes on the device (practically never written). */
 size_t pq_stream_read(const void *src, size_t bytes, int n_wavefronts, uint32_t *sink, void *stream);
 
+/* Measurement aid (no reference counterpart): the HBM reads of pq_decode_attn's main kernel (byte-per-code
+ * rows, half-precision values) without its arithmetic: `planes` (batch x KV head) planes of `tokens` tokens,
+ * each cut into `n_slices` slices read by one wavefront with the kernel's own loads, order and prefetch depth.
+ * codes: `planes` planes of `code_plane_tokens` 64-byte rows; v: `planes` planes of `v_plane_tokens`
+ * 256-byte rows.  Returns the bytes one launch reads (320 per token; slices are whole multiples of 128
+ * tokens), 0 on a bad argument or a failed launch.  Time it beside the kernel: the difference is what the
+ * kernel's table, score and softmax work costs on top of its memory access. */
+size_t pq_attn_load_replica(const uint8_t *codes, const void *v, int planes, int64_t code_plane_tokens,
+                            int64_t v_plane_tokens, int64_t tokens, int n_slices, uint32_t *sink, void *stream);
+
 /* Layout converter for code rows: pack != 0 turns `n_rows` byte-per-code rows (64 bytes each, every
  * code < 64) into packed 6-bit rows (48 bytes each), pack == 0 the reverse.  For caches built by the
  * reference (always byte-per-code) that are to be kept packed, and back.  No reference counterpart. */

@@ -68,6 +68,7 @@ SIGNATURES = {
     "pq_validate_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int]),
     "pq_stream_read": (c_size_t, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
+    "pq_attn_load_replica": (c_size_t, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
     "pq_convert_codes6": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),
     "pq_decode_attn_v4_plan": (c_int, [c_int] * 5),

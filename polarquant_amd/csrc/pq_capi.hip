@@ -334,6 +334,21 @@ size_t pq_stream_read(const void* src, size_t bytes, int n_wavefronts, uint32_t*
     return per_wave * static_cast<size_t>(n_wavefronts);
 }
 
+size_t pq_attn_load_replica(const uint8_t* codes, const void* v, int planes, int64_t code_plane_tokens,
+                            int64_t v_plane_tokens, int64_t tokens, int n_slices, uint32_t* sink, void* stream) {
+    if (!codes || !v || !sink || !aligned(codes, 16) || !aligned(v, 16) || !aligned(sink, 4)) return 0;
+    if (planes <= 0 || n_slices <= 0 || static_cast<long long>(planes) * n_slices > (1ll << 24)) return 0;
+    if (tokens <= 0 || tokens > code_plane_tokens || tokens > v_plane_tokens) return 0;
+    if (v_plane_tokens > ((int64_t{1} << 31) - 1) / 256 || code_plane_tokens > ((int64_t{1} << 31) - 1) / 64) return 0;
+    const int64_t per_slice = tokens / n_slices / 128 * 128;          // whole pairs of 64-token tiles
+    if (per_slice == 0) return 0;
+    if (pq::launch_attn_load_replica(codes, v, planes, static_cast<uint32_t>(code_plane_tokens),
+                                     static_cast<uint32_t>(v_plane_tokens), static_cast<uint32_t>(per_slice), n_slices, sink,
+                                     static_cast<hipStream_t>(stream)) != 0)
+        return 0;
+    return static_cast<size_t>(per_slice) * n_slices * static_cast<size_t>(planes) * 320;
+}
+
 int pq_validate_qkv_rope_append(const void* x, int64_t x_row_stride, const void* w_qkv, const void* bias, int M, int K,
                                 int dtype, const void* cos_table, const void* sin_table, int64_t table_rows,
                                 const int64_t* pos, const void* q_out, const void* k_dst, int64_t k_rows,

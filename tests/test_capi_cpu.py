@@ -239,6 +239,19 @@ def test_stream_read_rejects_bad_arguments(lib):
     assert lib.pq_stream_read(P, 1000, 1024, P, None) == 0          # less than one 16 KiB trip per wavefront
 
 
+def test_attn_load_replica_rejects_bad_arguments(lib):
+    ok = [P, P, 128, 32768, 32769, 32768, 8, P]
+    def bad(i, v):
+        a = list(ok)
+        a[i] = v
+        return lib.pq_attn_load_replica(*a, None)
+    assert bad(0, None) == 0 and bad(1, None) == 0 and bad(7, None) == 0 and bad(0, P + 8) == 0
+    assert bad(2, 0) == 0 and bad(6, 0) == 0 and bad(5, 0) == 0
+    assert bad(5, 40000) == 0                       # more tokens than a plane holds
+    assert bad(4, 1 << 24) == 0 and bad(3, 1 << 26) == 0   # a plane a 32-bit byte offset cannot span
+    assert bad(6, 512) == 0                         # slices shorter than two tiles
+
+
 def test_convert_codes6_rejects_bad_arguments(lib):
     assert lib.pq_convert_codes6(None, P, 4, 1, None) == -1 and lib.pq_convert_codes6(P, None, 4, 0, None) == -1
     assert lib.pq_convert_codes6(P, P, 0, 1, None) == -2

@@ -94,3 +94,22 @@ def test_silu_mul_matches_eager(gpu, dtype):
     # the two halves of one fused gate|up projection output
     gu = torch.cat([g, u], dim=-1)
     assert torch.equal(silu_mul(gu[..., :14336], gu[..., 14336:]), got)
+
+
+def test_measurement_aids_launch_and_report_their_bytes(gpu):
+    """pq_stream_read and pq_attn_load_replica read what they say (whole 16 KiB trips / whole pairs of tiles) and
+    leave their inputs and the sink alone."""
+    from polarquant_amd import _ffi
+    from polarquant_amd.kernel4group import _stream_ptr
+    lib = _ffi.lib()
+    planes, tokens = 6, 1000
+    codes = torch.randint(0, 255, (planes, 1024, 64), dtype=torch.uint8, device=gpu)
+    v = torch.randn(planes, tokens + 5, 128, device=gpu).half()
+    before = (codes.clone(), v.clone())
+    sink = torch.zeros(1, dtype=torch.int32, device=gpu)
+    got = lib.pq_attn_load_replica(codes.data_ptr(), v.data_ptr(), planes, 1024, tokens + 5, tokens, 3, sink.data_ptr(), _stream_ptr(gpu))
+    assert got == planes * 3 * 256 * 320            # 1000 // 3 = 333 tokens -> 256 per slice
+    got = lib.pq_stream_read(v.data_ptr(), v.numel() * 2, 7, sink.data_ptr(), _stream_ptr(gpu))
+    assert got == 7 * (v.numel() * 2 // 7 // 16384 * 16384)
+    torch.cuda.synchronize()
+    assert torch.equal(codes, before[0]) and torch.equal(v, before[1]) and int(sink) == 0
