@@ -316,6 +316,17 @@ int pq_decode_attn_v4(const void *q,
                       int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
                       void *out, unsigned flags, void *stream);
 
+/* RoPE over whole sequences, the prompt pass's `apply_rotary_pos_emb(query_states, key_states, cos, sin)`
+ * (models/modeling_llama_polar.py:56-59) in one launch, bit-identical to the eager
+ * (x * cos) + (rotate_half(x) * sin) in the model dtype.  q_lin / k_lin: outputs of q_proj / k_proj, token
+ * t = b * L + l at element offset t * token_stride (0 = dense, N * 128 resp. Nk * 128; multiples of 8);
+ * cos_rows / sin_rows [1 or B, L, 128] in the dtype, batch b at b * cos_sin_batch_stride (0 when shared);
+ * q_out [B, L, N, 128], k_out [B, L, Nk, 128] contiguous (read them as [B, heads, L, 128] by a transposed view,
+ * as the reference's .view().transpose(1, 2) does). */
+int pq_rope_qk(const void *q_lin, int64_t q_token_stride, const void *k_lin, int64_t k_token_stride, const void *cos_rows,
+               const void *sin_rows, int64_t cos_sin_batch_stride, void *q_out, void *k_out, int B, int L, int N, int Nk,
+               int dtype, void *stream);
+
 /* ---------------------------------------------------------------------------
  * A — the elementwise steps around the attention call of one decode step, each a
  * chain of 8-12 eager launches on a [B,1,hidden] activation in the reference.

@@ -63,6 +63,8 @@ SIGNATURES = {
     "pq_silu_mul": (c_int, [c_void_p] * 3 + [c_int, c_int, c_int64, c_int, c_void_p]),
     "pq_linear_small_m": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "pq_validate_linear_small_m": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int]),
+    "pq_rope_qk": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+                           c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "pq_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "pq_validate_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,

@@ -271,6 +271,27 @@ int pq_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, cons
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
+int pq_rope_qk(const void* q_lin, int64_t q_token_stride, const void* k_lin, int64_t k_token_stride, const void* cos_rows,
+               const void* sin_rows, int64_t cos_sin_batch_stride, void* q_out, void* k_out, int B, int L, int N, int Nk,
+               int dtype, void* stream) {
+    if (!q_lin || !k_lin || !cos_rows || !sin_rows || !q_out || !k_out) return PQ_ERR_NULL_POINTER;
+    if (B <= 0 || L <= 0 || N <= 0 || Nk <= 0 || static_cast<long long>(B) * L > 0x7fffffffll || N + Nk > 4096)
+        return PQ_ERR_BAD_SHAPE;
+    if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
+    if (q_token_stride == 0) q_token_stride = static_cast<int64_t>(N) * PQ_HEAD_DIM;      // dense
+    if (k_token_stride == 0) k_token_stride = static_cast<int64_t>(Nk) * PQ_HEAD_DIM;
+    if (q_token_stride < static_cast<int64_t>(N) * PQ_HEAD_DIM || k_token_stride < static_cast<int64_t>(Nk) * PQ_HEAD_DIM ||
+        (q_token_stride % 8) != 0 || (k_token_stride % 8) != 0 ||
+        (cos_sin_batch_stride != 0 && (cos_sin_batch_stride < static_cast<int64_t>(L) * PQ_HEAD_DIM || (cos_sin_batch_stride % 8) != 0)))
+        return PQ_ERR_BAD_STRIDE;
+    if (!aligned(q_lin, 16) || !aligned(k_lin, 16) || !aligned(cos_rows, 16) || !aligned(sin_rows, 16) || !aligned(q_out, 16) ||
+        !aligned(k_out, 16))
+        return PQ_ERR_MISALIGNED;
+    const int err = pq::launch_rope_qk(q_lin, q_token_stride, k_lin, k_token_stride, cos_rows, sin_rows, cos_sin_batch_stride,
+                                       q_out, k_out, B, L, N, Nk, dtype, static_cast<hipStream_t>(stream));
+    return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+
 int pq_rmsnorm(const void* x, const void* residual, const void* weight, void* y, void* sum_out, int rows, int hidden,
                float eps, int dtype, void* stream) {
     if (!x || !weight || !y) return PQ_ERR_NULL_POINTER;

@@ -68,6 +68,55 @@ __global__ __launch_bounds__(kWave) void rope_append_kernel(
     dst[d + kPairs] = f2lo<T>(o2);
 }
 
+// RoPE over whole sequences (the prompt pass, models/modeling_llama_polar.py:56-59): one workgroup per token,
+// all query and key heads of it; a thread takes dims c..c+7 and 64+c..64+c+7 of one head (two 16-byte loads), the
+// token's cos / sin rows are shared by its heads.  Same arithmetic as rope_append_kernel, so the same bits as the
+// eager (x * cos) + (rotate_half(x) * sin).
+//   q_lin / k_lin: projection outputs, token t = b * L + l at q_lin + t * q_stride (k likewise)
+//   cos / sin [1 or B, L, 128]: batch b at b * cs_batch_stride (0 when shared)
+//   q_out [B, L, N, 128], k_out [B, L, Nk, 128] contiguous
+template <typename T>
+__global__ __launch_bounds__(256) void rope_qk_kernel(
+    const uint16_t* __restrict__ q_lin, int64_t q_stride, const uint16_t* __restrict__ k_lin, int64_t k_stride,
+    const uint16_t* __restrict__ cos_t, const uint16_t* __restrict__ sin_t, int64_t cs_batch_stride,
+    uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_out, int L, int N, int Nk) {
+    const size_t tok = blockIdx.x;
+    const size_t b = tok / L, l = tok - b * L;
+    const size_t cs = b * cs_batch_stride + l * kHeadDim;
+    for (int item = threadIdx.x; item < (N + Nk) * 8; item += 256) {
+        const int head = item >> 3, c = (item & 7) * 8;
+        const bool is_q = head < N;
+        const uint16_t* src = is_q ? q_lin + tok * q_stride + static_cast<size_t>(head) * kHeadDim
+                                   : k_lin + tok * k_stride + static_cast<size_t>(head - N) * kHeadDim;
+        uint16_t* dst = is_q ? q_out + (tok * N + head) * kHeadDim : k_out + (tok * Nk + (head - N)) * kHeadDim;
+        const uint4 a1 = *reinterpret_cast<const uint4*>(src + c), a2 = *reinterpret_cast<const uint4*>(src + kPairs + c);
+        const uint4 vc1 = *reinterpret_cast<const uint4*>(cos_t + cs + c), vc2 = *reinterpret_cast<const uint4*>(cos_t + cs + kPairs + c);
+        const uint4 vs1 = *reinterpret_cast<const uint4*>(sin_t + cs + c), vs2 = *reinterpret_cast<const uint4*>(sin_t + cs + kPairs + c);
+        const uint32_t x1w[4] = {a1.x, a1.y, a1.z, a1.w}, x2w[4] = {a2.x, a2.y, a2.z, a2.w};
+        const uint32_t c1w[4] = {vc1.x, vc1.y, vc1.z, vc1.w}, c2w[4] = {vc2.x, vc2.y, vc2.z, vc2.w};
+        const uint32_t s1w[4] = {vs1.x, vs1.y, vs1.z, vs1.w}, s2w[4] = {vs2.x, vs2.y, vs2.z, vs2.w};
+        uint32_t o1w[4], o2w[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t r1 = 0, r2 = 0;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+                const int sh = 16 * hh;
+                const float x1 = lo2f<T>(static_cast<uint16_t>(x1w[j] >> sh)), x2 = lo2f<T>(static_cast<uint16_t>(x2w[j] >> sh));
+                const float c1 = lo2f<T>(static_cast<uint16_t>(c1w[j] >> sh)), c2 = lo2f<T>(static_cast<uint16_t>(c2w[j] >> sh));
+                const float s1 = lo2f<T>(static_cast<uint16_t>(s1w[j] >> sh)), s2 = lo2f<T>(static_cast<uint16_t>(s2w[j] >> sh));
+                const float o1 = rnd_a<T>(x1 * c1) + rnd_a<T>(-x2 * s1);
+                const float o2 = rnd_a<T>(x2 * c2) + rnd_a<T>(x1 * s2);
+                r1 |= static_cast<uint32_t>(f2lo<T>(o1)) << sh;
+                r2 |= static_cast<uint32_t>(f2lo<T>(o2)) << sh;
+            }
+            o1w[j] = r1; o2w[j] = r2;
+        }
+        *reinterpret_cast<uint4*>(dst + c) = make_uint4(o1w[0], o1w[1], o1w[2], o1w[3]);
+        *reinterpret_cast<uint4*>(dst + kPairs + c) = make_uint4(o2w[0], o2w[1], o2w[2], o2w[3]);
+    }
+}
+
 // One 256-thread block per row of `hidden` elements (hidden % 8 == 0).
 //   s = x (+ res, rounded to the dtype; written to sum_out if given)
 //   y = w * dtype( float(s) * rsqrt(mean(float(s)^2) + eps) )
@@ -210,6 +259,19 @@ int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, 
                        q_stride, kv_stride)
     if (dtype == 0) PQ_RA(F16); else PQ_RA(BF16);
 #undef PQ_RA
+    return static_cast<int>(hipGetLastError());
+}
+
+int launch_rope_qk(const void* q_lin, int64_t q_stride, const void* k_lin, int64_t k_stride, const void* cos_t,
+                   const void* sin_t, int64_t cs_batch_stride, void* q_out, void* k_out, int B, int L, int N, int Nk,
+                   int dtype, hipStream_t st) {
+    dim3 grid(static_cast<unsigned>(static_cast<size_t>(B) * L)), block(256);
+#define PQ_RQ(T)                                                                                                     \
+    hipLaunchKernelGGL(rope_qk_kernel<T>, grid, block, 0, st, (const uint16_t*)q_lin, q_stride, (const uint16_t*)k_lin, \
+                       k_stride, (const uint16_t*)cos_t, (const uint16_t*)sin_t, cs_batch_stride, (uint16_t*)q_out,   \
+                       (uint16_t*)k_out, L, N, Nk)
+    if (dtype == 0) PQ_RQ(F16); else PQ_RQ(BF16);
+#undef PQ_RQ
     return static_cast<int>(hipGetLastError());
 }
 

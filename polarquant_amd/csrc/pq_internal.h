@@ -19,6 +19,9 @@ int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st);
 int launch_quantize_values(const void* v, const int64_t* strides, int dtype, int B, int Nk, int T,
                            int32_t* codes, void* scale, void* mn, int64_t cap, int64_t off, hipStream_t st);
 
+int launch_rope_qk(const void* q_lin, int64_t q_stride, const void* k_lin, int64_t k_stride, const void* cos_t,
+                   const void* sin_t, int64_t cs_batch_stride, void* q_out, void* k_out, int B, int L, int N, int Nk,
+                   int dtype, hipStream_t st);
 int launch_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_tab, const void* sin_tab,
                        const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,
                        void* v_dst, int64_t v_rows, const int64_t* v_row, int B, int N, int Nk, int64_t max_pos, int dtype,

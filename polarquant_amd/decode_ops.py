@@ -136,3 +136,33 @@ def qkv_rope_append(x: torch.Tensor, w_qkv: torch.Tensor, b_qkv: Optional[torch.
                                            _stream_ptr(x.device))
     _ffi.check(rc, "pq_qkv_rope_append")
     return q_out
+
+
+def rope_qk(q_lin: torch.Tensor, k_lin: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, n_heads: int, n_kv_heads: int):
+    """`apply_rotary_pos_emb` on projection outputs in one launch, bit-identical to the eager ops: q_lin [B,L,N*128],
+    k_lin [B,L,Nk*128] (unit element stride, uniform token stride), cos / sin [1 or B, L, 128] in the same dtype.
+    Returns (q [B,N,L,128], k [B,Nk,L,128]) as transposed views of [B,L,heads,128] tensors, the layout the eager
+    `.view(B, L, heads, 128).transpose(1, 2)` followed by the rotation produces."""
+    _gpu(q_lin)
+    B, L = q_lin.shape[0], q_lin.shape[1]
+    assert q_lin.shape[-1] == n_heads * 128 and k_lin.shape[-1] == n_kv_heads * 128 and k_lin.shape[:2] == (B, L)
+    assert cos.shape == sin.shape and cos.shape[-2:] == (L, 128) and cos.shape[0] in (1, B) and cos.dtype == q_lin.dtype == k_lin.dtype
+
+    def rows(t):                       # token b * L + l at (b * L + l) * token_stride, unit element stride
+        def token_stride(u):
+            return u.stride(1) if L > 1 else (u.stride(0) if B > 1 else u.shape[-1])
+        if (t.stride(-1) != 1 or (B > 1 and L > 1 and t.stride(0) != L * t.stride(1)) or token_stride(t) % 8 != 0
+                or token_stride(t) < t.shape[-1] or t.data_ptr() % 16):
+            t = t.contiguous()
+        return t, token_stride(t)
+    q_lin, qs = rows(q_lin)
+    k_lin, ks = rows(k_lin)
+    cos, sin = cos.contiguous(), sin.contiguous()
+    q_out = torch.empty((B, L, n_heads, 128), dtype=q_lin.dtype, device=q_lin.device)
+    k_out = torch.empty((B, L, n_kv_heads, 128), dtype=q_lin.dtype, device=q_lin.device)
+    with torch.cuda.device(q_lin.device):
+        rc = _ffi.lib().pq_rope_qk(q_lin.data_ptr(), qs, k_lin.data_ptr(), ks, cos.data_ptr(), sin.data_ptr(),
+                                   0 if cos.shape[0] == 1 else L * 128, q_out.data_ptr(), k_out.data_ptr(), B, L, n_heads,
+                                   n_kv_heads, _dtype_code(q_lin), _stream_ptr(q_lin.device))
+    _ffi.check(rc, "pq_rope_qk")
+    return q_out.transpose(1, 2), k_out.transpose(1, 2)

@@ -92,6 +92,20 @@ def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim: int = 1):
     return (q * cos) + (rotate_half(q) * sin), (k * cos) + (rotate_half(k) * sin)
 
 
+def project_heads_and_rotate(q_lin, k_lin, cos, sin, n_heads: int, n_kv_heads: int, head_dim: int):
+    """The reference's `.view(B, L, heads, d).transpose(1, 2)` on the q / k projections followed by
+    `apply_rotary_pos_emb` (models/modeling_llama_polar.py:53-59).  On the GPU, at head_dim 128 in half precision, one
+    HIP launch with the same bits as the eager chain of multiplies, negation, concatenation and add."""
+    B, L = q_lin.shape[0], q_lin.shape[1]
+    if (q_lin.is_cuda and head_dim == 128 and q_lin.dtype in (torch.float16, torch.bfloat16) and cos.dtype == q_lin.dtype
+            and cos.dim() == 3 and cos.shape[0] in (1, B) and tuple(cos.shape[1:]) == (L, 128) and not torch.is_grad_enabled()):
+        from .decode_ops import rope_qk
+        return rope_qk(q_lin, k_lin, cos, sin, n_heads, n_kv_heads)
+    q = q_lin.view(B, L, n_heads, head_dim).transpose(1, 2)
+    k = k_lin.view(B, L, n_kv_heads, head_dim).transpose(1, 2)
+    return apply_rotary_pos_emb(q, k, cos, sin)
+
+
 def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
     b, h, s, d = hidden_states.shape
     if n_rep == 1:
@@ -310,11 +324,10 @@ class PolarGroupAttention(nn.Module):
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 past_key_value=None, position_embeddings: Tuple[torch.Tensor, torch.Tensor] = None, **kwargs):
         bsz, q_len, _ = hidden_states.size()
-        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         cos, sin = position_embeddings
-        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        query_states, key_states = project_heads_and_rotate(self.q_proj(hidden_states), self.k_proj(hidden_states), cos, sin,
+                                                            self.num_heads, self.num_key_value_heads, self.head_dim)
         if self.capture is not None:
             self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
 
@@ -448,11 +461,10 @@ class PolarMixedGroupAttention(PolarGroupAttention):
     def forward(self, hidden_states: torch.Tensor, attention_mask: Optional[torch.Tensor] = None,
                 past_key_value=None, position_embeddings: Tuple[torch.Tensor, torch.Tensor] = None, **kwargs):
         bsz, q_len, _ = hidden_states.size()
-        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         cos, sin = position_embeddings
-        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        query_states, key_states = project_heads_and_rotate(self.q_proj(hidden_states), self.k_proj(hidden_states), cos, sin,
+                                                            self.num_heads, self.num_key_value_heads, self.head_dim)
         if self.capture is not None:
             self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
 
@@ -529,11 +541,10 @@ class PolarSnapKVAttention(PolarGroupAttention):
         if q_len == 1:
             assert bsz == 1                                                # :327 (no per-sequence mask after eviction)
             return super().forward(hidden_states, None, past_key_value, position_embeddings, **kwargs)
-        query_states = self.q_proj(hidden_states).view(bsz, q_len, self.num_heads, self.head_dim).transpose(1, 2)
-        key_states = self.k_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         value_states = self.v_proj(hidden_states).view(bsz, q_len, self.num_key_value_heads, self.head_dim).transpose(1, 2)
         cos, sin = position_embeddings
-        query_states, key_states = apply_rotary_pos_emb(query_states, key_states, cos, sin)
+        query_states, key_states = project_heads_and_rotate(self.q_proj(hidden_states), self.k_proj(hidden_states), cos, sin,
+                                                            self.num_heads, self.num_key_value_heads, self.head_dim)
         if self.capture is not None:
             self.capture.append((query_states.detach().clone(), key_states.detach().clone(), value_states.detach().clone()))
         assert past_key_value is None

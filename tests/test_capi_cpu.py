@@ -239,6 +239,22 @@ def test_stream_read_rejects_bad_arguments(lib):
     assert lib.pq_stream_read(P, 1000, 1024, P, None) == 0          # less than one 16 KiB trip per wavefront
 
 
+def test_rope_qk_rejects_bad_arguments(lib):
+    ok = [P, 0, P, 0, P, P, 0, P, P, 2, 300, 32, 8, 1]
+    def call(a):
+        return lib.pq_rope_qk(*a, None)
+    def bad(i, v):
+        a = list(ok)
+        a[i] = v
+        return call(a)
+    for i in (0, 2, 4, 5, 7, 8):
+        assert bad(i, None) == -1, i
+    assert bad(13, 2) == -4
+    assert bad(9, 0) == -2 and bad(10, 0) == -2 and bad(11, 0) == -2 and bad(12, 0) == -2
+    assert bad(1, 4000) == -6 and bad(1, 4100) == -6 and bad(3, 1000) == -6 and bad(6, 128) == -6 and bad(6, 300 * 128 + 4) == -6
+    assert bad(0, P + 8) == -5 and bad(4, P + 2) == -5 and bad(8, P + 4) == -5
+
+
 def test_attn_load_replica_rejects_bad_arguments(lib):
     ok = [P, P, 128, 32768, 32769, 32768, 8, P]
     def bad(i, v):

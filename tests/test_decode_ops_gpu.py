@@ -113,3 +113,26 @@ def test_measurement_aids_launch_and_report_their_bytes(gpu):
     assert got == 7 * (v.numel() * 2 // 7 // 16384 * 16384)
     torch.cuda.synchronize()
     assert torch.equal(codes, before[0]) and torch.equal(v, before[1]) and int(sink) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,L,N,Nk,per_seq", [(2, 300, 4, 2, False), (3, 1, 7, 1, True), (1, 129, 32, 8, False), (2, 64, 28, 4, True)])
+def test_rope_qk_is_the_eager_rotation_bit_for_bit(gpu, dtype, B, L, N, Nk, per_seq):
+    from polarquant_amd.decode_ops import rope_qk
+    from polarquant_amd.modeling_common import apply_rotary_pos_emb
+    g = torch.Generator().manual_seed(B * 100 + L + N)
+    fused = (torch.randn(B, L, (N + 2 * Nk) * 128, generator=g) * 3).to(dtype).to(gpu)      # slices of one projection output
+    q_lin, k_lin = fused[..., :N * 128], fused[..., N * 128:(N + Nk) * 128]
+    pos = torch.arange(L, dtype=torch.float32)[None].repeat(B if per_seq else 1, 1)
+    if per_seq:
+        pos = pos + torch.arange(pos.shape[0], dtype=torch.float32)[:, None] * 17
+    ang = pos[..., None] * (5e5 ** (-torch.arange(0, 128, 2).float() / 128))
+    emb = torch.cat([ang, ang], -1)
+    cos, sin = emb.cos().to(dtype).to(gpu), emb.sin().to(dtype).to(gpu)
+    q_ref, k_ref = apply_rotary_pos_emb(q_lin.reshape(B, L, N, 128).transpose(1, 2), k_lin.reshape(B, L, Nk, 128).transpose(1, 2), cos, sin)
+    q, k = rope_qk(q_lin, k_lin, cos, sin, N, Nk)
+    assert q.shape == (B, N, L, 128) and k.shape == (B, Nk, L, 128)
+    assert torch.equal(q, q_ref) and torch.equal(k, k_ref)
+    # dense inputs take the same path
+    q2, k2 = rope_qk(q_lin.contiguous(), k_lin.contiguous(), cos, sin, N, Nk)
+    assert torch.equal(q2, q_ref) and torch.equal(k2, k_ref)
