@@ -196,6 +196,35 @@ def test_generate_with_the_graph_decoder(gpu):
     assert smp.shape == (B, 4) and int(smp.min()) >= 0 and int(smp.max()) < cfg.vocab_size
 
 
+def test_generate_with_the_graph_decoder_on_the_mixed_variant(gpu):
+    """4-bit values (11-slot cache) and a Qwen-shaped model with biases through `generate(..., graph_decoder=True)`:
+    same tokens as the decoder driven by hand, every pick within rounding of the eager model's best."""
+    from polarquant_amd.modeling_common import GenerationConfig, generate
+    for cls, cfg, dtype in ((LlamaPolarForCausalLM, _tiny(8, 2, vbits=4), torch.float16),
+                            (Qwen2PolarForCausalLM, _tiny(7, 1, rbits=3, tbits=3, attention_bias=True), torch.bfloat16)):
+        torch.manual_seed(37)
+        model = cls(cfg).to(dtype).to(gpu).eval()
+        B, L, new = 2, 250, 10                     # flush at 256 tokens
+        ids = torch.randint(0, cfg.vocab_size, (B, L), device=gpu)
+        got = generate(model, ids, None, GenerationConfig(eos_token_id=[999999]), max_new_tokens=new, graph_decoder=True)
+        assert got.shape == (B, new)
+        dec = PolarGraphDecoder(model, max_len=L + new + 1)
+        with torch.no_grad():
+            tok = dec.prefill(ids).argmax(-1)
+            by_hand = [tok]
+            for _ in range(new - 1):
+                tok = dec.step(tok).argmax(-1)
+                by_hand.append(tok)
+            assert torch.equal(got, torch.cat(by_hand, dim=-1))
+            cache, tok = None, ids
+            for s in range(new):
+                out = model(input_ids=tok, attention_mask=None, past_key_values=cache, num_logits_to_keep=1)
+                cache, rl = out.past_key_values, out.logits.float()
+                tok = got[:, s:s + 1]
+                pick = rl.gather(-1, tok.unsqueeze(-1)).squeeze(-1)
+                assert bool((rl.max(-1).values - pick <= 4e-2 * max(1.0, rl.abs().max().item())).all()), (cls.__name__, s)
+
+
 def test_graph_decoder_rejects_overflow(gpu):
     torch.manual_seed(12)
     cfg = _tiny(layers=1)
