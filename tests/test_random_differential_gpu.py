@@ -12,11 +12,14 @@ from polarquant_amd import workloads as wl
 from polarquant_amd.attention import polar_decode_attention, polar_decode_attention_v4
 
 pytestmark = pytest.mark.gpu
+# more seeds: PQ_RANDOM_CASES=300; another stretch of them: PQ_RANDOM_FIRST=1000
+SEEDS = range(int(os.environ.get("PQ_RANDOM_FIRST", "0")),
+              int(os.environ.get("PQ_RANDOM_FIRST", "0")) + int(os.environ.get("PQ_RANDOM_CASES", "24")))
 HEADS = [(1, 1), (2, 1), (4, 4), (8, 2), (3, 1), (6, 1), (7, 1), (8, 1), (16, 2), (12, 4)]
 BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 4)]
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))   # more seeds: PQ_RANDOM_CASES=300
+@pytest.mark.parametrize("seed", SEEDS)
 def test_random_decode_attention_case(gpu, seed):
     rnd = random.Random(1000 + seed)
     N, Nk = rnd.choice(HEADS)
@@ -103,7 +106,7 @@ def test_random_decode_attention_case(gpu, seed):
         assert bad == 0, (b, bad, float(err.max()))
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))
+@pytest.mark.parametrize("seed", SEEDS)
 def test_random_quantizer_case(gpu, seed):
     """Key and value quantizers, bit for bit against the oracle, on keys / values of random scale
     (1e-6 .. 1e4), distribution (normal, heavy-tailed, sparse, nearly constant) and bit widths."""
@@ -140,7 +143,7 @@ def test_random_quantizer_case(gpu, seed):
         assert bool(((a == b) | (a.isnan() & b.isnan())).all()), name
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("PQ_RANDOM_CASES", "24"))))
+@pytest.mark.parametrize("seed", SEEDS)
 def test_random_scores_case(gpu, seed):
     """The score op on random heads / bit widths / group counts, with quantized keys or (as the reference's
     micro-benchmark does) arbitrary codes and randn metadata, byte-per-code or packed 6-bit rows."""
