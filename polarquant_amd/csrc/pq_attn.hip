@@ -23,8 +23,9 @@
 // kLazyThreshold (in log2 units): probabilities stay below 2^8, and the
 // 32-register rescale of the accumulators is skipped on almost every tile.
 //
-// merge_kernel: grid B*N, 128 threads (one per output dim): combines the
-// n_splits partials (m, l, acc[128]) of a query head and writes half words.
+// merge_kernel: grid B*N, 128 threads (one per output dim), or four / eight such
+// groups that share the partials when there are 32 / 128 or more: combines the n_splits
+// partials (m, l, acc[128]) of a query head and writes half words.
 #include "pq_device.h"
 #include "pq_internal.h"
 
@@ -576,26 +577,31 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 }
 #pragma clang diagnostic pop
 
-template <typename T>
-__global__ __launch_bounds__(kHeadDim) void merge_kernel(const float* __restrict__ ws, int n_part, uint16_t* __restrict__ out) {
-    // one block per query head, thread == output dim.  The partial headers (m, l)
-    // are fetched by one thread each, so that all loads of the block are issued
-    // at once instead of one dependent load per partial.
+template <typename T, int G>
+__global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __restrict__ ws, int n_part, uint16_t* __restrict__ out) {
+    // one block per query head, G groups of 128 threads: thread (grp, d) sums output dim d over
+    // the grp-th share of the partials, and the G sums are added in a fixed order through LDS.
+    // The partial headers (m, l) are fetched by one thread each, so that all loads of the block
+    // are issued at once instead of one dependent load per partial.
+    constexpr int NT = kHeadDim * G, NW = NT / kWave;
     __shared__ float wgt[1024];
-    __shared__ float red[2][kHeadDim / kWave];
-    const int bn = blockIdx.x, d = threadIdx.x;
+    __shared__ float red[2][NW];
+    __shared__ float part[G][kHeadDim];
+    const int bn = blockIdx.x, tid = threadIdx.x, d = tid & (kHeadDim - 1), grp = tid / kHeadDim;
     const float* p = ws + static_cast<size_t>(bn) * n_part * kPartialFloats;
     float M = -INFINITY;
-    for (int s = d; s < n_part; s += kHeadDim) M = fmaxf(M, p[static_cast<size_t>(s) * kPartialFloats]);
+    for (int s = tid; s < n_part; s += NT) M = fmaxf(M, p[static_cast<size_t>(s) * kPartialFloats]);
     M = wave_max(M);
-    if ((d & (kWave - 1)) == 0) red[0][d / kWave] = M;
+    if ((tid & (kWave - 1)) == 0) red[0][tid / kWave] = M;
     __syncthreads();
-    M = fmaxf(red[0][0], red[0][1]);
+    M = red[0][0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) M = fmaxf(M, red[0][i]);
     float num = 0.0f, den = 0.0f;
     for (int s0 = 0; s0 < n_part; s0 += 1024) {
         const int cnt = (n_part - s0) < 1024 ? (n_part - s0) : 1024;
         __syncthreads();
-        for (int s = d; s < cnt; s += kHeadDim) {
+        for (int s = tid; s < cnt; s += NT) {
             const float m = p[static_cast<size_t>(s0 + s) * kPartialFloats];
             const float w = (m == -INFINITY) ? 0.0f : exp2f(m - M);
             wgt[s] = w;
@@ -603,24 +609,39 @@ __global__ __launch_bounds__(kHeadDim) void merge_kernel(const float* __restrict
         }
         __syncthreads();
         const float* pa = p + static_cast<size_t>(s0) * kPartialFloats + 4 + d;
-        int s = 0;
-        for (; s + 8 <= cnt; s += 8) {
+        const int per = (cnt + G - 1) / G;
+        int s = grp * per;
+        const int se = (s + per) < cnt ? (s + per) : cnt;
+        for (; s + 16 <= se; s += 16) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) v[u] = pa[static_cast<size_t>(s + u) * kPartialFloats];
+#pragma unroll
+            for (int u = 0; u < 16; u++) num = wgt[s + u] != 0.0f ? __builtin_fmaf(wgt[s + u], v[u], num) : num;
+        }
+        for (; s + 8 <= se; s += 8) {
             float v[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) v[u] = pa[static_cast<size_t>(s + u) * kPartialFloats];
 #pragma unroll
             for (int u = 0; u < 8; u++) num = wgt[s + u] != 0.0f ? __builtin_fmaf(wgt[s + u], v[u], num) : num;
         }
-        for (; s < cnt; s++) {
+        for (; s < se; s++) {
             const float v = pa[static_cast<size_t>(s) * kPartialFloats];
             num = wgt[s] != 0.0f ? __builtin_fmaf(wgt[s], v, num) : num;
         }
     }
     den = wave_sum(den);
     __syncthreads();
-    if ((d & (kWave - 1)) == 0) red[1][d / kWave] = den;
+    if ((tid & (kWave - 1)) == 0) red[1][tid / kWave] = den;
+    if (G > 1) part[grp][d] = num;
     __syncthreads();
-    den = red[1][0] + red[1][1];
+    if (grp != 0) return;
+    den = red[1][0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) den += red[1][i];
+#pragma unroll
+    for (int i = 1; i < G; i++) num += part[i][d];
     out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : 0.0f);
 }
 
@@ -679,11 +700,25 @@ int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
     return a.dtype == 0 ? launch_attn_t<F16>(a, st) : launch_attn_t<BF16>(a, st);
 }
 
+constexpr int kMergeWideFrom = 32, kMergeWidestFrom = 128;
+
 int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st) {
-    if (dtype == 0)
-        hipLaunchKernelGGL(merge_kernel<F16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
-    else
-        hipLaunchKernelGGL(merge_kernel<BF16>, dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
+    // many partials per head (a long context cut into many slices): four or eight groups of threads share them
+    if (n_splits >= kMergeWidestFrom) {
+        if (dtype == 0)
+            hipLaunchKernelGGL((merge_kernel<F16, 8>), dim3(B * N), dim3(kHeadDim * 8), 0, st, ws, n_splits, (uint16_t*)out);
+        else
+            hipLaunchKernelGGL((merge_kernel<BF16, 8>), dim3(B * N), dim3(kHeadDim * 8), 0, st, ws, n_splits, (uint16_t*)out);
+    } else if (n_splits >= kMergeWideFrom) {
+        if (dtype == 0)
+            hipLaunchKernelGGL((merge_kernel<F16, 4>), dim3(B * N), dim3(kHeadDim * 4), 0, st, ws, n_splits, (uint16_t*)out);
+        else
+            hipLaunchKernelGGL((merge_kernel<BF16, 4>), dim3(B * N), dim3(kHeadDim * 4), 0, st, ws, n_splits, (uint16_t*)out);
+    } else if (dtype == 0) {
+        hipLaunchKernelGGL((merge_kernel<F16, 1>), dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
+    } else {
+        hipLaunchKernelGGL((merge_kernel<BF16, 1>), dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
+    }
     return static_cast<int>(hipGetLastError());
 }
 
