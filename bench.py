@@ -31,8 +31,9 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 MEASURED_TRAFFIC_BYTES = int(676933 * 2.0 * 1024 + 2176 * 1.0 * 1024)
 
 
-def build_cfg1(dev, dtype=torch.float16):
-    return build_workload(1, dev, dtype)
+def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):
+    from polarquant_amd import workloads as wl
+    return wl.build_workload(1, dev, dtype, keep_keys_of=keep_keys_of)
 
 
 def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False):
@@ -85,6 +86,21 @@ def cpu_baseline(w):
                   "of the reference path (dequantize, matmul, softmax, P.V), scaled x%d to the batch"
                   % (sh.batch, len(times), sh.batch),
     }
+
+
+def code_flips(w):
+    """Codes and metadata the HIP quantizer wrote for sequence 0 against the CPU restatement of the
+    reference's quantizer (modeling_llama_polar.py:135-157) on the same keys: a differing code is a
+    bin-edge flip (a rounding or arctangent difference), a differing metadata word a min/max or scale
+    that came out in another half-precision value.  Both counts are meant to be 0."""
+    from oracle import polar_oracle as po
+    sh = w["shape"]
+    ref = po.quantize_and_pack_nbit(w["keys"][0:1].cpu(), sh.rbits, sh.tbits)
+    got = [w["codes"][0:1].cpu()] + [m[0:1].cpu() for m in w["meta"]]
+    return {"codes": ref[0].numel(), "flips": int((ref[0] != got[0]).sum()),
+            "metadata_words": sum(m.numel() for m in ref[1:]),
+            "metadata_words_differing": sum(int((a.view(torch.int16) != b.view(torch.int16)).sum()) for a, b in zip(ref[1:], got[1:])),
+            "sample": "sequence 0 of %d: %d KV heads x %d keys" % (sh.batch, sh.n_kv_heads, sh.context)}
 
 
 def fp16_baselines(w, steps, warmup):
@@ -186,7 +202,7 @@ def main():
     lib = _ffi.lib()
     # two independent copies of the workload, used alternately: no step can find its inputs in a
     # cache left by the previous one (the Infinity Cache holds 256 MB; one copy is 1.36 GB)
-    w = build_cfg1(dev)
+    w = build_cfg1(dev, keep_keys_of=None if args.no_baselines else 1)
     w_alt = build_cfg1(dev)
     sh = w["shape"]
     B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
@@ -312,6 +328,8 @@ def main():
         torch.cuda.empty_cache()
         ref, cpu = cpu_baseline(w)
         result["cpu_baseline"] = cpu
+        result["code_flips_vs_cpu_sample"] = code_flips(w)
+        w["keys"] = None
         got = out[0:1].cpu()
         err = (got.double() - ref.double()).abs()
         result["parity_vs_cpu_sample"] = {"max_abs_err": float(err.max()),

@@ -124,10 +124,12 @@ def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], re
 
 
 # ----------------------------------------------------------------------------- GPU-resident workloads and timing
-def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False):
+def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False, keep_keys_of=None):
     """configs[idx] resident in HBM: polar key cache of L/128 groups per (sequence, KV head),
     fp16 V cache, one new token whose key sits in the fp16 residual buffer.  Ragged shapes
-    (configs[2]) carry per-sequence group / residual counts; their caches are sized for the longest."""
+    (configs[2]) carry per-sequence group / residual counts; their caches are sized for the longest.
+    keep_keys keeps the half-precision keys of every sequence in w["keys"], keep_keys_of=n those of the
+    first n sequences only."""
     from .quantize import quantize_and_pack_nbit
 
     sh = CONFIGS[idx]
@@ -147,7 +149,7 @@ def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False)
         k[..., outl] *= 8.0
         k = (k * cos + torch.cat([-k[..., 64:], k[..., :64]], -1) * sin).to(dtype)
         quantize_and_pack_nbit(k, sh.rbits, sh.tbits, packed=packed, out=(codes[b:b + 1], *[m[b:b + 1] for m in meta]))
-        if keep_keys:
+        if keep_keys or (keep_keys_of is not None and b < keep_keys_of):
             keys.append(k)
     v = torch.empty(B, Nk, L + 1, 128, dtype=dtype, device=dev)
     for b in range(B):
@@ -157,7 +159,7 @@ def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False)
     kres = torch.zeros(B, Nk, 128, 128, dtype=dtype, device=dev)
     kres[:, :, :1] = k_new
     w = dict(shape=sh, q=q, codes=codes, meta=meta, kres=kres, v=v, n_groups=Nb, n_resid=1, lengths=None,
-             groups_per_seq=None, resid_per_seq=None, keys=torch.cat(keys, 0) if keep_keys else None)
+             groups_per_seq=None, resid_per_seq=None, keys=torch.cat(keys, 0) if keys else None)
     if sh.ragged:
         # per-sequence context lengths, uniform in [512, L]: full groups are quantized, the tail
         # (L % 128 tokens) stays fp16 in the residual buffer, which is filled from the keys' tail
