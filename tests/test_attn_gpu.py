@@ -96,6 +96,16 @@ def test_attn_split_invariance(gpu, n_splits):
     assert _close(out, ref64)[0] == 0
 
 
+@pytest.mark.parametrize("n_splits,dtype", [(33, torch.float16), (70, torch.bfloat16), (130, torch.float16), (1030, torch.float16)])
+def test_attn_many_splits(gpu, n_splits, dtype):
+    """32 or more / 128 or more partials per head take the merge kernel's 4- and 8-group forms; more
+    slices than groups leave empty partials, more than 1024 a second pass over the weight buffer."""
+    print("case", n_splits, dtype, flush=True)
+    out, ref, ref64 = _case(gpu, 1, 8, 2, 130, 3, 4, 4, dtype, seed=11, n_splits=n_splits)
+    rtol, atol = (RTOL, ATOL) if dtype == torch.float16 else (2e-2, 4e-3)   # bf16 has 8 mantissa bits
+    assert _close(out, ref64, rtol, atol)[0] == 0
+
+
 def test_attn_left_padding_mask(gpu):
     out, ref, ref64 = _case(gpu, 3, 32, 8, 4, 19, 4, 4, torch.float16, seed=4, mask_pad=150)
     assert _close(out, ref64)[0] == 0 and _close(out, ref)[0] == 0
