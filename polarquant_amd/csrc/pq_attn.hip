@@ -420,12 +420,12 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             uint16_t vsz[2][2] = {{0, 0}, {0, 0}};             // (scale, zero-point) words of this lane's token, by tile parity
             auto load_values = [&](int buf, uint32_t tile_tok, bool in_range) {
                 if constexpr (V4) {
-                    load_v4_tile(vv[buf].r, rq, voff_q, in_range ? tile_tok * 64u : 0xFFFFFF00u);
+                    load_v4_tile(vv[buf].r, rq, voff_q, in_range ? tile_tok * 64u : 0xFFFF0000u);
                     const int so = in_range ? static_cast<int>(tile_tok * 2u) : static_cast<int>(0x7FFFFF00);
                     vsz[buf][0] = __builtin_amdgcn_raw_buffer_load_b16(rvs, lane * 2, so, 0);
                     vsz[buf][1] = __builtin_amdgcn_raw_buffer_load_b16(rvz, lane * 2, so, 0);
                 } else {
-                    load_v_tile(vv[buf].r, rv, voff_v, in_range ? tile_tok * (kHeadDim * 2) : 0xFFFFFF00u);
+                    load_v_tile(vv[buf].r, rv, voff_v, in_range ? tile_tok * (kHeadDim * 2) : 0xFFFF0000u);
                 }
             };
             load_values(0, static_cast<uint32_t>(2 * g0) * kWave, true);
@@ -446,7 +446,8 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
                 for (int half = 0; half < 2; half++) {
                     const int tt = 2 * grp + half;
                     const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
-                    // past the last tile of this slice the loads run off the buffer's end and return zeros
+                    // past the last tile of this slice the loads run off the buffer's end and return zeros (the
+                    // out-of-range offset leaves room for the 16 KiB of row offsets added to it: no 32-bit wrap)
                     PQ_T_MARK();
                     load_values(half ^ 1, tok0 + kWave, half == 0 || grp + 1 < g1);
                     PQ_T_ADD(1);
