@@ -22,6 +22,12 @@ the checks live in tests/test_oracle_pins.py):
   decode_attention         pinned: composition of torch.matmul/softmax library
                            routines; cross-checked against a one-shot softmax
                            over the concatenated dequantized+residual keys.
+  residual_score_rounding_band
+                           (a tolerance aid, no reference counterpart: how far the
+                           reference's own rounding of the window's scores, :79,
+                           can move the output) pinned: it covers the movement
+                           measured when those scores are actually rounded, and
+                           that movement reaches a fair fraction of it.
   prefill_cache/decode_step pinned: shape/bookkeeping property tests (quantized
                            token count, residual length, kv_seq_len).
   quantize_values_along_last_dim / dequantize_values / decode_attention_mixed
@@ -285,6 +291,42 @@ def decode_attention_exact(query_states, key_resid, indices, rscale, rmn, tscale
         attn = attn.masked_fill(attention_mask[:, None, None, :] == 0, float("-inf"))
     p = torch.softmax(attn, dim=-1)
     return torch.matmul(p, repeat_kv(value_states.to(torch.float64), rep))
+
+
+def residual_score_rounding_band(query_states, key_resid, indices, rscale, rmn, tscale, tmn, value_states,
+                                 attention_mask=None, rbits=4, tbits=4) -> torch.Tensor:
+    """How far the output can move, to first order, when each score of the residual window is rounded
+    to the model dtype to either neighbour: fp64 [B,N,1,128].
+
+    The reference multiplies q.K^T of the un-quantized keys in the model dtype (:79), so those scores
+    carry one rounding of up to half an ulp (0.125 for a bfloat16 score between 32 and 64), and two
+    correct evaluations of that line may round a score to different neighbours when their fp32 sums
+    differ in the last bits.  With d(out) = sum_i p_i (v_i - out) d(logit_i), the bound is
+        sum_{i in window} p_i |v_i - out| ulp(s_i) / 2 / sqrt(head_dim),
+    everything evaluated in fp64 as in decode_attention_exact.  `value_states`: the values of all
+    attended tokens (for the 4-bit variant: dequantized rows followed by the window's rows)."""
+    B, N, _, hd = query_states.shape
+    Nk = value_states.shape[1]
+    rep = N // Nk
+    ks, n_quant = [], 0
+    if indices is not None:
+        ks.append(dequantize_keys(indices, rscale, rmn, tscale, tmn, rbits, tbits, torch.float64))
+        n_quant = ks[0].shape[2]
+    if key_resid is None or key_resid.shape[2] == 0:
+        return torch.zeros(B, N, 1, hd, dtype=torch.float64)
+    ks.append(key_resid.to(torch.float64))
+    k = torch.cat(ks, dim=2)
+    s = torch.matmul(query_states.to(torch.float64), repeat_kv(k, rep).transpose(2, 3))      # [B,N,1,L], unscaled
+    attn = s / math.sqrt(hd)
+    if attention_mask is not None:
+        attn = attn.masked_fill(attention_mask[:, None, None, :] == 0, float("-inf"))
+    p = torch.softmax(attn, dim=-1)
+    v = repeat_kv(value_states.to(torch.float64), rep)                                       # [B,N,L,hd]
+    out = torch.matmul(p, v)                                                                 # [B,N,1,hd]
+    mant = 10 if query_states.dtype == torch.float16 else 7
+    half_ulp = torch.exp2(torch.floor(torch.log2(s[..., n_quant:].abs().clamp_min(2.0 ** -14))) - mant - 1)
+    w = (p[..., n_quant:] * half_ulp / math.sqrt(hd)).transpose(2, 3)                        # [B,N,R,1]
+    return (w * (v[:, :, n_quant:] - out).abs()).sum(dim=2, keepdim=True)
 
 
 # --------------------------------------------------------------------------

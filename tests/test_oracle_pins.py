@@ -481,3 +481,35 @@ def test_packed6_layout_known_answer_and_round_trip():
     codes = torch.randint(0, 64, (2, 3, 5, 128, 64), generator=g, dtype=torch.uint8)
     packed = po.pack_codes6(codes)
     assert packed.shape == (2, 3, 5, 128, 48) and torch.equal(po.unpack_codes6(packed), codes)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_residual_score_rounding_band_covers_the_actual_rounding(dtype):
+    """The band is a first-order bound: rounding the window's scores to the model dtype (what the
+    reference's half-precision matmul does, :79) must move the fp64 output by no more than it,
+    and a band with a dropped factor (half of it) must be exceeded somewhere (so the bound is not slack by construction)."""
+    g = torch.Generator().manual_seed(41)
+    B, N, Nk, nb, nr = 2, 8, 2, 1, 37
+    L = nb * 128 + nr
+    k = wl.make_keys(B, Nk, L, 5e5, g, dtype)
+    v = wl.make_half((B, Nk, L, 128), g, dtype)
+    q = wl.make_half((B, N, 1, 128), g, dtype)
+    quant = po.quantize_and_pack_nbit(k[:, :, :nb * 128].contiguous(), 4, 4)
+    kr = k[:, :, nb * 128:]
+    mask = torch.ones(B, L, dtype=torch.int64)
+    mask[1, :140] = 0                                   # sequence 1 attends to 25 window tokens only
+    exact = po.decode_attention_exact(q, kr, *quant, v, mask, 4, 4)
+    band = po.residual_score_rounding_band(q, kr, *quant, v, mask, 4, 4)
+    assert band.shape == exact.shape and bool((band >= 0).all())
+    # the same attention with the window's scores rounded to the dtype
+    kd = torch.cat([po.dequantize_keys(*quant, 4, 4, torch.float64), kr.double()], dim=2)
+    s = torch.matmul(q.double(), po.repeat_kv(kd, N // Nk).transpose(2, 3))
+    s[..., nb * 128:] = s[..., nb * 128:].to(dtype).double()
+    a = (s / math.sqrt(128)).masked_fill(mask[:, None, None, :] == 0, float("-inf"))
+    rounded = torch.matmul(torch.softmax(a, -1), po.repeat_kv(v.double(), N // Nk))
+    moved = (rounded - exact).abs()
+    assert bool((moved <= band * 1.02 + 1e-12).all()), float((moved - band).max())
+    assert bool((moved > band * 0.15).any())           # typical movement is a fair fraction of the worst case
+    # no window, no band
+    z = po.residual_score_rounding_band(q, None, *quant, v[:, :, :nb * 128], None, 4, 4)
+    assert float(z.abs().max()) == 0.0
