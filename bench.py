@@ -28,7 +28,7 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # HBM bytes per launch of the dominant kernel at this workload, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
 # read for a copy kernel of known size; see profiles/attn_kernel_cfg1_pmc.md.
-MEASURED_TRAFFIC_BYTES = int(676933 * 2.0 * 1024 + 2176 * 1.0 * 1024)
+MEASURED_TRAFFIC_BYTES = int(669602 * 2.0 * 1024 + 2176 * 1.0 * 1024)
 
 
 def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):
