@@ -56,7 +56,7 @@ SIGNATURES = {
     "pq_validate_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                             c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                             c_void_p, c_int64, c_float]
-                                   + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
+                                   + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint]),
     "pq_rope_append": (c_int, [c_void_p] * 5 + [c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                                c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
     "pq_rmsnorm": (c_int, [c_void_p] * 5 + [c_int, c_int, c_float, c_int, c_void_p]),

@@ -358,8 +358,13 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
         int gps = (nb + n_splits - 1) / n_splits;
         gps = gps < min_gps ? min_gps : gps;
         if (split > 0 && split * gps >= nb) {
-            if (lane < rep)
-                ws[((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats] = -INFINITY;
+            if (lane < rep) {
+                // both header words: the workspace is not cleared between calls, and the merge must not
+                // meet a stale probability sum (0 * NaN) in a slice that holds nothing
+                float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats;
+                pw[0] = -INFINITY;
+                pw[1] = 0.0f;
+            }
             return;
         }
     }
@@ -606,7 +611,8 @@ __global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __rest
             const float m = p[static_cast<size_t>(s0 + s) * kPartialFloats];
             const float w = (m == -INFINITY) ? 0.0f : exp2f(m - M);
             wgt[s] = w;
-            den = __builtin_fmaf(w, p[static_cast<size_t>(s0 + s) * kPartialFloats + 1], den);
+            // an empty slice contributes nothing, whatever its sum word holds
+            den = w != 0.0f ? __builtin_fmaf(w, p[static_cast<size_t>(s0 + s) * kPartialFloats + 1], den) : den;
         }
         __syncthreads();
         const float* pa = p + static_cast<size_t>(s0) * kPartialFloats + 4 + d;
