@@ -250,7 +250,7 @@ def main():
         def stream_once():
             v = sets[turn[0] & 1]["v"]
             turn[0] += 1
-            got[0] = lib.pq_stream_read(v.data_ptr(), v.numel() * 2, n_waves, sink.data_ptr(), _stream_ptr(dev))
+            got[0] = _ffi.bench_lib().pq_stream_read(v.data_ptr(), v.numel() * 2, n_waves, sink.data_ptr(), _stream_ptr(dev))
             assert got[0] > 0
         s_ms = time_events(stream_once, 20, 4)
         stream_gbps = max(stream_gbps, got[0] / (s_ms * 1e-3) / 1e9)
@@ -262,7 +262,7 @@ def main():
     def replica_once():
         x = sets[turn[0] & 1]
         turn[0] += 1
-        replica[0] = lib.pq_attn_load_replica(x["codes"].data_ptr(), x["v"].data_ptr(), B * Nk, x["codes"].shape[2] * 128,
+        replica[0] = _ffi.bench_lib().pq_attn_load_replica(x["codes"].data_ptr(), x["v"].data_ptr(), B * Nk, x["codes"].shape[2] * 128,
                                               x["v"].shape[2], n_tok, n_splits, sink.data_ptr(), _stream_ptr(dev))
         assert replica[0] > 0
     replica_once()

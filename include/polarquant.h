@@ -34,6 +34,8 @@ extern "C" {
 #define PQ_GROUP 128
 #define PQ_MAX_REP 8          /* query heads per KV head (GQA ratio) supported by the kernels */
 #define PQ_PARTIAL_FLOATS 132 /* floats per split-K partial: m, l, 2 pad, acc[128] */
+#define PQ_MAX_PLANE_TOKENS 16776960 /* 2^24 - 256: most value rows (v_capacity, v4_capacity) or residual
+                                        keys (resid_capacity) of one (batch, KV head) plane */
 
 typedef enum {
     PQ_OK = 0,
@@ -94,24 +96,6 @@ int pq_validate_qkv_rope_append(const void *x, int64_t x_row_stride, const void 
                                 int dtype, const void *cos_table, const void *sin_table, int64_t table_rows,
                                 const int64_t *pos, const void *q_out, const void *k_dst, int64_t k_rows,
                                 const int64_t *k_row, const void *v_dst, int64_t v_rows, const int64_t *v_row, int N, int Nk);
-
-/* Measurement aid (no reference counterpart): a plain streaming read of `bytes` bytes at `src` by
- * `n_wavefronts` wavefronts, each reading one contiguous slice with 16 KiB in flight, with the
- * non-temporal loads the decode kernels use.  Time it to learn what a read-once kernel can be
- * delivered on the GPU at hand.  Returns the number of bytes the launch reads (slices are whole
- * multiples of 16 KiB, so slightly fewer than `bytes`), 0 on a bad argument or a failed launch.
- * `sink`: 4 writable bytes on the device (practically never written). */
-size_t pq_stream_read(const void *src, size_t bytes, int n_wavefronts, uint32_t *sink, void *stream);
-
-/* Measurement aid (no reference counterpart): the HBM reads of pq_decode_attn's main kernel (byte-per-code
- * rows, half-precision values) without its arithmetic: `planes` (batch x KV head) planes of `tokens` tokens,
- * each cut into `n_slices` slices read by one wavefront with the kernel's own loads, order and prefetch depth.
- * codes: `planes` planes of `code_plane_tokens` 64-byte rows; v: `planes` planes of `v_plane_tokens`
- * 256-byte rows.  Returns the bytes one launch reads (320 per token; slices are whole multiples of 128
- * tokens), 0 on a bad argument or a failed launch.  Time it beside the kernel: the difference is what the
- * kernel's table, score and softmax work costs on top of its memory access. */
-size_t pq_attn_load_replica(const uint8_t *codes, const void *v, int planes, int64_t code_plane_tokens,
-                            int64_t v_plane_tokens, int64_t tokens, int n_slices, uint32_t *sink, void *stream);
 
 /* Layout converter for code rows: pack != 0 turns `n_rows` byte-per-code rows (64 bytes each, every
  * code < 64) into packed 6-bit rows (48 bytes each), pack == 0 the reverse.  For caches built by the
@@ -227,8 +211,8 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
  *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48)
- * Limits: v_capacity <= 2^24 tokens and group_capacity <= 2^17 groups per (batch, KV head)
- * plane (32-bit byte offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
+ * Limits: v_capacity <= PQ_MAX_PLANE_TOKENS tokens and group_capacity <= 2^17 groups per (batch, KV head)
+ * plane (32-bit byte sizes and offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */
 int pq_decode_attn(const void *q,
                    const uint8_t *codes, const void *rscale, const void *rmn,

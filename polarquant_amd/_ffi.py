@@ -69,12 +69,18 @@ SIGNATURES = {
                                    c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "pq_validate_qkv_rope_append": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int64,
                                             c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int]),
-    "pq_stream_read": (c_size_t, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
-    "pq_attn_load_replica": (c_size_t, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
     "pq_convert_codes6": (c_int, [c_void_p, c_void_p, c_size_t, c_int, c_void_p]),
     "pq_decode_attn_plan": (c_int, [c_int] * 4),
     "pq_decode_attn_v4_plan": (c_int, [c_int] * 5),
     "pq_decode_attn_workspace_bytes": (c_size_t, [c_int] * 3),
+}
+
+
+# the bench-only library (include/polarquant_bench.h): measurement aids, loaded by bench.py and its tests
+BENCH_LIB_PATH = os.path.join(HERE, "libpolarquant_bench.so")
+BENCH_SIGNATURES = {
+    "pq_stream_read": (c_size_t, [c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
+    "pq_attn_load_replica": (c_size_t, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p]),
 }
 
 
@@ -107,6 +113,24 @@ def lib() -> ctypes.CDLL:
             fn.argtypes = args
         _LIB = handle
     return _LIB
+
+
+_BENCH_LIB = None
+
+
+def bench_lib() -> ctypes.CDLL:
+    """The measurement-aid library.  Raises if it has not been built."""
+    global _BENCH_LIB
+    if _BENCH_LIB is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise RuntimeError("polarquant_amd: %s is missing; build it with `python -m polarquant_amd.build`" % BENCH_LIB_PATH)
+        handle = ctypes.CDLL(BENCH_LIB_PATH)
+        for name, (res, args) in BENCH_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _BENCH_LIB = handle
+    return _BENCH_LIB
 
 
 def check(status: int, where: str) -> None:

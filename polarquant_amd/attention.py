@@ -26,15 +26,39 @@ def plan_splits(B: int, Nk: int, max_groups: int, device: torch.device) -> int:
     return _ffi.lib().pq_decode_attn_plan(B, Nk, max(max_groups, 1), _num_cus(device))
 
 
+def workspace_bytes(B: int, N: int, n_splits: int) -> int:
+    return _ffi.lib().pq_decode_attn_workspace_bytes(B, N, n_splits)
+
+
+def new_workspace(B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
+    """An fp32 workspace for the split-K partials that the caller owns (pass it as `workspace=`).
+    A caller that records the attention call into a HIP graph must own its workspace: the graph keeps
+    the buffer's address, not a reference to the tensor."""
+    return torch.empty((workspace_bytes(B, N, n_splits) + 3) // 4, dtype=torch.float32, device=device)
+
+
 def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
-    """A cached fp32 workspace for the split-K partials (grown on demand, one per device)."""
-    need = _ffi.lib().pq_decode_attn_workspace_bytes(B, N, n_splits)
-    key = (device.type, device.index)
+    """The cached workspace of eager calls: one per (device, stream), grown on demand.  Calls on one
+    stream are ordered, so they can share it; calls on different streams get different buffers.  A
+    replaced buffer goes back to torch's allocator, which hands it out again only behind the work
+    already queued on that stream."""
+    need = workspace_bytes(B, N, n_splits)
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _WORKSPACES.get(key)
     if ws is None or ws.numel() * 4 < need:
         ws = torch.empty((need + 3) // 4, dtype=torch.float32, device=device)
         _WORKSPACES[key] = ws
     return ws
+
+
+def _pick_workspace(workspace: Optional[torch.Tensor], B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
+    if workspace is None:
+        return workspace_for(B, N, n_splits, device)
+    if (workspace.dtype != torch.float32 or workspace.device != device or not workspace.is_contiguous()
+            or workspace.numel() * 4 < workspace_bytes(B, N, n_splits)):
+        raise ValueError("polarquant_amd: workspace must be a contiguous fp32 tensor on %s with at least %d bytes"
+                         % (device, workspace_bytes(B, N, n_splits)))
+    return workspace
 
 
 def polar_decode_attention(
@@ -50,13 +74,16 @@ def polar_decode_attention(
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
     total_groups: Optional[int] = None, min_groups_per_split: Optional[int] = None,
+    workspace: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """-> attention output [B,N,1,128] in the query dtype.
 
     Ragged batches (`n_groups_per_seq` given): `total_groups`, the sum of the per-sequence group
     counts if the caller knows it on the host (no device sync is made here), lets the context be
     cut into slices of equal size across sequences, so that short sequences do not leave
-    wavefronts idle; without it the average sequence is assumed to be half the capacity."""
+    wavefronts idle; without it the average sequence is assumed to be half the capacity.
+    `workspace`: a buffer from `new_workspace` that the caller owns (needed under graph capture);
+    by default the cached buffer of the current stream is used."""
     if not query_states.is_cuda:
         raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
     dev = query_states.device
@@ -102,7 +129,7 @@ def polar_decode_attention(
         min_gps = min_groups_per_split
     if n_splits is None:
         n_splits = plan_splits(B, Nk, max_groups, dev)
-    ws = workspace_for(B, N, n_splits, dev)
+    ws = _pick_workspace(workspace, B, N, n_splits, dev)
     if out is None:
         out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
     gps = n_groups_per_seq.data_ptr() if n_groups_per_seq is not None else None
@@ -129,6 +156,7 @@ def polar_decode_attention_v4(
     rbits: int = 4, tbits: int = 4, sm_scale: Optional[float] = None,
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None, min_groups_per_split: int = 0,
+    workspace: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Decode attention of the reference's Mixed variant (polar keys + 4-bit values,
     models/modeling_llama_polar.py:185-241) -> [B,N,1,128] in the query dtype."""
@@ -166,7 +194,7 @@ def polar_decode_attention_v4(
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
     if n_splits is None:
         n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, N, Nk, max(max_groups, 1), _num_cus(dev))
-    ws = workspace_for(B, N, n_splits, dev)
+    ws = _pick_workspace(workspace, B, N, n_splits, dev)
     if out is None:
         out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
     gps = n_groups_per_seq.data_ptr() if n_groups_per_seq is not None else None

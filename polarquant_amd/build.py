@@ -1,6 +1,6 @@
 """Build recipe of the HIP library: hipcc for gfx950, in-tree.
 
-    python -m polarquant_amd.build            # (re)build polarquant_amd/libpolarquant_hip.so
+    python -m polarquant_amd.build            # (re)build polarquant_amd/libpolarquant_hip.so and libpolarquant_bench.so
 
 hipcc cross-compiles without a GPU.  Flags that matter:
   -ffp-contract=off            the quantizer reproduces eager half-precision torch
@@ -18,7 +18,11 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libpolarquant_hip.so")
-SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_stream.hip", "pq_attn.hip"]
+SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_attn.hip"]
+# measurement aids (a plain streaming read, the attention kernel's loads without its arithmetic): a library of
+# their own, loaded by bench.py and its tests only
+BENCH_LIB = os.path.join(HERE, "libpolarquant_bench.so")
+BENCH_SOURCES = ["pq_stream.hip"]
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
@@ -46,6 +50,15 @@ def _compile(src: str, defines=(), tag: str = "") -> str:
     return obj
 
 
+def _link(objs, lib: str) -> None:
+    tmp = lib + ".tmp"
+    r = subprocess.run([_hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + list(objs),
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    os.replace(tmp, lib)
+
+
 def build(verbose: bool = True, phase_timers: bool = False) -> str:
     """The library the package loads; or, with phase_timers, a second library (same ABI, not loaded by default)
     whose attention kernel times its phases with the wall clock and prints them: a measuring build for
@@ -55,12 +68,11 @@ def build(verbose: bool = True, phase_timers: bool = False) -> str:
     lib, defines, tag = (TIMERS_LIB, ("PQ_ATTN_PHASE_TIMERS",), ".timers") if phase_timers else (LIB, (), "")
     with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
         objs = list(ex.map(lambda s_: _compile(s_, defines, tag), srcs))
-    tmp = lib + ".tmp"
-    r = subprocess.run([_hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs,
-                       capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n" + r.stderr)
-    os.replace(tmp, lib)
+    _link(objs, lib)
+    if not phase_timers:
+        _link([_compile(s_) for s_ in BENCH_SOURCES], BENCH_LIB)
+        if verbose:
+            print("built", BENCH_LIB)
     if verbose:
         print("built", lib)
     return lib

@@ -88,7 +88,8 @@ int pq_validate_quantize_groups(const void* k, const int64_t* k_strides, int dty
     if (!k || !k_strides || !codes || !rscale || !rmn || !tscale || !tmn) return PQ_ERR_NULL_POINTER;
     if (B <= 0 || Nk <= 0 || Nb <= 0 || Nb > 65535 * 32 || static_cast<long long>(B) * Nk > 65535)
         return PQ_ERR_BAD_SHAPE;
-    if (rbits < 1 || tbits < 1 || rbits + tbits > 8) return PQ_ERR_BAD_BITS;
+    // the same bit widths as the decode entry points: no cache is written that nothing here can read
+    if (int rc = check_bits(rbits, tbits)) return rc;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
     if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM | PQ_CODES_PACKED6)) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && rbits + tbits > 6) return PQ_ERR_BAD_BITS;
@@ -166,9 +167,12 @@ int pq_validate_decode_attn(const void* q,
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
     if (group_capacity < 0 || resid_capacity < 0 || n_groups < 0 || n_resid < 0 || v_capacity <= 0)
         return PQ_ERR_BAD_STRIDE;
-    // the kernels address one (batch, KV head) plane with 32-bit byte offsets: at most 2^24 tokens
-    // of 256-byte value rows (and 2^17 groups of 8 KiB of codes) per plane
-    if (v_capacity > (int64_t{1} << 24) || group_capacity > (1 << 17) || resid_capacity > (1 << 24)) return PQ_ERR_BAD_SHAPE;
+    // the kernels address one (batch, KV head) plane through a buffer resource with a 32-bit size and
+    // 32-bit byte offsets, and park loads that must read nothing at offset 0xFFFF0000, which therefore
+    // has to lie past the end of every plane: at most PQ_MAX_PLANE_TOKENS (2^24 - 256) rows of 256 bytes
+    // of values or residual keys, and 2^17 groups of 8 KiB of codes
+    if (v_capacity > PQ_MAX_PLANE_TOKENS || group_capacity > (1 << 17) || resid_capacity > PQ_MAX_PLANE_TOKENS)
+        return PQ_ERR_BAD_SHAPE;
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     if (any_groups && (!codes || !rscale || !rmn || !tscale || !tmn)) return PQ_ERR_NULL_POINTER;
     const bool any_resid = n_resid_per_seq ? resid_capacity > 0 : n_resid > 0;
@@ -345,31 +349,6 @@ int pq_linear_small_m(const void* x, int64_t x_row_stride, const void* w, const 
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
 }
 
-size_t pq_stream_read(const void* src, size_t bytes, int n_wavefronts, uint32_t* sink, void* stream) {
-    if (!src || !sink || n_wavefronts <= 0 || n_wavefronts > (1 << 20) || !aligned(src, 16) || !aligned(sink, 4)) return 0;
-    const size_t chunk = 16 * 1024;                       // what one wavefront requests per trip
-    size_t per_wave = bytes / static_cast<size_t>(n_wavefronts) / chunk * chunk;
-    if (per_wave > (size_t{1} << 31) - chunk) per_wave = ((size_t{1} << 31) - chunk) / chunk * chunk;
-    if (per_wave == 0) return 0;
-    if (pq::launch_stream_read(src, per_wave, n_wavefronts, sink, static_cast<hipStream_t>(stream)) != 0) return 0;
-    return per_wave * static_cast<size_t>(n_wavefronts);
-}
-
-size_t pq_attn_load_replica(const uint8_t* codes, const void* v, int planes, int64_t code_plane_tokens,
-                            int64_t v_plane_tokens, int64_t tokens, int n_slices, uint32_t* sink, void* stream) {
-    if (!codes || !v || !sink || !aligned(codes, 16) || !aligned(v, 16) || !aligned(sink, 4)) return 0;
-    if (planes <= 0 || n_slices <= 0 || static_cast<long long>(planes) * n_slices > (1ll << 24)) return 0;
-    if (tokens <= 0 || tokens > code_plane_tokens || tokens > v_plane_tokens) return 0;
-    if (v_plane_tokens > ((int64_t{1} << 31) - 1) / 256 || code_plane_tokens > ((int64_t{1} << 31) - 1) / 64) return 0;
-    const int64_t per_slice = tokens / n_slices / 128 * 128;          // whole pairs of 64-token tiles
-    if (per_slice == 0) return 0;
-    if (pq::launch_attn_load_replica(codes, v, planes, static_cast<uint32_t>(code_plane_tokens),
-                                     static_cast<uint32_t>(v_plane_tokens), static_cast<uint32_t>(per_slice), n_slices, sink,
-                                     static_cast<hipStream_t>(stream)) != 0)
-        return 0;
-    return static_cast<size_t>(per_slice) * n_slices * static_cast<size_t>(planes) * 320;
-}
-
 int pq_validate_qkv_rope_append(const void* x, int64_t x_row_stride, const void* w_qkv, const void* bias, int M, int K,
                                 int dtype, const void* cos_table, const void* sin_table, int64_t table_rows,
                                 const int64_t* pos, const void* q_out, const void* k_dst, int64_t k_rows,
@@ -459,7 +438,9 @@ int pq_validate_decode_attn_v4(const void* q,
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     if (any_groups && (!v_codes || !v_scale || !v_zero)) return PQ_ERR_NULL_POINTER;
     if (v4_capacity < 0) return PQ_ERR_BAD_STRIDE;
-    if (v4_capacity > (int64_t{1} << 24)) return PQ_ERR_BAD_SHAPE;          // 32-bit byte offsets inside a plane
+    // (only whole groups of the 4-bit planes are read, at most group_capacity <= 2^17 of them, so their
+    // 32-bit sizes cannot wrap; the limit keeps the two value entry points alike)
+    if (v4_capacity > PQ_MAX_PLANE_TOKENS) return PQ_ERR_BAD_SHAPE;
     if (!n_groups_per_seq && static_cast<int64_t>(n_groups) * PQ_GROUP > v4_capacity) return PQ_ERR_BAD_STRIDE;
     if ((v_codes && !aligned(v_codes, 4)) || (v_resid && !aligned(v_resid, 16))) return PQ_ERR_MISALIGNED;
     // everything else as in the fp16-value entry point; its V-capacity rule is met by construction here

@@ -35,10 +35,6 @@ int launch_convert_codes6(const uint8_t* src, uint8_t* dst, size_t n_rows, bool 
 int launch_small_m_linear(const void* x, int64_t x_stride, const void* w, const void* w_up, const void* bias, void* y,
                           int64_t y_stride, int M, int N, int K, int dtype, hipStream_t st);
 
-int launch_attn_load_replica(const void* codes, const void* v, int planes, uint32_t code_plane_tokens,
-                             uint32_t v_plane_tokens, uint32_t tokens_per_slice, int n_slices, uint32_t* sink, hipStream_t st);
-int launch_stream_read(const void* src, size_t bytes_per_wave, int n_waves, uint32_t* sink, hipStream_t st);
-
 int launch_qkv_rope_append(const void* x, int64_t x_stride, const void* w, const void* bias, int M, int K, int dtype,
                            const void* cos_tab, const void* sin_tab, int64_t max_pos, const int64_t* pos, void* q_out,
                            void* k_dst, int64_t k_rows, const int64_t* k_row, void* v_dst, int64_t v_rows,

@@ -1,10 +1,14 @@
+// The bench-only library (libpolarquant_bench.so, declared in include/polarquant_bench.h): kernels that
+// measure what the memory system delivers, for bench.py and the profiles.  Not part of the product
+// library and not needed by any caller of the decode path.
+//
 // Measurement aid: a plain streaming read of a device buffer, the access pattern every kernel of
 // this library is compared against.  Each wavefront owns one contiguous slice and keeps 16 loads
 // of 16 bytes per lane in flight (16 KiB per wavefront), with the same non-temporal buffer loads
 // the decode kernels use for their code and value streams.  What it reaches on a given GPU is
 // the bandwidth a read-once kernel can be delivered there; the published HBM peak is not.
+#include "../../include/polarquant_bench.h"
 #include "pq_device.h"
-#include "pq_internal.h"
 
 namespace pq {
 
@@ -97,3 +101,36 @@ int launch_stream_read(const void* src, size_t bytes_per_wave, int n_waves, uint
 }
 
 }  // namespace pq
+
+namespace {
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+}  // namespace
+
+extern "C" {
+
+size_t pq_stream_read(const void* src, size_t bytes, int n_wavefronts, uint32_t* sink, void* stream) {
+    if (!src || !sink || n_wavefronts <= 0 || n_wavefronts > (1 << 20) || !aligned(src, 16) || !aligned(sink, 4)) return 0;
+    const size_t chunk = 16 * 1024;                       // what one wavefront requests per trip
+    size_t per_wave = bytes / static_cast<size_t>(n_wavefronts) / chunk * chunk;
+    if (per_wave > (size_t{1} << 31) - chunk) per_wave = ((size_t{1} << 31) - chunk) / chunk * chunk;
+    if (per_wave == 0) return 0;
+    if (pq::launch_stream_read(src, per_wave, n_wavefronts, sink, static_cast<hipStream_t>(stream)) != 0) return 0;
+    return per_wave * static_cast<size_t>(n_wavefronts);
+}
+
+size_t pq_attn_load_replica(const uint8_t* codes, const void* v, int planes, int64_t code_plane_tokens,
+                            int64_t v_plane_tokens, int64_t tokens, int n_slices, uint32_t* sink, void* stream) {
+    if (!codes || !v || !sink || !aligned(codes, 16) || !aligned(v, 16) || !aligned(sink, 4)) return 0;
+    if (planes <= 0 || n_slices <= 0 || static_cast<long long>(planes) * n_slices > (1ll << 24)) return 0;
+    if (tokens <= 0 || tokens > code_plane_tokens || tokens > v_plane_tokens) return 0;
+    if (v_plane_tokens > ((int64_t{1} << 31) - 1) / 256 || code_plane_tokens > ((int64_t{1} << 31) - 1) / 64) return 0;
+    const int64_t per_slice = tokens / n_slices / 128 * 128;          // whole pairs of 64-token tiles
+    if (per_slice == 0) return 0;
+    if (pq::launch_attn_load_replica(codes, v, planes, static_cast<uint32_t>(code_plane_tokens),
+                                     static_cast<uint32_t>(v_plane_tokens), static_cast<uint32_t>(per_slice), n_slices, sink,
+                                     static_cast<hipStream_t>(stream)) != 0)
+        return 0;
+    return static_cast<size_t>(per_slice) * n_slices * static_cast<size_t>(planes) * 320;
+}
+
+}  // extern "C"

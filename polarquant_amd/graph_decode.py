@@ -23,7 +23,7 @@ from typing import List, Optional
 import torch
 
 from . import _ffi
-from .attention import _num_cus, plan_splits, polar_decode_attention, polar_decode_attention_v4, workspace_for
+from .attention import _num_cus, new_workspace, plan_splits, polar_decode_attention, polar_decode_attention_v4
 from .modeling_common import GROUP, apply_rotary_pos_emb
 
 
@@ -99,7 +99,8 @@ class PolarGraphDecoder:
             self.n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, cfg.num_attention_heads, nk, max(self.max_len // GROUP, 1), _num_cus(dev))
         else:
             self.n_splits = plan_splits(B, nk, max(self.max_len // GROUP, 1), dev)
-        workspace_for(B, cfg.num_attention_heads, self.n_splits, dev)                     # allocate before capture
+        # the captured graph keeps this buffer's address: the decoder owns it, so that no other call can replace it
+        self.workspace = new_workspace(B, cfg.num_attention_heads, self.n_splits, dev)
         self.logits = None
         self.graph = None
         if self.fused_ops:
@@ -163,7 +164,7 @@ class PolarGraphDecoder:
     def _attend(self, att, ar, q):
         common = dict(rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
                       n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits,
-                      attention_mask=self.mask8)
+                      attention_mask=self.mask8, workspace=self.workspace)
         if self.mixed:
             return polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0, **common)
         return polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, **common)
@@ -237,12 +238,13 @@ class PolarGraphDecoder:
                 o = polar_decode_attention_v4(q, ar.codes, *ar.meta, ar.kres, ar.vres, ar.vcodes, *ar.vmeta, 0, 0,
                                               rbits=att.rbits, tbits=att.tbits, sm_scale=1.0 / math.sqrt(att.head_dim),
                                               n_groups_per_seq=self.n_groups_dev, n_resid_per_seq=self.n_resid_dev,
-                                              n_splits=self.n_splits, attention_mask=self.mask8)
+                                              n_splits=self.n_splits, attention_mask=self.mask8, workspace=self.workspace)
             else:
                 ar.v.index_copy_(2, self.pos, v)
                 o = polar_decode_attention(q, ar.codes, *ar.meta, ar.kres, ar.v, 0, 0, rbits=att.rbits, tbits=att.tbits,
                                            sm_scale=1.0 / math.sqrt(att.head_dim), n_groups_per_seq=self.n_groups_dev,
-                                           n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits, attention_mask=self.mask8)
+                                           n_resid_per_seq=self.n_resid_dev, n_splits=self.n_splits, attention_mask=self.mask8,
+                                           workspace=self.workspace)
             x = x + att.o_proj(o.reshape(B, 1, -1))
             x = x + layer.mlp(layer.post_attention_layernorm(x))
         logits = model.lm_head(model.model.norm(x))

@@ -249,18 +249,22 @@ class PolarCache(tuple):
         return obj
 
 
-_MASK_CACHE = {"key": None, "u8": None}
+_MASK_CACHE = {"src": None, "version": -1, "u8": None}
 
 
 def _mask_u8(mask: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
-    """attention_mask [B, L] of {0,1} (any dtype) -> uint8, converted once per step, not once per layer."""
+    """attention_mask [B, L] of {0,1} (any dtype) -> uint8, converted once per step, not once per layer.
+
+    The cache entry is recognised by the identity of the mask tensor (and its version counter), and it
+    keeps that tensor alive: an address can then not be handed to a different mask while the entry
+    exists, which a key made of the address alone would not notice."""
     if mask is None:
         return None
     if mask.dtype == torch.uint8:
         return mask
-    key = (mask.data_ptr(), tuple(mask.shape), mask._version, mask.dtype)
-    if _MASK_CACHE["key"] != key:
-        _MASK_CACHE["key"], _MASK_CACHE["u8"] = key, (mask != 0).to(torch.uint8)
+    if _MASK_CACHE["src"] is not mask or _MASK_CACHE["version"] != mask._version:
+        _MASK_CACHE["u8"] = (mask != 0).to(torch.uint8)
+        _MASK_CACHE["src"], _MASK_CACHE["version"] = mask, mask._version
     return _MASK_CACHE["u8"]
 
 

@@ -26,7 +26,7 @@ def _close(got, ref, rtol=RTOL, atol=ATOL):
 
 
 def _case(gpu, B, N, Nk, n_groups, n_resid, rbits, tbits, dtype, theta=5e5, mask_pad=0, seed=0, n_splits=None,
-          caps=(0, 0, 0)):
+          caps=(0, 0, 0), workspace=None):
     g = torch.Generator().manual_seed(seed)
     L = n_groups * 128 + n_resid
     k = wl.make_keys(B, Nk, max(L, 1), theta, g, dtype)
@@ -61,7 +61,7 @@ def _case(gpu, B, N, Nk, n_groups, n_resid, rbits, tbits, dtype, theta=5e5, mask
         dv[:, :, L:] = float("nan")     # rows past the end must never contribute
     out = polar_decode_attention(q.to(gpu), *dq, dk, dv, n_groups, n_resid,
                                  attention_mask=None if mask is None else mask.to(gpu),
-                                 rbits=rbits, tbits=tbits, n_splits=n_splits)
+                                 rbits=rbits, tbits=tbits, n_splits=n_splits, workspace=workspace)
     torch.cuda.synchronize()
     out = out.cpu()
     assert out.shape == (B, N, 1, 128) and out.dtype == dtype
@@ -104,6 +104,55 @@ def test_attn_many_splits(gpu, n_splits, dtype):
     out, ref, ref64 = _case(gpu, 1, 8, 2, 130, 3, 4, 4, dtype, seed=11, n_splits=n_splits)
     rtol, atol = (RTOL, ATOL) if dtype == torch.float16 else (2e-2, 4e-3)   # bf16 has 8 mantissa bits
     assert _close(out, ref64, rtol, atol)[0] == 0
+
+
+@pytest.mark.parametrize("poison", [float("nan"), float("inf"), -1.0])
+def test_attn_ignores_what_the_workspace_held(gpu, poison):
+    """The workspace is never cleared, and slices past a sequence's last group write only an empty
+    header: whatever bits the buffer held before (NaN, Inf, integer -1 patterns from other tensors
+    that owned the memory) must not reach the output.  More slices than groups, and a ragged batch
+    whose short sequences leave most slices empty, both through a caller-owned and the cached buffer."""
+    from polarquant_amd import attention
+    print("case poison", poison, flush=True)
+    ws = attention.new_workspace(1, 8, 9, gpu)
+    if poison < 0:
+        ws.view(torch.int32).fill_(-1)
+    else:
+        ws.fill_(poison)
+    out, ref, ref64 = _case(gpu, 1, 8, 2, 4, 3, 4, 4, torch.float16, seed=21, n_splits=9, workspace=ws)
+    assert _close(out, ref64)[0] == 0
+    # ragged: sequences of 1 and 5 groups cut into 5 slices; the cached buffer of the current stream is poisoned
+    g = torch.Generator().manual_seed(22)
+    B, N, Nk = 2, 8, 2
+    lens = [1 * 128 + 7, 5 * 128]
+    k = wl.make_keys(B, Nk, max(lens), 5e5, g)
+    q = wl.make_half((B, N, 1, 128), g)
+    v = wl.make_half((B, Nk, max(lens), 128), g)
+    codes = torch.zeros(B, Nk, 5, 128, 64, dtype=torch.uint8)
+    meta = [torch.zeros(B, Nk, 5, 1, 64, dtype=torch.float16) for _ in range(4)]
+    kres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16)
+    refs = []
+    for b, L in enumerate(lens):
+        ng, nr = L // 128, L % 128
+        quant = po.quantize_and_pack_nbit(k[b:b + 1, :, :ng * 128].contiguous())
+        codes[b, :, :ng] = quant[0][0]
+        for m, t in zip(meta, quant[1:]):
+            m[b, :, :ng] = t[0]
+        kr = k[b:b + 1, :, ng * 128:L].contiguous() if nr else None
+        if nr:
+            kres[b, :, :nr] = kr[0]
+        refs.append(po.decode_attention_exact(q[b:b + 1], kr, *quant, v[b:b + 1, :, :L]))
+    cached = attention.workspace_for(B, N, 5, gpu)
+    if poison < 0:
+        cached.view(torch.int32).fill_(-1)
+    else:
+        cached.fill_(poison)
+    out = polar_decode_attention(q.to(gpu), codes.to(gpu), *[m.to(gpu) for m in meta], kres.to(gpu), v.to(gpu), 0, 0,
+                                 n_groups_per_seq=torch.tensor([1, 5], dtype=torch.int32, device=gpu),
+                                 n_resid_per_seq=torch.tensor([7, 0], dtype=torch.int32, device=gpu), n_splits=5)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert _close(out.cpu(), torch.cat(refs, 0))[0] == 0
 
 
 def test_attn_left_padding_mask(gpu):

@@ -18,8 +18,8 @@ def lib():
     return _ffi.lib()
 
 
-def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "polarquant.h")).read()
+def _declared_functions(header="polarquant.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(pq_[a-z0-9_]+)\s*\(", text)))
 
@@ -32,6 +32,12 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
         assert hasattr(raw, n), "libpolarquant_hip.so does not export %s" % n
         assert n in _ffi.SIGNATURES, "%s is declared in the header but has no ctypes signature" % n
     assert set(_ffi.SIGNATURES) == set(names)
+    # the measurement aids live in a library of their own, not in the product ABI
+    bench_names = _declared_functions("polarquant_bench.h")
+    assert bench_names == sorted(_ffi.BENCH_SIGNATURES) and not set(bench_names) & set(names)
+    raw_bench = ctypes.CDLL(_ffi.BENCH_LIB_PATH)
+    for n in bench_names:
+        assert hasattr(raw_bench, n) and not hasattr(raw, n)
 
 
 def test_version_and_status_strings(lib):
@@ -74,6 +80,11 @@ def test_validate_quantize_groups(lib):
     assert bad(0, None) == -1 and bad(1, None) == -1 and bad(9, None) == -1
     assert bad(3, 0) == -2 and bad(5, 0) == -2
     assert bad(6, 5) == -3 and bad(7, 0) == -3
+    # bit widths the decode entry points cannot read are refused by the quantizer too (tbits > 4)
+    a = list(ok); a[6], a[7] = 2, 5
+    assert lib.pq_validate_quantize_groups(*a) == -3
+    a[6], a[7] = 1, 7
+    assert lib.pq_validate_quantize_groups(*a) == -3
     assert bad(2, 7) == -4
     assert bad(8, 1) == 0 and bad(8, 2) == 0 and bad(8, 3) == 0   # PQ_WRAP_FP32, PQ_ANGLE_UNIFORM
     assert bad(8, 4) == -3                           # packed 6-bit codes need rbits + tbits <= 6
@@ -117,6 +128,12 @@ def test_validate_decode_attn_and_plan(lib):
     assert bad(20, 5) == -2 and bad(22, 5) == -3 and bad(23, 3) == -4
     assert bad(13, P + 8) == -5
     assert bad(14, (1 << 24) + 1) == -2 and bad(6, (1 << 17) + 1) == -2      # plane too large for 32-bit offsets
+    # the value plane's byte size is a 32-bit field (2^24 rows of 256 bytes would read as 0 bytes: every value
+    # a silent zero) and the parking offset 0xFFFF0000 of loads that must read nothing has to lie past it
+    max_rows = (1 << 24) - 256
+    assert max_rows * 256 == 0xFFFF0000
+    assert bad(14, max_rows) == 0 and bad(14, max_rows + 1) == -2 and bad(14, 1 << 24) == -2
+    assert bad(10, max_rows) == 0 and bad(10, max_rows + 1) == -2 and bad(10, 1 << 24) == -2
     a = list(ok); a[15] = P; a[16] = 100          # mask row shorter than the context
     assert lib.pq_validate_decode_attn(*a) == -6
     # no quantized groups yet: codes may be NULL
@@ -233,7 +250,8 @@ def test_qkv_rope_append_rejects_bad_arguments(lib):
     assert lib.pq_qkv_rope_append(*(ok[:2] + [None] + ok[3:] + [None])) == -1
 
 
-def test_stream_read_rejects_bad_arguments(lib):
+def test_stream_read_rejects_bad_arguments():
+    lib = _ffi.bench_lib()
     assert lib.pq_stream_read(None, 1 << 30, 1024, P, None) == 0 and lib.pq_stream_read(P, 1 << 30, 1024, None, None) == 0
     assert lib.pq_stream_read(P, 1 << 30, 0, P, None) == 0 and lib.pq_stream_read(P + 8, 1 << 30, 1024, P, None) == 0
     assert lib.pq_stream_read(P, 1000, 1024, P, None) == 0          # less than one 16 KiB trip per wavefront
@@ -255,7 +273,8 @@ def test_rope_qk_rejects_bad_arguments(lib):
     assert bad(0, P + 8) == -5 and bad(4, P + 2) == -5 and bad(8, P + 4) == -5
 
 
-def test_attn_load_replica_rejects_bad_arguments(lib):
+def test_attn_load_replica_rejects_bad_arguments():
+    lib = _ffi.bench_lib()
     ok = [P, P, 128, 32768, 32769, 32768, 8, P]
     def bad(i, v):
         a = list(ok)

@@ -101,7 +101,7 @@ def test_measurement_aids_launch_and_report_their_bytes(gpu):
     leave their inputs and the sink alone."""
     from polarquant_amd import _ffi
     from polarquant_amd.kernel4group import _stream_ptr
-    lib = _ffi.lib()
+    lib = _ffi.bench_lib()
     planes, tokens = 6, 1000
     codes = torch.randint(0, 255, (planes, 1024, 64), dtype=torch.uint8, device=gpu)
     v = torch.randn(planes, tokens + 5, 128, device=gpu).half()

@@ -128,3 +128,31 @@ def test_top_p_keep_mask_matches_the_filter():
     keep = return_top_p_filtered_indices(logits, 0.6)
     filtered = top_k_top_p_filtering(logits.reshape(-1, 19).clone(), top_k=0, top_p=0.6).reshape(2, 3, 19)
     assert torch.equal(keep, torch.isfinite(filtered))
+
+
+def test_padding_mask_conversion_is_not_fooled_by_a_recycled_address():
+    """The uint8 form of the step's attention mask is cached across the layers of one step.  `generate` builds a
+    fresh mask tensor per step, and an allocator hands a freed block of the same size straight back: two masks of
+    the same shape and address with different padding must each get their own conversion."""
+    from polarquant_amd.modeling_common import _mask_u8
+    shape = (4, 333)
+    first = torch.ones(shape, dtype=torch.int64)
+    first[:, :100] = 0
+    u_first = _mask_u8(first)
+    assert torch.equal(u_first, (first != 0).to(torch.uint8))
+    assert _mask_u8(first) is u_first                    # same tensor, same step: converted once
+    addr = first.data_ptr()
+    recycled = 0
+    for pad in (7, 50, 200, 13):
+        del first
+        first = torch.ones(shape, dtype=torch.int64)     # usually lands on the block just freed
+        first[:, :pad] = 0
+        recycled += first.data_ptr() == addr
+        addr = first.data_ptr()
+        assert torch.equal(_mask_u8(first), (first != 0).to(torch.uint8)), pad
+    # an in-place edit of the same tensor is seen through its version counter
+    first[:, :300] = 0
+    assert torch.equal(_mask_u8(first), (first != 0).to(torch.uint8))
+    # a uint8 mask passes through untouched
+    m8 = torch.ones(shape, dtype=torch.uint8)
+    assert _mask_u8(m8) is m8 and _mask_u8(None) is None
