@@ -257,6 +257,26 @@ int pq_decode_attn_partials(const void *q,
 int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
                          void *out, void *stream);
 
+/* pq_decode_attn for callers that cannot allocate device memory and have no workspace to pass:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments, checks and results as pq_decode_attn (the same two
+ * kernels), but the split partials go to a buffer inside the library: a file-scope device array of
+ * PQ_STATIC_MAX_PARTIALS partials (8.25 MiB, held by every GPU the library runs on until the process
+ * ends).  The call allocates and frees nothing.  B * N * n_splits above PQ_STATIC_MAX_PARTIALS is
+ * rejected with PQ_ERR_WORKSPACE.  All calls on one GPU share that buffer: calls that overlap on one
+ * GPU (different streams, several threads) race on it; calls on one stream do not.  The first call
+ * on a device asks the runtime for the array's device address; make that call outside a capture. */
+#define PQ_STATIC_MAX_PARTIALS 16384
+int pq_decode_attn_static(const void *q,
+                          const uint8_t *codes, const void *rscale, const void *rmn,
+                          const void *tscale, const void *tmn, int group_capacity,
+                          int n_groups, const int32_t *n_groups_per_seq,
+                          const void *k_resid, int resid_capacity, int n_resid, const int32_t *n_resid_per_seq,
+                          const void *v, int64_t v_capacity,
+                          const uint8_t *mask, int64_t mask_stride,
+                          float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                          int n_splits, int min_groups_per_split, void *out, unsigned flags, void *stream);
+
 /* ---------------------------------------------------------------------------
  * 4-bit values: the reference's Mixed variant (LlamaPolarMixedGroupAttention,
  * models/modeling_llama_polar.py:158-292).

@@ -38,6 +38,9 @@ SIGNATURES = {
     "pq_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_int64, c_void_p, c_int64, c_float]
                        + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p]),
+    "pq_decode_attn_static": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                                                       c_void_p, c_int64, c_void_p, c_int64, c_float]
+                              + [c_int] * 8 + [c_void_p, c_uint, c_void_p]),
     "pq_validate_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
                                 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint]),

@@ -28,6 +28,7 @@
 // partials (m, l, acc[128]) of a query head and writes half words.
 #include "pq_device.h"
 #include "pq_internal.h"
+#include <mutex>
 
 // Measuring build only (-DPQ_ATTN_PHASE_TIMERS, `python -m polarquant_amd.build --phase-timers`): wall-clock
 // (100 MHz) time of each phase of the group loop, summed per wavefront and printed by a few of them.
@@ -727,6 +728,31 @@ int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, vo
         hipLaunchKernelGGL((merge_kernel<BF16, 1>), dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
     }
     return static_cast<int>(hipGetLastError());
+}
+
+// ---- scratch of the entry point that allocates nothing (pq_decode_attn_static) -----------------
+// The split partials of that entry point live in this file-scope device array instead of a caller's
+// workspace.  Every GPU the library runs on holds its own copy at its own address until the process
+// ends; the array's name is only a host-side handle, so the device address is asked for once per
+// device (with that device current) and kept.
+static __device__ __align__(256) float scratch[static_cast<size_t>(kStaticMaxPartials) * kPartialFloats];
+
+int attn_static_scratch(float** ptr) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static float* per_device[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!p) return static_cast<int>(hipErrorInvalidSymbol);
+        per_device[dev] = static_cast<float*>(p);
+    }
+    *ptr = per_device[dev];
+    return 0;
 }
 
 }  // namespace pq

@@ -255,6 +255,28 @@ int pq_decode_attn(const void* q,
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
 
+int pq_decode_attn_static(const void* q,
+                          const uint8_t* codes, const void* rscale, const void* rmn,
+                          const void* tscale, const void* tmn, int group_capacity,
+                          int n_groups, const int32_t* n_groups_per_seq,
+                          const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                          const void* v, int64_t v_capacity,
+                          const uint8_t* mask, int64_t mask_stride,
+                          float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                          int n_splits, int min_groups_per_split, void* out, unsigned flags, void* stream) {
+    static_assert(PQ_STATIC_MAX_PARTIALS == pq::kStaticMaxPartials, "header and library disagree");
+    if (B <= 0 || N <= 0 || n_splits < 1) return PQ_ERR_BAD_SHAPE;
+    if (static_cast<long long>(B) * N * n_splits > PQ_STATIC_MAX_PARTIALS) return PQ_ERR_WORKSPACE;
+    float* ws = nullptr;
+    if (pq::attn_static_scratch(&ws) != 0) return PQ_ERR_NO_DEVICE;
+    // every (query head, slice) partial header is rewritten by each call and the merge skips the
+    // body of an empty one, so nothing of the previous call's contents needs clearing
+    return pq_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq, k_resid,
+                          resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask, mask_stride, sm_scale, B, N, Nk,
+                          rbits, tbits, dtype, n_splits, min_groups_per_split, ws,
+                          static_cast<size_t>(PQ_STATIC_MAX_PARTIALS) * PQ_PARTIAL_FLOATS * sizeof(float), out, flags, stream);
+}
+
 // ---- fused elementwise steps of the decode layer -----------------------------------------------
 int pq_rope_append(const void* q_lin, const void* k_lin, const void* v_lin, const void* cos_table, const void* sin_table,
                    int64_t table_rows, const int64_t* pos, void* q_out, void* k_dst, int64_t k_rows, const int64_t* k_row,

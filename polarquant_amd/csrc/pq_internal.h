@@ -65,6 +65,11 @@ struct AttnArgs {
 int launch_attn_partials(const AttnArgs& a, hipStream_t st);
 int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st);
 
+// Device address, on the current device, of the library's own buffer for split partials
+// (kStaticMaxPartials partials of 132 floats); 0 or a hipError_t.
+constexpr int kStaticMaxPartials = 16384;
+int attn_static_scratch(float** ptr);
+
 inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 : 8; }
 
 }  // namespace pq
