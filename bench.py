@@ -29,6 +29,7 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
 # read for a copy kernel of known size; see profiles/attn_kernel_cfg1_pmc.md.
 MEASURED_TRAFFIC_BYTES = int(669602 * 2.0 * 1024 + 2176 * 1.0 * 1024)
+TRAFFIC_SOURCE = "constant, not read in this run: rocprofv3 --pmc runs of 2026-11-25 at commit 0b769ba (profiles/attn_kernel_cfg1_pmc.md)"
 
 
 def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):
@@ -46,45 +47,76 @@ def time_events(fn, steps, warmup):
     return wl.time_events(fn, steps, warmup)
 
 
-def kernel_duration_ms(launch, steps):
-    """Average duration of one launch, each launch bracketed by its own pair of
-    events on the launching stream."""
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+def kernel_duration_ms(launch, steps, warmup=4):
+    """Average duration of one launch in a back-to-back series of `steps` launches between one pair
+    of events on the launching stream."""
+    return time_events(launch, steps, warmup)
+
+
+def bracketed_step_ms(first, second, steps, warmup=4):
+    """A second timed region of `steps` steps in which the step's two launches are issued separately
+    (`first`, then `second`: the same kernels, stream and order as the fused call) with an event before,
+    between and after them.  -> (ms per step over the region, mean ms of `first`, mean ms of `second`).
+    All three come from the same events, so first + second <= step by construction; the gap between a
+    step's end and the next step's start belongs to neither kernel."""
+    for _ in range(warmup):
+        first()
+        second()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
     torch.cuda.synchronize()
-    for a, b in evs:
+    for a, b, c in evs:
         a.record()
-        launch()
+        first()
         b.record()
+        second()
+        c.record()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in evs) / steps
+    k = sum(a.elapsed_time(b) for a, b, _ in evs) / steps
+    m = sum(b.elapsed_time(c) for _, b, c in evs) / steps
+    return evs[0][0].elapsed_time(evs[-1][2]) / steps, k, m
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(w):
     """The reference path on the host cores: dequantize-then-matmul scores, /sqrt(d),
     fp32 softmax, P.V (oracle restatement of modeling_llama_polar.py:66-99 and
-    kernel4group.py:151-155), on one of the 16 sequences, scaled to the batch."""
+    kernel4group.py:151-155), on every sequence of the batch in turn (a loop over batch
+    elements, summed): the median of three runs per sequence."""
     from oracle import polar_oracle as po
     sh = w["shape"]
-    b = 0
-    cq = w["q"][b:b + 1].cpu()
-    quant = [w["codes"][b:b + 1].cpu()] + [m[b:b + 1].cpu() for m in w["meta"]]
-    kres = w["kres"][b:b + 1, :, :w["n_resid"]].cpu()
-    v = w["v"][b:b + 1].cpu()
     threads = torch.get_num_threads()
-    po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)        # warm-up
-    times = []
-    t_all = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 20):
-        t0 = time.perf_counter()
-        ref = po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
-    return ref, {
-        "value": round(med * sh.batch * 1e6, 1), "unit": "us/step", "cores": threads, "kind": "port",
-        "sample": "sequence 0 of %d (8 KV heads x 32768 tokens), median of %d runs of the torch-CPU restatement "
-                  "of the reference path (dequantize, matmul, softmax, P.V), scaled x%d to the batch"
-                  % (sh.batch, len(times), sh.batch),
+    per_seq, ref0 = [], None
+    for b in range(sh.batch):
+        cq = w["q"][b:b + 1].cpu()
+        quant = [w["codes"][b:b + 1].cpu()] + [m[b:b + 1].cpu() for m in w["meta"]]
+        kres = w["kres"][b:b + 1, :, :w["n_resid"]].cpu()
+        v = w["v"][b:b + 1].cpu()
+        if b == 0:
+            po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)        # warm-up
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            ref = po.decode_attention(cq, kres, *quant, v, None, sh.rbits, sh.tbits)
+            times.append(time.perf_counter() - t0)
+        per_seq.append(sorted(times)[1])
+        if b == 0:
+            ref0 = ref
+    return ref0, {
+        "value": round(sum(per_seq) * 1e6, 1), "unit": "us/step", "cores": threads, "cpu": cpu_model(), "kind": "port",
+        "per_sequence_us_min_max": [round(min(per_seq) * 1e6, 1), round(max(per_seq) * 1e6, 1)],
+        "sample": "all %d sequences (8 KV heads x 32768 tokens each), one after the other, median of 3 runs each, summed: the "
+                  "torch-CPU restatement of the reference path (dequantize, matmul, softmax, P.V) on all host threads"
+                  % sh.batch,
     }
 
 
@@ -173,6 +205,74 @@ def fp16_baselines(w, steps, warmup):
     return out
 
 
+def _roof(entry):
+    return {"bound": "hbm", "achieved": entry["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": entry["frac_of_hbm_peak"]}
+
+
+def _flips(got, ref):
+    return {"codes": ref[0].numel(), "flips": int((ref[0] != got[0]).sum()),
+            "metadata_words": sum(m.numel() for m in ref[1:]),
+            "metadata_words_differing": sum(int((a.view(torch.int16) != b.view(torch.int16)).sum()) for a, b in zip(ref[1:], got[1:]))}
+
+
+def _attn_parity(got, ref64):
+    err = (got.double().reshape(ref64.shape) - ref64).abs()
+    return {"max_abs_err": float(err.max()), "within_rtol1e-2_atol1e-3": bool((err <= 1e-3 + 1e-2 * ref64.abs()).all())}
+
+
+def other_configs(dev, steps):
+    """configs[0], [2] and [3] with the same kernels and timing (HIP events around `steps` calls, inputs in
+    HBM), each with its algorithmic bytes, fraction of the 8 TB/s peak, and a check of the timed calls' own
+    results against the CPU oracle on a sampled plane."""
+    from oracle import polar_oracle as po            # the checker, after the timing
+    from polarquant_amd import config_bench as cb
+    out = {}
+
+    res, w = cb.measure(0, dev, steps=steps)
+    sh = w["shape"]
+    quant = [w["codes"].cpu()] + [m.cpu() for m in w["meta"]]
+    ref = po.decode_scores(w["q"].cpu(), *quant, sh.rbits, sh.tbits, dtype=torch.float64)
+    rel = ((w["scores"].cpu().double() - ref).abs() / ref.abs().amax(-1, keepdim=True)).max()
+    fl = _flips(quant, po.quantize_and_pack_nbit(w["keys"].cpu(), sh.rbits, sh.tbits))
+    out["cfg0_scores"] = dict(res[0], workload="configs[0]: score op, batch 1, 32 heads (MHA), context 4096, 4/4 bits",
+                              roofline=_roof(res[0]),
+                              parity={"scores_max_err_rel_to_row_max_vs_fp64_oracle": float(rel), "within_1e-3": bool(rel < 1e-3),
+                                      "quantizer_vs_cpu_oracle": fl, "sample": "all 32 heads x 4096 tokens"})
+    del w, quant, ref
+    torch.cuda.empty_cache()
+
+    res, w = cb.measure(2, dev, steps=steps)
+    sh = w["shape"]
+    b = int(w["lengths"].argmax())
+    L = int(w["lengths"][b]); ng, nr = L // 128, L % 128
+    quant = [w["codes"][b:b + 1, :, :ng].cpu()] + [m[b:b + 1, :, :ng].cpu() for m in w["meta"]]
+    kres = w["kres"][b:b + 1, :, :nr].cpu() if nr else None
+    ref = po.decode_attention_exact(w["q"][b:b + 1].cpu(), kres, *quant, w["v"][b:b + 1, :, :L].cpu(), None, sh.rbits, sh.tbits)
+    out["cfg2_decode"] = dict(res[0], workload="configs[2]: ragged decode attention, batch 64, 28 q / 4 KV heads, lengths uniform in "
+                                               "[512, 8192], 3/3 bits (one byte per code), fp16 V",
+                              roofline=_roof(res[0]),
+                              parity=dict(_attn_parity(w["out"][b:b + 1].cpu(), ref), sample="sequence %d (the longest, %d tokens), all 28 heads, vs the fp64 oracle" % (b, L)))
+    del w, quant, ref
+    torch.cuda.empty_cache()
+
+    res, w = cb.measure(3, dev, steps=steps)
+    sh = w["shape"]
+    quant = [w["codes"][:, :1].cpu()] + [m[:, :1].cpu() for m in w["meta"]]
+    rep = sh.n_heads // sh.n_kv_heads
+    ref = po.decode_attention_exact(w["q"][:, :rep].cpu(), w["kres"][:, :1, :w["n_resid"]].cpu(), *quant, w["v"][:, :1].cpu(), None, sh.rbits, sh.tbits)
+    out["cfg3_decode"] = dict(res[0], workload="configs[3]: decode attention, batch 1, context 131072, 32 q / 8 KV heads, 4/4 bits, split over the context",
+                              roofline=_roof(res[0]),
+                              parity=dict(_attn_parity(w["out"][:, :rep].cpu(), ref), sample="KV head 0 (query heads 0-3), all 131072 tokens, vs the fp64 oracle"))
+    got = [w["append_out"][0][:, :1].cpu()] + [m[:, :1].cpu() for m in w["append_out"][1:]]
+    fl = _flips(got, po.quantize_and_pack_nbit(w["keys"][:, :1].cpu(), sh.rbits, sh.tbits))
+    out["cfg3_append"] = dict(res[1], workload="configs[3]: prompt quantization of 131072 fp16 post-RoPE keys x 8 KV heads (read keys, write codes and metadata)",
+                              roofline=_roof(res[1]),
+                              parity=dict(fl, sample="KV head 0, all 131072 keys, vs the CPU oracle's quantizer"))
+    del w, quant, ref, got
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -181,6 +281,7 @@ def main():
     ap.add_argument("--no-baselines", action="store_true", help="skip the CPU and fp16 baselines")
     ap.add_argument("--splits", type=int, default=0, help="override the context split count")
     ap.add_argument("--no-values4", action="store_true", help="skip the 4-bit-value (Mixed variant) measurement")
+    ap.add_argument("--no-configs", action="store_true", help="skip configs[0], [2] and [3]")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run 3 plain 1 GiB device copies (torch clone): under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` "
                          "their counter values give the scale factor for the attention kernel's")
@@ -237,8 +338,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    def merge_only():
+        rc = lib.pq_decode_attn_merge(ws.data_ptr(), ws.numel() * 4, B, N, n_splits, _ffi.PQ_F16, out.data_ptr(), _stream_ptr(dev))
+        assert rc == 0, rc
+
     ms = time_events(step, args.steps, args.warmup)
-    k_ms = kernel_duration_ms(partials_only, args.steps)
+    ms2, k_ms, m_ms = bracketed_step_ms(partials_only, merge_only, args.steps)
 
     # what a plain read-once kernel is delivered on this GPU: the V tensors of the two input sets
     # (1 GiB each) streamed alternately, one wavefront per SIMD and two per SIMD, best of the two
@@ -284,7 +389,9 @@ def main():
         "pct_of_hbm_peak": round(100 * alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 2),
         "roofline": {"bound": "hbm", "kernel": "attn_kernel<F16,4,4>", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "kernel_us": round(k_ms * 1e3, 2), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel_us": round(k_ms * 1e3, 2), "merge_kernel_us": round(m_ms * 1e3, 2),
+                     "step_us_in_the_bracketed_region": round(ms2 * 1e3, 2),
+                     "traffic": MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                      "plain_stream_read_gbps": round(stream_gbps, 1),
                      "frac_of_plain_stream_read": round(achieved / stream_gbps, 4),
                      "load_only_replica_us": round(r_ms * 1e3, 2),
@@ -324,7 +431,8 @@ def main():
     step()                                   # leave set 0's result in `out` for the parity check
     torch.cuda.synchronize()
     if not args.no_baselines:
-        del w_alt, sets[1:]
+        w_alt = None
+        del sets[1:]
         torch.cuda.empty_cache()
         ref, cpu = cpu_baseline(w)
         result["cpu_baseline"] = cpu
@@ -349,6 +457,11 @@ def main():
                 result["values4"]["speedup_vs_fp16_sdpa_splitk"] = round(fp["fp16_sdpa_splitk_us"] / result["values4"]["us_per_step"], 2)
     else:
         result["cpu_baseline"] = None
+    if not args.no_configs:
+        w = w_alt = None
+        sets.clear()
+        torch.cuda.empty_cache()
+        result["configs"] = other_configs(dev, max(args.steps, 20))
     print(json.dumps(result))
 
 

@@ -55,6 +55,11 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
 /* flags for pq_quantize_groups */
 #define PQ_WRAP_FP32 1u /* add 2*pi in fp32 (eager CUDA semantics) instead of the
                            dtype-rounded 6.28125 that eager CPU torch adds */
+#define PQ_DEVICE_ATAN2 8u /* the angle is round_dtype(atan2f(y, x)) with the GPU math library's atan2f, which
+                              is what eager torch evaluates on device tensors, instead of SLEEF's
+                              Sleef_atan2f_u10, which eager torch evaluates on the CPU */
+#define PQ_EAGER_GPU (PQ_WRAP_FP32 | PQ_DEVICE_ATAN2) /* codes and metadata as the reference's lines produce them
+                              when they run on the GPU (where the reference runs them): both switches */
 #define PQ_ANGLE_UNIFORM 2u /* fixed angle bins over [-pi, pi) instead of the group's own
                                [min, max]: the reference formula (:148) with the constants
                                tmn = -pi and tscale = 2*pi / 2^tbits, both rounded to the key
@@ -172,7 +177,9 @@ int pq_validate_quantize_groups(const void *k, const int64_t *k_strides, int dty
  * two fused multiply-adds; counters[2] receives the number of (dividend, scale)
  * pairs of the dtype, over the whole range the quantizers can meet, whose
  * quotient rounded to the dtype differs from the divided one (must stay 0).
- * `counters`: device uint64[3], zeroed by the caller. Takes ~0.1 s. */
+ * counters[3] and [4]: as [0] and [1] with PQ_DEVICE_ATAN2 (the GPU math library's
+ * arctangent as the exact routine, a wider guard band); [3] must stay 0.
+ * `counters`: device uint64[5], zeroed by the caller. Takes ~0.2 s. */
 int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
 
 /* ---------------------------------------------------------------------------

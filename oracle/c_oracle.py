@@ -36,14 +36,23 @@ def _p(a: np.ndarray):
     return a.ctypes.data_as(ctypes.c_void_p)
 
 
-def quantize(key_states: torch.Tensor, rbits=4, tbits=4, group_size=128, wrap_fp32=False, angle_mode="group"):
+def sleef_atan2f(y: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """The C restatement of Sleef_atan2f_u10 on float32 tensors, element by element."""
+    fn = lib().po_sleef_atan2f_u10
+    fn.restype, fn.argtypes = ctypes.c_float, [ctypes.c_float, ctypes.c_float]
+    ya, xa = y.contiguous().view(-1).tolist(), x.contiguous().view(-1).tolist()
+    return torch.tensor([fn(a, b) for a, b in zip(ya, xa)], dtype=torch.float32).view(y.shape)
+
+
+def quantize(key_states: torch.Tensor, rbits=4, tbits=4, group_size=128, wrap_fp32=False, angle_mode="group", libm_atan2=False):
+    """libm_atan2: the angle by libm's atan2f instead of the SLEEF routine eager torch evaluates."""
     B, Nk, L, D2 = key_states.shape
     D, G, Nb = D2 // 2, group_size, L // group_size
     bf = int(key_states.dtype == torch.bfloat16)
     k = _words(key_states)
     codes = np.empty((B, Nk, Nb, G, D), np.uint8)
     meta = [np.empty((B, Nk, Nb, 1, D), np.uint16) for _ in range(4)]
-    rc = lib().po_quantize(_p(k), bf, int(wrap_fp32) | (2 if angle_mode == "uniform" else 0), B, Nk, L, D, G, rbits, tbits, _p(codes), *[_p(m) for m in meta])
+    rc = lib().po_quantize(_p(k), bf, int(wrap_fp32) | (2 if angle_mode == "uniform" else 0) | (4 if libm_atan2 else 0), B, Nk, L, D, G, rbits, tbits, _p(codes), *[_p(m) for m in meta])
     assert rc == 0
     back = lambda m: torch.from_numpy(m.view(np.int16)).view(key_states.dtype)
     return (torch.from_numpy(codes),) + tuple(back(m) for m in meta)

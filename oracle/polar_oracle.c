@@ -12,9 +12,17 @@
  *
  * Pin status: see the header of oracle/polar_oracle.py; the two restatements
  * are checked against each other bit-for-bit (codes, metadata) and to 1e-6
- * (scores) in tests/test_oracle_pins.py.  The angle uses libm atan2f where the
- * torch restatement uses torch.atan2 (Sleef): a last-ulp difference between the
- * two can move a code across a bin edge; the tests count such flips.
+ * (scores) in tests/test_oracle_pins.py.
+ *
+ * The angle: eager torch evaluates atan2 on half / bfloat16 CPU tensors as
+ * round_dtype(Sleef_atan2f_u10(float y, float x)).  SLEEF is a dependency of PyTorch
+ * that is not in the reference tree (PyTorch vendors SLEEF 3.x; the routine is
+ * xatan2f_u1 with atan2kf_u1 in sleefsp.c).  sleef_atan2f_u10 below restates that
+ * published algorithm in plain C (two-float division, Horner scheme with fused
+ * multiply-adds); tests/test_oracle_pins.py checks it bit for bit against
+ * torch.atan2 on float32.  Flag bit 2 of po_quantize takes libm's atan2f instead:
+ * a third opinion whose last-ulp differences can move a code across a bin edge;
+ * the tests count such flips.
  */
 #include <math.h>
 #include <stdint.h>
@@ -64,6 +72,65 @@ static inline float rnd(float f, int bf) { return lo2f(f2lo(f, bf), bf); }
 float po_half_to_float(uint16_t h) { return h2f(h); }
 uint16_t po_float_to_half(float f) { return f2h(f); }
 
+/* ---- Sleef_atan2f_u10 (SLEEF 3.x, sleefsp.c: xatan2f_u1 / atan2kf_u1), restated ---- */
+typedef struct { float x, y; } f2;
+static inline float mulsignf_(float x, float y) {
+    uint32_t a, b; memcpy(&a, &x, 4); memcpy(&b, &y, 4); a ^= b & 0x80000000u; memcpy(&x, &a, 4); return x;
+}
+static inline f2 df(float x, float y) { f2 r; r.x = x; r.y = y; return r; }
+static inline f2 dfnormalize(f2 t) { f2 s; s.x = t.x + t.y; s.y = t.x - s.x + t.y; return s; }
+static inline f2 dfadd_f_f(float a, float b) { f2 r; r.x = a + b; r.y = a - r.x + b; return r; }
+static inline f2 dfadd_f_f2(float a, f2 b) { f2 r; r.x = a + b.x; r.y = a - r.x + b.x + b.y; return r; }
+static inline f2 dfadd_f2_f2(f2 a, f2 b) { f2 r; r.x = a.x + b.x; r.y = a.x - r.x + b.x + a.y + b.y; return r; }
+static inline f2 dfmul_f2_f2(f2 a, f2 b) {
+    f2 r; r.x = a.x * b.x; r.y = fmaf(a.x, b.y, fmaf(a.y, b.x, fmaf(a.x, b.x, -r.x))); return r;
+}
+static inline f2 dfmul_f2_f(f2 a, float b) { f2 r; r.x = a.x * b; r.y = fmaf(a.y, b, fmaf(a.x, b, -r.x)); return r; }
+static inline f2 dfsqu(f2 a) { f2 r; r.x = a.x * a.x; r.y = fmaf(a.x + a.x, a.y, fmaf(a.x, a.x, -r.x)); return r; }
+static inline f2 dfdiv(f2 n, f2 d) {
+    float t = 1.0f / d.x, u;
+    f2 q;
+    q.x = n.x * t;
+    u = fmaf(t, n.x, -q.x);
+    q.y = fmaf(-d.y, t, fmaf(-d.x, t, 1.0f));
+    q.y = fmaf(q.x, q.y, fmaf(n.y, t, u));
+    return q;
+}
+static f2 atan2kf_u1(f2 y, f2 x) {
+    int q = 0;
+    f2 s, t;
+    float u;
+    if (x.x < 0) { x.x = -x.x; x.y = -x.y; q = -2; }
+    if (x.x < y.x) { t = x; x = y; y.x = -t.x; y.y = -t.y; q += 1; }
+    s = dfdiv(y, x);
+    t = dfnormalize(dfsqu(s));
+    u = -0.00176397908944636583328247f;
+    u = fmaf(u, t.x, 0.0107900900766253471374512f);
+    u = fmaf(u, t.x, -0.0309564601629972457885742f);
+    u = fmaf(u, t.x, 0.0577365085482597351074219f);
+    u = fmaf(u, t.x, -0.0838950723409652709960938f);
+    u = fmaf(u, t.x, 0.109463557600975036621094f);
+    u = fmaf(u, t.x, -0.142626821994781494140625f);
+    u = fmaf(u, t.x, 0.199983194470405578613281f);
+    t = dfmul_f2_f2(t, dfadd_f_f(-0.333332866430282592773438f, u * t.x));
+    t = dfmul_f2_f2(s, dfadd_f_f2(1.0f, t));
+    t = dfadd_f2_f2(dfmul_f2_f(df(1.5707963705062866211f, -4.3711388286737928865e-08f), (float)q), t);
+    return t;
+}
+float po_sleef_atan2f_u10(float y, float x) {
+    f2 d;
+    float r;
+    if (fabsf(x) < 2.9387372783541830947e-39f) { y *= 16777216.0f; x *= 16777216.0f; }   /* x denormal: scale both */
+    d = atan2kf_u1(df(fabsf(y), 0), df(x, 0));
+    r = d.x + d.y;
+    r = mulsignf_(r, x);
+    if (isinf(x) || x == 0) r = 1.570796326794896557998982f - (isinf(x) ? mulsignf_(1.570796326794896557998982f, x) : 0.0f);
+    if (isinf(y)) r = 1.570796326794896557998982f - (isinf(x) ? mulsignf_(0.785398163397448278999491f, x) : 0.0f);
+    if (y == 0) r = signbit(x) ? 3.141592653589793238462643f : 0.0f;
+    if (isnan(x) || isnan(y)) return NAN;
+    return mulsignf_(r, y);
+}
+
 static uint8_t code_of(float v, float mn, float scale, int bits, int bf) {
     float d = rnd(v - mn, bf);
     float q = rnd(d / scale, bf);
@@ -81,8 +148,9 @@ int po_quantize(const uint16_t *k, int bf, int flags, int B, int Nk, int L, int 
                 uint8_t *codes, uint16_t *rscale, uint16_t *rmn, uint16_t *tscale, uint16_t *tmn) {
     if (L % G || rbits + tbits > 8) return -1;
     /* flags: bit 0 = wrap in fp32, bit 1 = uniform angle bins over [-pi, pi) (no reference
-     * counterpart: tmn = -pi, tscale = 2*pi / 2^tbits as key-dtype constants, no wrap) */
-    const int wrap_fp32 = flags & 1, uniform = (flags >> 1) & 1;
+     * counterpart: tmn = -pi, tscale = 2*pi / 2^tbits as key-dtype constants, no wrap),
+     * bit 2 = libm's atan2f instead of the SLEEF routine eager torch evaluates */
+    const int wrap_fp32 = flags & 1, uniform = (flags >> 1) & 1, libm_atan = (flags >> 2) & 1;
     /* torch-CPU casts the python scalar 2*pi to the tensor dtype before the add
      * (6.28125 in both half and bfloat16); wrap_fp32 != 0 keeps it in fp32, which
      * is what an eager CUDA add of a half tensor and a python scalar does. */
@@ -97,7 +165,7 @@ int po_quantize(const uint16_t *k, int bf, int flags, int B, int Nk, int L, int 
                 float pmx = -INFINITY, pmn = INFINITY, rmx_ = -INFINITY, rmn_ = INFINITY;
                 for (int g = 0; g < G; g++) {
                     float x = lo2f(base[(long)g * 2 * D + d], bf), y = lo2f(base[(long)g * 2 * D + D + d], bf);
-                    float p = rnd(atan2f(y, x), bf);                       /* :143 */
+                    float p = rnd(libm_atan ? atan2f(y, x) : po_sleef_atan2f_u10(y, x), bf);   /* :143 */
                     if (p < 0 && !uniform) p = rnd(p + TWO_PI, bf);        /* :144 */
                     float r = rnd(sqrtf(x * x + y * y), bf);               /* :150 */
                     phi[g] = p; rad[g] = r;

@@ -12,8 +12,15 @@ the checks live in tests/test_oracle_pins.py):
                            closed-form known-answer group (angles on bin
                            centres), min/max-element invariants, error bounds,
                            cross-check against the independent C restatement
-                           (oracle/polar_oracle.c).  The reference holds no
-                           golden vectors for it.
+                           (oracle/polar_oracle.c, bit for bit, its own restatement
+                           of SLEEF's arctangent included).  The reference holds no
+                           golden vectors for it.  Its wrap_fp32 switch (the one
+                           line eager torch evaluates differently on GPU tensors)
+                           is pinned the same way; the remaining difference of a
+                           GPU evaluation, the device library's atan2f, cannot be
+                           restated on the CPU and is pinned on the GPU against
+                           eager torch ops on device tensors
+                           (tests/test_quantize_gpu.py).
   dequantize_keys          pinned: closed form on the known-answer group,
                            error bounds |phi-phi^|<=tscale/2, |r-r^|<=rscale/2.
   decode_scores            pinned: textbook q.K^T (torch.matmul) on the
@@ -96,7 +103,7 @@ def _to_u8_defined(x: torch.Tensor) -> torch.Tensor:
 
 
 def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4,
-                           group_size: int = GROUP_SIZE, angle_mode: str = "group"):
+                           group_size: int = GROUP_SIZE, angle_mode: str = "group", wrap_fp32: bool = False):
     """key_states [B,Nk,L,2*D] half/bf16 (post-RoPE) ->
     (indices u8 [B,Nk,Nb,G,D], rscale, rmn, tscale, tmn [B,Nk,Nb,1,D] in key dtype).
 
@@ -106,6 +113,10 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     angle_mode="uniform" (no reference counterpart; the fixed-grid special case of the same
     formula): the angle is not wrapped, tmn = -pi and tscale = 2*pi / 2^tbits as key-dtype
     constants, theta by line :148 unchanged.
+
+    wrap_fp32: line :144 as eager torch evaluates it on GPU tensors, where a python scalar added to a
+    half tensor stays fp32 (phi is widened, 2*pi added as the fp32 6.2831855, the sum rounded once);
+    on CPU tensors, the default here, the scalar is first cast to the tensor dtype (6.28125).
     """
     B, N, L, D2 = key_states.shape
     assert D2 % 2 == 0 and L % group_size == 0 and rbits + tbits <= 8
@@ -117,7 +128,8 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
         tmn = torch.full_like(phi[..., :1, :], -math.pi)
         tscale = torch.full_like(tmn, 2 * math.pi) / (2 ** tbits)
     else:
-        phi = torch.where(phi < 0, phi + 2 * math.pi, phi)                    # :144
+        wrapped = (phi.float() + 2 * math.pi).to(phi.dtype) if wrap_fp32 else phi + 2 * math.pi
+        phi = torch.where(phi < 0, wrapped, phi)                              # :144
         tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]  # :146
         tscale = (tmx - tmn) / (2 ** tbits)                                   # :147
     theta = torch.clamp(_to_u8_defined((phi - tmn) / tscale), 0, 2 ** tbits - 1)  # :148

@@ -17,6 +17,8 @@ PQ_F16, PQ_BF16 = 0, 1
 PQ_WRAP_FP32 = 1
 PQ_ANGLE_UNIFORM = 2
 PQ_CODES_PACKED6 = 4
+PQ_DEVICE_ATAN2 = 8
+PQ_EAGER_GPU = PQ_WRAP_FP32 | PQ_DEVICE_ATAN2
 
 STATUS_NAMES = {
     0: "PQ_OK", -1: "PQ_ERR_NULL_POINTER", -2: "PQ_ERR_BAD_SHAPE", -3: "PQ_ERR_BAD_BITS", -4: "PQ_ERR_BAD_DTYPE",

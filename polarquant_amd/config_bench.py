@@ -1,5 +1,5 @@
 """The other benchmark configurations on one GPU, same kernels and timing as bench.py
-(which carries the headline, configs[1]):
+(which carries the headline, configs[1], and calls `measure` here for the rest):
 
   configs[0]  score op, Llama-2-7B shape (batch 1, 32 heads MHA, context 4096)
   configs[2]  ragged continuous-batch decode attention, Qwen2.5-7B shape (batch 64, GQA 7, 3/3 bits)
@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import time
 
 import torch
 
@@ -27,16 +28,21 @@ from .values import quantize_values
 HBM_PEAK_GBPS = 8000.0
 
 
-def _line(cfg, op, ms, nbytes, **extra):
+def _entry(op, ms, nbytes, **extra):
     gbps = nbytes / (ms * 1e-3) / 1e9
-    print(json.dumps(dict(config=cfg, op=op, us=round(ms * 1e3, 2), algorithmic_bytes=int(nbytes), hbm_gbps=round(gbps, 1),
-                          frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)), flush=True)
+    return dict(op=op, us=round(ms * 1e3, 2), algorithmic_bytes=int(nbytes), hbm_gbps=round(gbps, 1),
+                frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)
 
 
-def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
-    w = wl.build_workload(idx, dev, keep_keys=(idx == 3), packed=packed)
+def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool = False):
+    """Time configs[idx] -> (list of measurement dicts, the workload).  The workload keeps what a caller
+    needs to check the timed calls' results against a CPU checker: w["scores"] (configs[0]), w["out"] (decode
+    attention output), w["append_out"] (configs[3]: codes and metadata the timed quantizer calls wrote) and
+    w["keys"] (configs[0] and configs[3])."""
+    w = wl.build_workload(idx, dev, keep_keys=(idx in (0, 3)), packed=packed)
     sh = w["shape"]
     B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
+    res = []
     if idx == 0:
         # 9 MB of inputs would sit in the 256 MB Infinity Cache: rotate over 8 independent copies
         sets = [(w["q"].clone(), w["codes"].clone(), [m.clone() for m in w["meta"]]) for _ in range(8)]
@@ -47,20 +53,34 @@ def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
             turn[0] += 1
             return attention_decode_forward_triton_impl(q, c, *m, rbits=sh.rbits, tbits=sh.tbits)
         ms = wl.time_events(score, 4 * steps, steps)
+        # the reference's own protocol (benchmark/benchmark_matmul.py:108-118): synchronize, host clock, call,
+        # synchronize, host clock; mean over the calls
+        total, calls = 0.0, 1000
+        for _ in range(calls):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            score()
+            torch.cuda.synchronize()
+            total += time.perf_counter() - t0
         nbytes = w["codes"].numel() + 4 * w["meta"][0].numel() * 2 + B * N * sh.context * 4 + w["q"].numel() * 2
-        _line(idx, "scores (pq_decode_scores)", ms, nbytes)
+        res.append(_entry("scores (pq_decode_scores)", ms, nbytes, us_host_clock_per_synchronized_call=round(total / calls * 1e6, 2),
+                          input_sets_rotated=8))
+        w["scores"] = attention_decode_forward_triton_impl(w["q"], w["codes"], *w["meta"], rbits=sh.rbits, tbits=sh.tbits)
+        return res, w
     if sh.ragged:
         lens = w["lengths"]
-        lq, res = ((lens // 128) * 128).tolist(), (lens % 128).tolist()
+        lq, rs = ((lens // 128) * 128).tolist(), (lens % 128).tolist()
         total_groups = int((lens // 128).sum())
     else:
-        lq, res, total_groups = [w["n_groups"] * 128] * B, [w["n_resid"]] * B, None
-    nbytes = wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits, code_bytes_per_pair=0.75 if packed else 1.0)
+        lq, rs, total_groups = [w["n_groups"] * 128] * B, [w["n_resid"]] * B, None
+    nbytes = wl.algorithmic_bytes(Nk, N, lq, rs, sh.rbits, sh.tbits, code_bytes_per_pair=0.75 if packed else 1.0)
+    out = torch.empty(B, N, 1, 128, dtype=w["q"].dtype, device=dev)
     ms = wl.time_events(lambda: polar_decode_attention(
         w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
-        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups), steps, 10)
-    _line(idx, "decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else ""), ms, nbytes,
-          tokens=int(sum(lq) + sum(res)))
+        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups, out=out), steps, 10)
+    res.append(_entry("decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else ""), ms, nbytes,
+                      tokens=int(sum(lq) + sum(rs))))
+    w["out"] = out
     if values4 and not sh.ragged:
         L = w["n_groups"] * 128
         vq = quantize_values(w["v"][:, :, :L])
@@ -68,15 +88,25 @@ def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
         vres[:, :, :w["n_resid"]] = w["v"][:, :, L:L + w["n_resid"]]
         ms4 = wl.time_events(lambda: polar_decode_attention_v4(
             w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits), steps, 10)
-        _line(idx, "decode attention, 4-bit values (pq_decode_attn_v4)", ms4,
-              wl.algorithmic_bytes(Nk, N, lq, res, sh.rbits, sh.tbits, value_bits=4))
+        res.append(_entry("decode attention, 4-bit values (pq_decode_attn_v4)", ms4,
+                          wl.algorithmic_bytes(Nk, N, lq, rs, sh.rbits, sh.tbits, value_bits=4)))
         msq = wl.time_events(lambda: quantize_values(w["v"][:, :, :L], out=vq), max(steps // 2, 5), 3)
-        _line(idx, "value quantization (pq_quantize_values)", msq, B * Nk * L * (256 + 64 + 4))
+        res.append(_entry("value quantization (pq_quantize_values)", msq, B * Nk * L * (256 + 64 + 4)))
+        del vq, vres
     if idx == 3:
         k = w["keys"]
-        out = (torch.empty_like(w["codes"]), *[torch.empty_like(m) for m in w["meta"]])
-        ms = wl.time_events(lambda: quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=out), max(steps // 2, 5), 5)
-        _line(idx, "append / prompt quantization (pq_quantize_groups)", ms, k.numel() * 2 + out[0].numel() + 4 * out[1].numel() * 2)
+        aout = (torch.empty_like(w["codes"]), *[torch.empty_like(m) for m in w["meta"]])
+        ms = wl.time_events(lambda: quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=aout), max(steps // 2, 5), 5)
+        res.append(_entry("append / prompt quantization (pq_quantize_groups)", ms,
+                          k.numel() * 2 + aout[0].numel() + 4 * aout[1].numel() * 2))
+        w["append_out"] = aout
+    return res, w
+
+
+def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
+    res, _ = measure(idx, dev, values4, steps, packed)
+    for r in res:
+        print(json.dumps(dict(config=idx, **r)), flush=True)
 
 
 def main():

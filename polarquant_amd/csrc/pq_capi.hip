@@ -91,7 +91,7 @@ int pq_validate_quantize_groups(const void* k, const int64_t* k_strides, int dty
     // the same bit widths as the decode entry points: no cache is written that nothing here can read
     if (int rc = check_bits(rbits, tbits)) return rc;
     if (dtype != PQ_F16 && dtype != PQ_BF16) return PQ_ERR_BAD_DTYPE;
-    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM | PQ_CODES_PACKED6)) return PQ_ERR_BAD_SHAPE;
+    if (flags & ~static_cast<unsigned>(PQ_WRAP_FP32 | PQ_ANGLE_UNIFORM | PQ_CODES_PACKED6 | PQ_DEVICE_ATAN2)) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && rbits + tbits > 6) return PQ_ERR_BAD_BITS;
     if (k_strides[3] != 1) return PQ_ERR_BAD_STRIDE;
     if (k_strides[0] < 0 || k_strides[1] < 0 || k_strides[2] < PQ_HEAD_DIM) return PQ_ERR_BAD_STRIDE;

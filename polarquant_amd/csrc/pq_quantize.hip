@@ -42,6 +42,20 @@ template <> struct DT<BF16> { static constexpr uint32_t kLowMask = 0xffffu, kMid
 constexpr uint32_t kAtanGuardUlps = 5;   // the fast arctangent stays within 4 ulp of the exact routine (exhaustive self-test)
 constexpr uint32_t kSqrtGuardUlps = 2;   // v_sqrt_f32 is within 1 ulp
 
+// Which arctangent the angle must reproduce.  Eager torch evaluates atan2 on half tensors in fp32 and
+// rounds once: on the CPU with SLEEF's Sleef_atan2f_u10 (restated in pq_math.h), on the GPU with the
+// device math library's atan2f, which is what `atan2f` in device code here resolves to as well.  The
+// two differ in the last fp32 bits on about a third of all operands, and after rounding to half on a
+// few dozen per million.  LIBM = true selects the device library's routine as the exact one; it lies
+// within 3 ulp of SLEEF's on every operand pair seen, so the estimate's guard band is widened by that
+// (the exhaustive self-test checks the wider band against the library routine itself).
+template <bool LIBM> struct Atan { static constexpr uint32_t kGuardUlps = LIBM ? kAtanGuardUlps + 4 : kAtanGuardUlps; };
+template <bool LIBM>
+__device__ __forceinline__ float atan2_exact(float y, float x) {
+    if constexpr (LIBM) return atan2f(y, x);
+    else return math::atan2f_sleef_u10(y, x);
+}
+
 template <typename T>
 __device__ __forceinline__ bool near_rounding_boundary(float a, uint32_t guard) {
     // |low mantissa bits - midpoint pattern| <= guard, computed without a branch
@@ -70,7 +84,7 @@ __device__ __forceinline__ float atan2_fast(float y, float x) {
 
 // Cheap estimates of the angle (in [-pi, pi]) and radius, NOT yet rounded; returns true when
 // the exact routines must be used instead (see above).
-template <typename T>
+template <typename T, bool LIBM = false>
 __device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out, float* r_out) {
     const float ss = __builtin_fmaf(x, x, y * y);          // x*x, y*y are exact for half/bf16 operands
     const float a = atan2_fast(y, x);
@@ -86,7 +100,7 @@ __device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out
     *a_out = a;
     *r_out = r;
     return (special | static_cast<int>(fminf(fabsf(a), r) < DT<T>::kMinNormal) |
-            static_cast<int>(near_rounding_boundary<T>(a, kAtanGuardUlps)) |
+            static_cast<int>(near_rounding_boundary<T>(a, Atan<LIBM>::kGuardUlps)) |
             static_cast<int>(near_rounding_boundary<T>(r, kSqrtGuardUlps))) != 0;
 }
 
@@ -97,20 +111,20 @@ __device__ __forceinline__ bool angle_radius_fast(float x, float y, float* a_out
 __device__ __forceinline__ float sqrt_rn(float s) { return __builtin_sqrtf(s); }
 
 // -> (angle in [-pi, pi], radius), both rounded to the key dtype
-template <typename T>
+template <typename T, bool LIBM = false>
 __device__ __forceinline__ void angle_radius(float x, float y, float* phi, float* rad) {
     float a, r;
-    if (__builtin_expect(angle_radius_fast<T>(x, y, &a, &r), 0)) {
-        a = math::atan2f_sleef_u10(y, x);
+    if (__builtin_expect(angle_radius_fast<T, LIBM>(x, y, &a, &r), 0)) {
+        a = atan2_exact<LIBM>(y, x);
         r = sqrt_rn(__builtin_fmaf(x, x, y * y));
     }
     *phi = rnd<T>(a);
     *rad = rnd<T>(r);
 }
 
-template <typename T>
+template <typename T, bool LIBM = false>
 __device__ __forceinline__ void angle_radius_exact(float x, float y, float* phi, float* rad) {
-    *phi = rnd<T>(math::atan2f_sleef_u10(y, x));
+    *phi = rnd<T>(atan2_exact<LIBM>(y, x));
     *rad = rnd<T>(sqrt_rn(__builtin_fmaf(x, x, y * y)));
 }
 
@@ -185,7 +199,7 @@ __device__ __forceinline__ uint32_t pack_angle_radius(float a, float r, const An
     return (aw | (static_cast<uint32_t>(f2lo<T>(r)) << 16)) & 0x7fff7fffu;
 }
 
-template <typename T, bool UNIFORM, bool PK6>
+template <typename T, bool UNIFORM, bool PK6, bool LIBM>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     const uint16_t* __restrict__ k, int64_t sb, int64_t sh, int64_t st, int Nk, int rbits, int tbits, AngleMode am,
     uint8_t* __restrict__ codes, uint16_t* __restrict__ rscale, uint16_t* __restrict__ rmn,
@@ -215,7 +229,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             float a, r;
-            const bool risky = angle_radius_fast<T>(lo2f<T>(xs[i]), lo2f<T>(ys[i]), &a, &r);   // :143, :150
+            const bool risky = angle_radius_fast<T, LIBM>(lo2f<T>(xs[i]), lo2f<T>(ys[i]), &a, &r);   // :143, :150
             risky_mask |= static_cast<uint32_t>(risky) << (it * 4 + i);
             pr[it * 4 + i][tid] = pack_angle_radius<T, UNIFORM>(a, rnd<T>(r), am);
         }
@@ -228,7 +242,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
         const uint16_t* row = kb + ((e >> 2) * 16 + tl) * st;
         const float x = lo2f<T>(row[4 * pq4 + (e & 3)]), y = lo2f<T>(row[kPairs + 4 * pq4 + (e & 3)]);
         float a, r;
-        angle_radius_exact<T>(x, y, &a, &r);
+        angle_radius_exact<T, LIBM>(x, y, &a, &r);
         pr[e][tid] = pack_angle_radius<T, UNIFORM>(a, r, am);
     }
     // ---- per-pair max / min of angle and radius over the 128 tokens (packed: both at once)
@@ -354,7 +368,7 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
 
 // Exhaustive check of angle_radius against angle_radius_exact: block == bit pattern of y,
 // thread t covers x patterns t, t+256, ...; NaN operands are skipped.
-template <typename T>
+template <typename T, bool LIBM>
 __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* mismatches, unsigned long long* slow_lanes) {
     const uint16_t yb = static_cast<uint16_t>(blockIdx.x);
     const float y = lo2f<T>(yb);
@@ -363,19 +377,19 @@ __global__ __launch_bounds__(256) void selftest_kernel(unsigned long long* misma
         const float x = lo2f<T>(static_cast<uint16_t>(xb));
         if (x != x || y != y) continue;
         float p0, r0, p1, r1;
-        angle_radius<T>(x, y, &p0, &r0);
-        angle_radius_exact<T>(x, y, &p1, &r1);
+        angle_radius<T, LIBM>(x, y, &p0, &r0);
+        angle_radius_exact<T, LIBM>(x, y, &p1, &r1);
         bad += (f2lo<T>(p0) != f2lo<T>(p1)) || (f2lo<T>(r0) != f2lo<T>(r1));
         // the exact radius: s lies between the squares of the midpoints to the two neighbours of sqrt_rn(s)
         const float s = __builtin_fmaf(x, x, y * y);
-        if (s > 0.0f && s < INFINITY) {
+        if (!LIBM && s > 0.0f && s < INFINITY) {
             const float rr = sqrt_rn(s);
             const double lo = 0.5 * (static_cast<double>(rr) + static_cast<double>(__uint_as_float(__float_as_uint(rr) - 1u)));
             const double hi = 0.5 * (static_cast<double>(rr) + static_cast<double>(__uint_as_float(__float_as_uint(rr) + 1u)));
             bad += !(lo * lo <= static_cast<double>(s) && static_cast<double>(s) <= hi * hi);
         }
         const float a = atan2_fast(y, x), r = __builtin_amdgcn_sqrtf(__builtin_fmaf(x, x, y * y));
-        slow += near_rounding_boundary<T>(a, kAtanGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
+        slow += near_rounding_boundary<T>(a, Atan<LIBM>::kGuardUlps) || near_rounding_boundary<T>(r, kSqrtGuardUlps);
     }
     if (bad) atomicAdd(mismatches, static_cast<unsigned long long>(bad));
     if (slow) atomicAdd(slow_lanes, static_cast<unsigned long long>(slow));
@@ -403,12 +417,16 @@ __global__ __launch_bounds__(256) void selftest_div_kernel(unsigned long long* m
 }
 
 int launch_selftest(int dtype, unsigned long long* counters, hipStream_t st) {
+    // counters: [0] mismatches, [1] exact-path pairs (SLEEF arctangent); [2] division mismatches;
+    // [3] mismatches, [4] exact-path pairs with the device library's arctangent as the exact routine
     if (dtype == 0) {
-        hipLaunchKernelGGL(selftest_kernel<F16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+        hipLaunchKernelGGL((selftest_kernel<F16, false>), dim3(65536), dim3(256), 0, st, counters, counters + 1);
         hipLaunchKernelGGL(selftest_div_kernel<F16>, dim3(65536), dim3(256), 0, st, counters + 2);
+        hipLaunchKernelGGL((selftest_kernel<F16, true>), dim3(65536), dim3(256), 0, st, counters + 3, counters + 4);
     } else {
-        hipLaunchKernelGGL(selftest_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters, counters + 1);
+        hipLaunchKernelGGL((selftest_kernel<BF16, false>), dim3(65536), dim3(256), 0, st, counters, counters + 1);
         hipLaunchKernelGGL(selftest_div_kernel<BF16>, dim3(65536), dim3(256), 0, st, counters + 2);
+        hipLaunchKernelGGL((selftest_kernel<BF16, true>), dim3(65536), dim3(256), 0, st, counters + 3, counters + 4);
     }
     return static_cast<int>(hipGetLastError());
 }
@@ -430,10 +448,16 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
     am.tmn = round_dt(-3.14159274101257324219f);
     am.tscale = round_dt(round_dt(two_pi_f) / static_cast<float>(1 << tbits));
     const bool packed6 = (flags & 4u) != 0;
-#define PQ_LAUNCH_QP(T, U, P)                                                                                        \
-    hipLaunchKernelGGL((quantize_kernel<T, U, P>), grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],  \
+    const bool libm = (flags & 8u) != 0;
+#define PQ_LAUNCH_QPL(T, U, P, L)                                                                                    \
+    hipLaunchKernelGGL((quantize_kernel<T, U, P, L>), grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1], \
                        strides[2], Nk, rbits, tbits, am, codes, (uint16_t*)rscale, (uint16_t*)rmn,                  \
                        (uint16_t*)tscale, (uint16_t*)tmn, cap, off)
+#define PQ_LAUNCH_QP(T, U, P)                                                                                        \
+    do {                                                                                                             \
+        if (libm) PQ_LAUNCH_QPL(T, U, P, true);                                                                      \
+        else PQ_LAUNCH_QPL(T, U, P, false);                                                                          \
+    } while (0)
 #define PQ_LAUNCH_Q(T, U)                                                                                            \
     do {                                                                                                             \
         if (packed6) PQ_LAUNCH_QP(T, U, true);                                                                       \
@@ -443,6 +467,7 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
     else            { if (uniform) PQ_LAUNCH_Q(BF16, true); else PQ_LAUNCH_Q(BF16, false); }
 #undef PQ_LAUNCH_Q
 #undef PQ_LAUNCH_QP
+#undef PQ_LAUNCH_QPL
     return static_cast<int>(hipGetLastError());
 }
 

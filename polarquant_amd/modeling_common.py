@@ -59,6 +59,8 @@ class PolarConfig:
     vbits: int = 16                     # 4: values in 4 bits as well (the Mixed variant); 16: half-precision values
     snapkv: bool = False                # SnapKV prompt eviction in front of the polar cache (batch 1 decode)
     packed_codes: bool = False          # 3/3-bit key codes as packed 6-bit rows (48 instead of 64 bytes per token and head)
+    eager_gpu_codes: bool = False       # key codes / metadata as the reference's lines give them on GPU tensors (fp32 wrap,
+                                        # device atan2f) instead of on CPU tensors; for caches shared with a GPU-run reference
     cache_capacity: int = 0             # tokens to pre-allocate per layer (0: prompt + 1024, grown by doubling)
 
     @staticmethod
@@ -196,9 +198,10 @@ class MLP(nn.Module):
 class _Arena:
     """Pre-allocated per-layer polar KV cache.  codes/meta/v grow by doubling."""
 
-    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False):
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False, eager_gpu=False):
         self.B, self.Nk, self.dtype, self.device = B, Nk, dtype, device
         self.rbits, self.tbits = rbits, tbits
+        self.eager_gpu = eager_gpu    # quantize as eager torch does on GPU tensors
         self.packed = packed          # code rows of 48 bytes (packed 6-bit codes) instead of 64
         self.row = 48 if packed else 64
         self.n_groups = self.n_resid = self.kv_len = 0
@@ -228,7 +231,7 @@ class _Arena:
         """keys [B,Nk,n*128,128] (any strides with unit dim stride) -> groups appended."""
         n = keys.shape[2] // GROUP
         quantize_and_pack_nbit(keys, self.rbits, self.tbits, packed=self.packed, out=(self.codes, *self.meta),
-                               group_offset=self.n_groups)
+                               group_offset=self.n_groups, eager_gpu=self.eager_gpu)
         self.n_groups += n
 
     def as_tuple(self) -> "PolarCache":
@@ -294,13 +297,15 @@ class PolarGroupAttention(nn.Module):
         # not in the reference (which stores one byte per pair for every bit width, kernel4group.py:1-3):
         # 3/3-bit codes stored as packed 6-bit rows, indices [B,Nk,Nb,128,48] in the cache tuple
         self.packed_codes = bool(_cfg(config, "packed_codes", False))
+        self.eager_gpu_codes = bool(_cfg(config, "eager_gpu_codes", False))
         assert not self.packed_codes or (self.tbits == 3 and self.rbits + self.tbits <= 6), "packed codes: tbits 3, rbits <= 3"
         self.capture = None   # test hook: a list that receives post-RoPE (q, k, v) of every call
 
     # -- cache plumbing --------------------------------------------------------
     def _new_arena(self, B, dtype, device, tokens):
         cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
-        return _Arena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes)
+        return _Arena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes,
+                      self.eager_gpu_codes)
 
     def _arena_of(self, past_key_value, dtype, device) -> _Arena:
         arena = getattr(past_key_value, "arena", None)
@@ -383,9 +388,9 @@ class _MixedArena(_Arena):
     """Per-layer cache of the Mixed variant: polar key groups, 4-bit value rows for the same tokens,
     and a shared 128-token residual window of half-precision keys and values."""
 
-    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False):
+    def __init__(self, B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed=False, eager_gpu=False):
         self.vres = torch.zeros(B, Nk, GROUP, 128, dtype=dtype, device=device)
-        super().__init__(B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed)
+        super().__init__(B, Nk, dtype, device, capacity_tokens, rbits, tbits, packed, eager_gpu)
 
     def _alloc(self, cap_tokens):
         gcap = (cap_tokens + GROUP - 1) // GROUP
@@ -435,7 +440,8 @@ class PolarMixedGroupAttention(PolarGroupAttention):
 
     def _new_arena(self, B, dtype, device, tokens):
         cap = _cfg(self.config, "cache_capacity", 0) or (tokens + 1024)
-        return _MixedArena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes)
+        return _MixedArena(B, self.num_key_value_heads, dtype, device, max(cap, tokens), self.rbits, self.tbits, self.packed_codes,
+                           self.eager_gpu_codes)
 
     def _arena_of(self, past_key_value, dtype, device) -> _MixedArena:
         arena = getattr(past_key_value, "arena", None)

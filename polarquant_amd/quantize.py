@@ -16,7 +16,8 @@ PAIRS = 64
 
 def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int = 4, group_size: int = GROUP,
                            wrap_fp32: bool = False, angle_mode: str = "group", packed: bool = False,
-                           out: Optional[Tuple[torch.Tensor, ...]] = None, group_offset: int = 0):
+                           out: Optional[Tuple[torch.Tensor, ...]] = None, group_offset: int = 0,
+                           device_atan2: bool = False, eager_gpu: bool = False):
     """key_states [B,Nk,L,128] half/bf16 on the GPU (any batch/head/token strides, unit dim stride)
     -> (indices u8 [B,Nk,Nb,128,64], rscale, rmn, tscale, tmn [B,Nk,Nb,1,64]).
 
@@ -27,6 +28,12 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     `angle_mode="group"` is the reference's binning (2^tbits bins over each group's own angle
     range); `"uniform"` uses fixed bins over [-pi, pi) and writes the constants
     tmn = -pi, tscale = 2*pi/2^tbits into the metadata, so decode is unchanged.
+
+    By default codes and metadata are those of the reference's lines evaluated by eager torch on CPU
+    tensors.  `eager_gpu=True` gives those of the same lines evaluated by eager torch on GPU tensors,
+    which is where the reference runs them; it differs in two places, selectable one by one:
+    `wrap_fp32` (2*pi is added to negative angles in fp32 instead of as the dtype-rounded 6.28125) and
+    `device_atan2` (the GPU math library's atan2f instead of SLEEF's).
 
     `packed=True` (rbits + tbits <= 6) stores the 64 codes of a token as 48 bytes of packed 6-bit
     codes ([B,Nk,Nb,128,48]) instead of one byte each; the decode entry points recognise the shape.
@@ -55,7 +62,9 @@ def quantize_and_pack_nbit(key_states: torch.Tensor, rbits: int = 4, tbits: int 
     strides = (ctypes.c_int64 * 4)(*key_states.stride())
     with torch.cuda.device(dev):
         rc = _ffi.lib().pq_quantize_groups(key_states.data_ptr(), ctypes.cast(strides, ctypes.c_void_p), dt, B, Nk, Nb,
-                                           rbits, tbits, (_ffi.PQ_WRAP_FP32 if wrap_fp32 else 0) | (_ffi.PQ_ANGLE_UNIFORM if angle_mode == "uniform" else 0)
+                                           rbits, tbits, (_ffi.PQ_WRAP_FP32 if wrap_fp32 or eager_gpu else 0)
+                                           | (_ffi.PQ_DEVICE_ATAN2 if device_atan2 or eager_gpu else 0)
+                                           | (_ffi.PQ_ANGLE_UNIFORM if angle_mode == "uniform" else 0)
                                            | (_ffi.PQ_CODES_PACKED6 if packed else 0),
                                            codes.data_ptr(), *[m.data_ptr() for m in meta], cap, off,
                                            _stream_ptr(dev))

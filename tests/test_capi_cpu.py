@@ -90,7 +90,8 @@ def test_validate_quantize_groups(lib):
     assert bad(8, 4) == -3                           # packed 6-bit codes need rbits + tbits <= 6
     a = list(ok); a[6], a[7], a[8] = 3, 3, 4
     assert lib.pq_validate_quantize_groups(*a) == 0
-    assert bad(8, 8) == -2                           # unknown flag bit
+    assert bad(8, 8) == 0 and bad(8, 9) == 0         # PQ_DEVICE_ATAN2, PQ_EAGER_GPU
+    assert bad(8, 16) == -2                          # unknown flag bit
     assert bad(14, 1) == -6 and bad(15, 1) == -6     # capacity < offset + Nb
     assert bad(0, P + 2) == -5                       # key pointer not 8-byte aligned
     for i, s in enumerate([(8 * 256 * 128, 256 * 128, 128, 2), (8 * 256 * 128, 256 * 128, 64, 1),

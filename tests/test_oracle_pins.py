@@ -143,19 +143,54 @@ def test_uniform_angle_mode_known_answers(dtype, tb):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (5, 3)])
 def test_c_and_torch_restatements_agree(dtype, rbits, tbits):
-    """Two independent restatements (torch eager ops with SLEEF atan2 / scalar C with libm atan2f)."""
+    """Two independent restatements: torch eager ops (whose atan2 is SLEEF's) and scalar C with its own
+    restatement of that SLEEF routine agree bit for bit; with libm's atan2f in the C one, a last-ulp
+    difference of the arctangents moves a few values across a rounding tie (counted, bounded)."""
     k, _ = _keys(2, 4, 1024, 4, dtype)
     a = po.quantize_and_pack_nbit(k, rbits, tbits)
     b = co.quantize(k, rbits, tbits)
     assert all(x.shape == y.shape for x, y in zip(a, b))
+    assert torch.equal(a[0], b[0])
+    for x, y in zip(a[1:], b[1:]):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16))
+    c = co.quantize(k, rbits, tbits, libm_atan2=True)
     # radius side shares no transcendental: bit-exact
-    assert torch.equal(a[1].view(torch.int16), b[1].view(torch.int16))
-    assert torch.equal(a[2].view(torch.int16), b[2].view(torch.int16))
-    # angle side: a last-ulp difference of the two arctangents can move a value across a rounding tie
-    flips = int((a[0] != b[0]).sum())
-    meta = int((a[3].view(torch.int16) != b[3].view(torch.int16)).sum()) + int((a[4].view(torch.int16) != b[4].view(torch.int16)).sum())
-    print("torch-vs-C flips: codes %d / %d, angle metadata %d" % (flips, a[0].numel(), meta))
+    assert torch.equal(a[1].view(torch.int16), c[1].view(torch.int16))
+    assert torch.equal(a[2].view(torch.int16), c[2].view(torch.int16))
+    flips = int((a[0] != c[0]).sum())
+    meta = int((a[3].view(torch.int16) != c[3].view(torch.int16)).sum()) + int((a[4].view(torch.int16) != c[4].view(torch.int16)).sum())
+    print("torch-vs-C(libm atan2f) flips: codes %d / %d, angle metadata %d" % (flips, a[0].numel(), meta))
     assert flips <= 1e-4 * a[0].numel() and meta <= 8
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_c_restatement_of_the_sleef_arctangent_rounds_like_torch(dtype):
+    """round_dtype(po_sleef_atan2f_u10(y, x)) == torch.atan2 on half / bfloat16 tensors (a library routine, not the
+    oracle's formula), on random operands over many exponents plus the special operands."""
+    g = torch.Generator().manual_seed(31)
+    n = 40000
+    e = torch.randint(-10, 6, (2, n), generator=g).float()
+    yx = (torch.randn(2, n, generator=g) * torch.exp2(e)).to(dtype)
+    special = torch.tensor([0.0, -0.0, 1.0, -1.0, float("inf"), -float("inf"), 6e-8, -6e-8, 65504.0], dtype=dtype)
+    y = torch.cat([yx[0], special.repeat_interleave(special.numel())])
+    x = torch.cat([yx[1], special.repeat(special.numel())])
+    want = torch.atan2(y, x)
+    got = co.sleef_atan2f(y.float(), x.float()).to(dtype)
+    assert torch.equal(want.view(torch.int16), got.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fp32_wrap_switch_of_both_restatements(dtype):
+    """The switch that adds 2*pi in fp32 (what an eager add on the GPU does) in the torch restatement and in the C one:
+    bit for bit the same codes and metadata, and different from the default wrap on a good share of the groups."""
+    k, _ = _keys(1, 2, 512, 9, dtype)
+    a = po.quantize_and_pack_nbit(k, 4, 4, wrap_fp32=True)
+    b = co.quantize(k, 4, 4, wrap_fp32=True)
+    assert torch.equal(a[0], b[0])
+    for x, y in zip(a[1:], b[1:]):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16))
+    d = po.quantize_and_pack_nbit(k, 4, 4)
+    assert int((a[3].view(torch.int16) != d[3].view(torch.int16)).sum()) > 0
 
 
 def test_rope_pair_convention_matches_hf_rotate_half():

@@ -3,6 +3,8 @@
 Bar: packed codes and the four metadata tensors bit-exact.  Any disagreement
 is an "edge flip"; flips are counted and the target (asserted) is 0.
 """
+import math
+
 import pytest
 import torch
 
@@ -126,32 +128,93 @@ def test_quantize_uniform_angle_mode(gpu, dtype, rbits, tbits):
     assert rel < (0.15 if tbits == 4 else 0.3), rel    # quantization noise of a fixed 2*pi/2^t grid
 
 
-def test_quantize_wrap_fp32_flag(gpu):
-    """PQ_WRAP_FP32 adds 2*pi in fp32 (what an eager GPU add of a half tensor and a
-    python float does); checked against the plain-C oracle's same switch."""
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,rbits,tbits,theta", [((1, 2, 512), 4, 4, 1e4), ((2, 4, 1024), 3, 3, 1e6), ((1, 8, 2048), 4, 4, 5e5)])
+def test_quantize_wrap_fp32_flag(gpu, dtype, shape, rbits, tbits, theta):
+    """PQ_WRAP_FP32 adds 2*pi in fp32 (what an eager GPU add of a half tensor and a python float does): bit for bit
+    the codes and metadata of both CPU restatements with the same switch (torch ops; plain C with its own SLEEF
+    arctangent)."""
     from oracle import c_oracle as co
+    print("case wrap_fp32", dtype, shape, rbits, tbits, flush=True)
     g = torch.Generator().manual_seed(2)
-    k = wl.make_keys(1, 2, 512, 1e4, g)
-    ref = co.quantize(k, 4, 4, wrap_fp32=True)
-    got = quantize_and_pack_nbit(k.to(gpu), 4, 4, wrap_fp32=True)
-    flips = count_flips(got, ref)
-    # libm atan2f (C oracle) vs the SLEEF restatement may differ in the last ulp: allow a handful, report them
-    print("wrap_fp32 flips vs C oracle", flips, flush=True)
-    assert flips["codes"] <= 4 and flips["rscale"] == 0 and flips["rmn"] == 0
+    k = wl.make_keys(*shape, theta, g, dtype)
+    got = quantize_and_pack_nbit(k.to(gpu), rbits, tbits, wrap_fp32=True)
+    for name, ref in (("torch", po.quantize_and_pack_nbit(k, rbits, tbits, wrap_fp32=True)), ("C", co.quantize(k, rbits, tbits, wrap_fp32=True))):
+        flips = count_flips(got, ref)
+        print("wrap_fp32 flips vs", name, "oracle", flips, flush=True)
+        assert all(v == 0 for v in flips.values()), (name, flips)
+
+
+def _reference_lines_on_device(key_states, rbits, tbits, G=128):
+    """models/modeling_llama_polar.py:141-155 as plain eager torch ops, meant to be called with tensors ON THE GPU:
+    torch-ROCm's own kernels (a library, not the reference) then evaluate each line the way the reference's lines
+    are evaluated when the model runs on a GPU.  Degenerate groups (0/0 -> uint8) are avoided by the callers."""
+    B, N, L, D = key_states.shape
+    D = D // 2
+    ks = key_states.view(B, N, L // G, G, 2, D)
+    phi = torch.atan2(ks[:, :, :, :, 1, :], ks[:, :, :, :, 0, :])
+    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)
+    tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]
+    tscale = (tmx - tmn) / (2 ** tbits)
+    theta = torch.clamp(torch.floor((phi - tmn) / tscale).to(torch.uint8), 0, 2 ** tbits - 1)
+    radii = torch.norm(ks, p=2, dim=-2)
+    rmx, rmn = radii.max(-2, keepdim=True)[0], radii.min(-2, keepdim=True)[0]
+    rscale = (rmx - rmn) / (2 ** rbits)
+    rho = torch.clamp(torch.floor((radii - rmn) / rscale).to(torch.uint8), 0, 2 ** rbits - 1)
+    return (rho << tbits) + theta, rscale, rmn, tscale, tmn
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("cfg,rbits,tbits", [(0, 4, 4), (2, 3, 3)])
+def test_quantize_eager_gpu_mode_against_eager_torch_on_the_device(gpu, dtype, cfg, rbits, tbits):
+    """eager_gpu=True (PQ_WRAP_FP32 | PQ_DEVICE_ATAN2) against the reference's lines evaluated by eager torch ops on
+    device tensors, on the keys of configs[0] (all 8.4 M codes) and a configs[2]-like shape.  The radius side and
+    its metadata must be identical; the angle side can only differ where the device library's atan2f linked into
+    this library and the one inside torch differ, which is counted, printed and required to be nil.  The default
+    (CPU-eager) mode is measured against the same device evaluation and reported: that distance is why the
+    switch exists."""
+    print("case eager gpu", dtype, cfg, flush=True)
+    sh = wl.CONFIGS[cfg]
+    g = torch.Generator().manual_seed(sh.seed)
+    k = wl.make_keys(1, sh.n_kv_heads, 4096, sh.rope_theta, g, dtype).to(gpu)
+    ref = _reference_lines_on_device(k, rbits, tbits)
+    got = quantize_and_pack_nbit(k, rbits, tbits, eager_gpu=True)
+    torch.cuda.synchronize()
+    flips = count_flips([t.cpu() for t in got], [t.cpu() for t in ref])
+    base = count_flips([t.cpu() for t in quantize_and_pack_nbit(k, rbits, tbits)], [t.cpu() for t in ref])
+    rho_flips = int(((got[0] >> tbits) != (ref[0] >> tbits)).sum())
+    print("eager_gpu mode vs eager torch on the device:", flips, "radius-code flips", rho_flips, "| default (CPU-eager) mode vs the same:", base, flush=True)
+    assert rho_flips == 0 and flips["rscale"] == 0 and flips["rmn"] == 0
+    assert all(v == 0 for v in flips.values()), flips
+
+
+def test_quantize_device_atan2_flag_alone(gpu):
+    """PQ_DEVICE_ATAN2 without the fp32 wrap differs from the default only through the arctangent: a few angle codes
+    and angle metadata words per million, never the radius side."""
+    g = torch.Generator().manual_seed(41)
+    k = wl.make_keys(1, 8, 4096, 5e5, g).to(gpu)
+    a = quantize_and_pack_nbit(k, 4, 4)
+    b = quantize_and_pack_nbit(k, 4, 4, device_atan2=True)
+    flips = count_flips([t.cpu() for t in b], [t.cpu() for t in a])
+    print("device atan2f vs SLEEF atan2f:", flips, flush=True)
+    assert flips["rscale"] == 0 and flips["rmn"] == 0 and int(((a[0] >> 4) != (b[0] >> 4)).sum()) == 0
+    assert flips["codes"] <= 1e-4 * a[0].numel()
 
 
 @pytest.mark.parametrize("dtype_code,name", [(0, "float16"), (1, "bfloat16")])
 def test_quantizer_math_selftest_exhaustive(gpu, dtype_code, name):
     """The cheap-estimate-with-guard path against the exact path on all 2^32 operand pairs of the dtype."""
     from polarquant_amd import _ffi
-    counters = torch.zeros(3, dtype=torch.int64, device=gpu)
+    counters = torch.zeros(5, dtype=torch.int64, device=gpu)
     rc = _ffi.lib().pq_selftest_quantizer_math(dtype_code, counters.data_ptr(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
-    bad, slow, bad_div = counters.tolist()
-    print("%s: %d mismatching pairs, %.3f%% of pairs take the exact path, %d mismatching quotients"
-          % (name, bad, 100.0 * slow / 2 ** 32, bad_div), flush=True)
+    bad, slow, bad_div, bad_dev, slow_dev = counters.tolist()
+    print("%s: %d mismatching pairs, %.3f%% of pairs take the exact path, %d mismatching quotients; with the device "
+          "library's atan2f as the exact routine: %d mismatching pairs, %.3f%% take the exact path"
+          % (name, bad, 100.0 * slow / 2 ** 32, bad_div, bad_dev, 100.0 * slow_dev / 2 ** 32), flush=True)
     assert bad == 0
+    assert bad_dev == 0
     assert bad_div == 0     # reciprocal + two fused multiply-adds against the fp32 division, every (dividend, scale) pair
 
 

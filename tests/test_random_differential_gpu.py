@@ -17,6 +17,8 @@ SEEDS = range(int(os.environ.get("PQ_RANDOM_FIRST", "0")),
               int(os.environ.get("PQ_RANDOM_FIRST", "0")) + int(os.environ.get("PQ_RANDOM_CASES", "24")))
 HEADS = [(1, 1), (2, 1), (4, 4), (8, 2), (3, 1), (6, 1), (7, 1), (8, 1), (16, 2), (12, 4)]
 BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 4)]
+# dtype -> [attention cases run, cases that needed the widened band, output elements that needed it]
+WIDENED = {"float16": [0, 0, 0], "bfloat16": [0, 0, 0]}
 
 
 @pytest.mark.parametrize("seed", SEEDS)
@@ -81,7 +83,7 @@ def test_random_decode_attention_case(gpu, seed):
         # from the exact one, and the first-order bound for its rounding of the window's scores (:79)
         v_all = v if not values4 else (vr if not nb else torch.cat([po.dequantize_values(*vq, 4, torch.float64), vr.double()], dim=2))
         band = po.residual_score_rounding_band(q[b:b + 1], kr, *quant, v_all, mb, rb, tb)
-        refs.append((exact, torch.maximum((literal.double() - exact).abs(), band)))
+        refs.append((exact, torch.maximum((literal.double() - exact).abs(), band), literal.double()))
     dev = lambda t: t.to(gpu)
     kw = dict(rbits=rb, tbits=tb, n_splits=n_splits, attention_mask=dev(mask) if use_mask else None)
     if ragged:
@@ -103,14 +105,35 @@ def test_random_decode_attention_case(gpu, seed):
     # reference path's own half-precision evaluation from it (scores of the residual window and
     # probabilities rounded to the dtype matter when only a few dozen tokens are attended to)
     rtol, atol = (1e-2, 1e-3) if dtype == torch.float16 else (2e-2, 4e-3)
+    name = "float16" if dtype == torch.float16 else "bfloat16"
+    needed = 0
     for b in range(B):
-        exact, ref_noise = refs[b]
+        exact, ref_noise, literal = refs[b]
         err = (out[b:b + 1].double() - exact).abs()
         over = err - (atol + rtol * exact.abs() + ref_noise)
         bad = int((over > 0).sum())
         worst = int(over.argmax())
         assert bad == 0, (b, bad, float(err.max()), "worst element: got %r exact %r reference-path noise %r" % (
             float(out[b:b + 1].double().flatten()[worst]), float(exact.flatten()[worst]), float(ref_noise.flatten()[worst])))
+        # elements that meet the plain tolerance neither against the exact value nor against the reference path's own
+        # (literal, half-precision) evaluation, which is what parity is stated against
+        err_lit = (out[b:b + 1].double() - literal).abs()
+        needed += int(((err > atol + rtol * exact.abs()) & (err_lit > atol + rtol * literal.abs())).sum())
+    WIDENED[name][0] += 1
+    WIDENED[name][1] += int(needed > 0)
+    WIDENED[name][2] += needed
+    # float16 is the dtype the stated tolerance (rtol 1e-2 / atol 1e-3) is for: there every element must meet it as it
+    # stands against the reference path's own evaluation or against the fp64 value, with no first-order allowance
+    if dtype == torch.float16:
+        assert needed == 0, "float16 case needs the widened band on %d output elements" % needed
+
+
+def test_random_widened_band_report(gpu):
+    """How many of the attention cases above were inside the stated tolerance only thanks to the allowance for the
+    reference path's own half-precision roundings: printed per dtype; for float16 it has to be none."""
+    for name, (cases, cases_needing, elements) in WIDENED.items():
+        print("%s: %d cases, %d needed the widened band (%d output elements)" % (name, cases, cases_needing, elements), flush=True)
+    assert WIDENED["float16"][1] == 0
 
 
 @pytest.mark.parametrize("seed", SEEDS)
@@ -142,6 +165,19 @@ def test_random_quantizer_case(gpu, seed):
     for name, a, b in zip(["rscale", "rmn", "tscale", "tmn"], got[1:], ref[1:]):
         a, b = a.cpu().float(), b.float()
         assert bool(((a == b) | (a.isnan() & b.isnan())).all()), name
+    if mode == "group":
+        # the same keys in the mode that follows eager torch on GPU tensors, against eager torch ops on the device
+        # (0/0 groups, undefined in the reference, are left out: their metadata must agree, their codes need not)
+        from test_quantize_gpu import _reference_lines_on_device
+        xd = x.to(gpu)
+        dref = [t.cpu() for t in _reference_lines_on_device(xd, rb, tb)]
+        dgot = [t.cpu() for t in quantize_and_pack_nbit(xd, rb, tb, eager_gpu=True)]
+        for name, a, b in zip(["rscale", "rmn", "tscale", "tmn"], dgot[1:], dref[1:]):
+            a, b = a.float(), b.float()
+            assert bool(((a == b) | (a.isnan() & b.isnan())).all()), "eager-GPU mode: " + name
+        defined = (dref[1].float() > 0) & (dref[3].float() > 0) & dref[1].float().isfinite() & dref[3].float().isfinite()
+        dflips = int(((dgot[0] != dref[0]) & defined).sum())
+        assert dflips == 0, "eager-GPU mode: %d code flips against eager torch on the device" % dflips
     vref = po.quantize_values_along_last_dim(x)
     vgot = quantize_values(x.to(gpu))
     assert torch.equal(vgot[0].cpu(), vref[0]), "value code words differ: %d" % int((vgot[0].cpu() != vref[0]).sum())
