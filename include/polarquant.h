@@ -73,6 +73,18 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * sub-byte store it announces there.  Code tensors are then [B,Nk,capacity,128,48]. */
 #define PQ_CODES_PACKED6 4u
 
+/* flag for the attention entry points (pq_decode_attn and its variants): the context slices are cut on
+ * the device from the per-sequence counts, so that every wavefront gets the same number of groups
+ * whatever the lengths are (ragged batches; batches that grow under a replayed graph).  All planes
+ * ((sequence, KV head) pairs) are laid end to end, one unit per quantized group plus one for a
+ * sequence's residual keys, and the line is cut into equal segments, one per wavefront the device holds
+ * at once; a segment may end one plane and begin the next.  n_splits is then the number of partial
+ * slots per query head (>= 2): no plane is cut into more pieces than that (the segment length is raised
+ * to ceil((group_capacity + 1) / (n_splits - 1)) if it has to be), min_groups_per_split a lower bound
+ * on the segment length.  Results do not depend on how the line is cut beyond fp32 summation order.
+ * No reference counterpart (the reference has no split over the context at all). */
+#define PQ_BALANCED_SLICES 16u
+
 /* Linear layer of a decode step: y[M, N] = x[M, K] . w[N, K]^T (+ bias[N]), M <= 16 rows (one new
  * token per sequence), fp32 accumulation, one rounding to the dtype.  Replaces the q/k/v, o and MLP
  * projections (`nn.Linear`) the decode step calls around the attention
@@ -192,7 +204,7 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  * The caller has already appended the step's new key to the residual buffer
  * and the new value to the V cache (reference :77,98).
  *
- *   q        [B,N,128] half words, contiguous
+ *   q        [B,N,128] half words, contiguous, 16-byte aligned
  *   codes    u8, (batch,head) plane stride = group_capacity*128*64; meta likewise
  *            with plane stride group_capacity*64; may be NULL when no sequence has
  *            a quantized group
@@ -217,7 +229,8 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *            ceil(groups / n_splits)) always covers the sequence.
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
- *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48)
+ *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48) and / or
+ *            PQ_BALANCED_SLICES (slices cut on the device from the per-sequence counts, see above)
  * Limits: v_capacity <= PQ_MAX_PLANE_TOKENS tokens and group_capacity <= 2^17 groups per (batch, KV head)
  * plane (32-bit byte sizes and offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */

@@ -51,6 +51,14 @@ def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.
     return ws
 
 
+def balanced_slots(B: int, Nk: int, group_capacity: int, total_groups: Optional[int], wave_slots: int) -> int:
+    """Partial slots per head for PQ_BALANCED_SLICES: enough for the segment length the device will pick
+    when the batch holds `total_groups` groups per KV head (None: sequences half full on average)."""
+    units = (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + B
+    seg = max(1, -(-units * Nk // max(wave_slots, 1)))
+    return max(2, -(-(group_capacity + 1) // seg) + 1)
+
+
 def _pick_workspace(workspace: Optional[torch.Tensor], B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
     if workspace is None:
         return workspace_for(B, N, n_splits, device)
@@ -74,7 +82,7 @@ def polar_decode_attention(
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
     total_groups: Optional[int] = None, min_groups_per_split: Optional[int] = None,
-    workspace: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None, balanced: Optional[bool] = None,
 ) -> torch.Tensor:
     """-> attention output [B,N,1,128] in the query dtype.
 
@@ -82,6 +90,9 @@ def polar_decode_attention(
     counts if the caller knows it on the host (no device sync is made here), lets the context be
     cut into slices of equal size across sequences, so that short sequences do not leave
     wavefronts idle; without it the average sequence is assumed to be half the capacity.
+    `balanced` (the default with per-sequence counts and no explicit split): the slices are cut on the
+    device from the actual counts so that all wavefronts get equal work (PQ_BALANCED_SLICES);
+    `n_splits` is then the number of partial slots per head.
     `workspace`: a buffer from `new_workspace` that the caller owns (needed under graph capture);
     by default the cached buffer of the current stream is used."""
     if not query_states.is_cuda:
@@ -93,8 +104,8 @@ def polar_decode_attention(
     assert hd == 128
     dt = _dtype_code(query_states)
     q = query_states.reshape(B, N, hd)
-    if not q.is_contiguous():
-        q = q.contiguous()
+    if not q.is_contiguous() or q.data_ptr() % 16:
+        q = q.clone(memory_format=torch.contiguous_format)
     assert value_states.is_contiguous() and value_states.dtype == query_states.dtype
     v_cap = value_states.shape[2]
     if indices is not None:
@@ -118,7 +129,13 @@ def polar_decode_attention(
         sm_scale = 1.0 / math.sqrt(hd)
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
     min_gps = 0
-    if n_groups_per_seq is not None and n_splits is None and max_groups > 0:
+    if balanced is None:
+        balanced = n_groups_per_seq is not None and n_splits is None and min_groups_per_split is None
+    if balanced:
+        flags |= _ffi.PQ_BALANCED_SLICES
+        if n_splits is None:
+            n_splits = balanced_slots(B, Nk, max_groups, total_groups, 4 * _num_cus(dev))
+    elif n_groups_per_seq is not None and n_splits is None and max_groups > 0:
         tot = total_groups if total_groups is not None else (B * max_groups + 1) // 2
         # one wavefront per SIMD; every (sequence, KV head) rounds its slice count up, so leave one
         # slot per plane for that and the whole batch still runs in a single round
@@ -156,7 +173,7 @@ def polar_decode_attention_v4(
     rbits: int = 4, tbits: int = 4, sm_scale: Optional[float] = None,
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None, min_groups_per_split: int = 0,
-    workspace: Optional[torch.Tensor] = None,
+    workspace: Optional[torch.Tensor] = None, balanced: bool = False, total_groups: Optional[int] = None,
 ) -> torch.Tensor:
     """Decode attention of the reference's Mixed variant (polar keys + 4-bit values,
     models/modeling_llama_polar.py:185-241) -> [B,N,1,128] in the query dtype."""
@@ -169,8 +186,8 @@ def polar_decode_attention_v4(
     assert hd == 128
     dt = _dtype_code(query_states)
     q = query_states.reshape(B, N, hd)
-    if not q.is_contiguous():
-        q = q.contiguous()
+    if not q.is_contiguous() or q.data_ptr() % 16:
+        q = q.clone(memory_format=torch.contiguous_format)
     assert key_resid.is_contiguous() and value_resid.is_contiguous() and key_resid.shape == value_resid.shape
     assert key_resid.dtype == query_states.dtype == value_resid.dtype
     r_cap = key_resid.shape[2]
@@ -192,6 +209,10 @@ def polar_decode_attention_v4(
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(hd)
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
+    if balanced:
+        flags |= _ffi.PQ_BALANCED_SLICES
+        if n_splits is None:
+            n_splits = balanced_slots(B, Nk, max_groups, total_groups, (8 if N // Nk <= 4 else 4) * _num_cus(dev))
     if n_splits is None:
         n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, N, Nk, max(max_groups, 1), _num_cus(dev))
     ws = _pick_workspace(workspace, B, N, n_splits, dev)

@@ -310,73 +310,71 @@ struct V4Args {
     int64_t capacity;          // tokens per (batch, KV head) plane
 };
 
-template <typename T, int TB, int REPP, bool V4, bool PK6>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
-void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
-                 const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
-                 const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
-                 int group_capacity, int n_groups, const int32_t* __restrict__ n_groups_per_seq,
-                 const uint16_t* __restrict__ k_resid, int resid_capacity, int n_resid,
-                 const int32_t* __restrict__ n_resid_per_seq,
-                 const uint16_t* __restrict__ v, int64_t v_capacity,
-                 const uint8_t* __restrict__ mask, int64_t mask_stride,
-                 float scale_log2, int N, int Nk, int rep, int n_splits, int min_gps, float* __restrict__ ws,
-                 V4Args v4) {
-    // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
-    // residual window, row 0 = first residual token; otherwise `v` holds every row.
-    using L = Lut<TB, REPP>;
-    // the table region doubles as the fp32 query buffer of the residual block
-    constexpr int kLutBytes = L::BYTES > REPP * kHeadDim * 4 ? L::BYTES : REPP * kHeadDim * 4;
-    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
-    __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
-    const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
+// Everything a wavefront needs to know about the call (the kernels' arguments).
+struct AttnParams {
+    const uint16_t* q;
+    const uint8_t* codes;
+    const uint16_t *rscale, *rmn, *tscale, *tmn;
+    int group_capacity, n_groups;
+    const int32_t* n_groups_per_seq;
+    const uint16_t* k_resid;
+    int resid_capacity, n_resid;
+    const int32_t* n_resid_per_seq;
+    const uint16_t* v;
+    int64_t v_capacity;
+    const uint8_t* mask;
+    int64_t mask_stride;
+    float scale_log2;
+    int B, N, Nk, rep, n_splits, min_gps;
+    float* ws;
+};
 
-    const int lane = threadIdx.x;
-    // 1-D grid, (batch, KV head) index fastest.  Consecutive workgroup ids go to different XCDs, so
-    // every XCD receives whole (batch, KV head) planes with all their slices; with the slice index
-    // fastest an XCD would receive one slice index of every plane, and in a ragged batch the XCDs
-    // that own the high slice indices would sit idle (measured: 165 us instead of 120 us).
-    const int units = gridDim.x / n_splits;
-    const int bh = blockIdx.x % units;
-    const int split = blockIdx.x / units;
-    const int b = bh / Nk, kvh = bh - b * Nk;
-
-    int nb = n_groups_per_seq ? n_groups_per_seq[b] : n_groups;
-    nb = nb < 0 ? 0 : (nb > group_capacity ? group_capacity : nb);
-    int nres = n_resid_per_seq ? n_resid_per_seq[b] : n_resid;
-    nres = nres < 0 ? 0 : (nres > resid_capacity ? resid_capacity : nres);
+// Token counts of one sequence as the kernels use them: groups and residual keys clamped to the
+// capacities, tokens clamped to what the value plane holds.
+struct SeqCounts { int nb, nres; int64_t n_tokens; };
+template <bool V4>
+__device__ __forceinline__ SeqCounts seq_counts(const AttnParams& p, const V4Args& v4, int b) {
+    SeqCounts c;
+    int nb = p.n_groups_per_seq ? p.n_groups_per_seq[b] : p.n_groups;
+    nb = nb < 0 ? 0 : (nb > p.group_capacity ? p.group_capacity : nb);
+    int nres = p.n_resid_per_seq ? p.n_resid_per_seq[b] : p.n_resid;
+    nres = nres < 0 ? 0 : (nres > p.resid_capacity ? p.resid_capacity : nres);
     int64_t n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
     if (V4) {
         nb = static_cast<int64_t>(nb) * kGroup > v4.capacity ? static_cast<int>(v4.capacity / kGroup) : nb;
-        nres = nres > v_capacity ? static_cast<int>(v_capacity) : nres;
+        nres = nres > p.v_capacity ? static_cast<int>(p.v_capacity) : nres;
         n_tokens = static_cast<int64_t>(nb) * kGroup + nres;
     } else {
-        n_tokens = n_tokens > v_capacity ? v_capacity : n_tokens;   // never read past the (batch, head) plane of V
+        n_tokens = n_tokens > p.v_capacity ? p.v_capacity : n_tokens;   // never read past the (batch, head) plane of V
     }
+    c.nb = nb; c.nres = nres; c.n_tokens = n_tokens;
+    return c;
+}
 
-    // slices past the end of a short sequence have nothing to do: mark their partials empty and leave
-    {
-        int gps = (nb + n_splits - 1) / n_splits;
-        gps = gps < min_gps ? min_gps : gps;
-        if (split > 0 && split * gps >= nb) {
-            if (lane < rep) {
-                // both header words: the workspace is not cleared between calls, and the merge must not
-                // meet a stale probability sum (0 * NaN) in a slice that holds nothing
-                float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats;
-                pw[0] = -INFINITY;
-                pw[1] = 0.0f;
-            }
-            return;
-        }
-    }
+// One piece of work of a wavefront: quantized groups [g0, g1) of (sequence b, KV head kvh), then,
+// if do_resid, the half-precision residual keys of that sequence; the partial result (m, l, acc) of
+// each of the `rep` query heads goes to partial slot `slot` of its head.
+template <typename T, int TB, int REPP, bool V4, bool PK6>
+__device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4, uint32_t lut, uint32_t pbuf, int lane,
+                                           int b, int kvh, const SeqCounts& sc, int g0, int g1, bool do_resid, int slot) {
+    // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
+    // residual window, row 0 = first residual token; otherwise `v` holds every row.
+    const int N = p.N, Nk = p.Nk, rep = p.rep, n_splits = p.n_splits;
+    const int bh = b * Nk + kvh;
+    const int nb = sc.nb, nres = sc.nres;
+    const int64_t n_tokens = sc.n_tokens;
+    const int64_t v_capacity = p.v_capacity;
+    const int group_capacity = p.group_capacity, resid_capacity = p.resid_capacity;
+    const float scale_log2 = p.scale_log2;
+    float* ws = p.ws;
 
-    const uint16_t* qb = q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
-    const __amdgpu_buffer_rsrc_t rv = make_rsrc(v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
+    const uint16_t* qb = p.q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
+    const __amdgpu_buffer_rsrc_t rv = make_rsrc(p.v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
                                                 static_cast<uint32_t>((V4 ? nres : n_tokens) * (kHeadDim * 2)));
     const uint32_t voff_v = static_cast<uint32_t>(lane >> 4) * (4 * kHeadDim * 2) + static_cast<uint32_t>(lane & 15) * 16;
-    const bool has_mask = mask != nullptr;
-    const __amdgpu_buffer_rsrc_t rm = make_rsrc(has_mask ? mask + static_cast<size_t>(b) * mask_stride : nullptr,
-                                                has_mask ? static_cast<uint32_t>(n_tokens < mask_stride ? n_tokens : mask_stride) : 0u);
+    const bool has_mask = p.mask != nullptr;
+    const __amdgpu_buffer_rsrc_t rm = make_rsrc(has_mask ? p.mask + static_cast<size_t>(b) * p.mask_stride : nullptr,
+                                                has_mask ? static_cast<uint32_t>(n_tokens < p.mask_stride ? n_tokens : p.mask_stride) : 0u);
 
     AttnState<REPP> st;
 #pragma unroll
@@ -386,12 +384,6 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
 
     {
         // ---------------- quantized groups [g0, g1) ----------------
-        // groups per slice: an even split of this sequence, but never fewer than min_gps (ragged
-        // batches: short sequences then use fewer slices, and the unused blocks return at once)
-        int gps = (nb + n_splits - 1) / n_splits;
-        gps = gps < min_gps ? min_gps : gps;
-        const int g0 = split * gps;
-        const int g1 = (g0 + gps) < nb ? (g0 + gps) : nb;
         if (g0 < g1) {
             float qx[REPP], qy[REPP];
 #pragma unroll
@@ -403,17 +395,17 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             const size_t plane = static_cast<size_t>(bh) * group_capacity;
             // a token's code row: 64 bytes, or 48 when the 6-bit codes are stored packed
             constexpr int kRowB = PK6 ? kPackedRowBytes : kPairs, kRowLoads = kRowB / 16;
-            const __amdgpu_buffer_rsrc_t rc = make_rsrc(codes + plane * (kGroup * kRowB),
+            const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.codes + plane * (kGroup * kRowB),
                                                         static_cast<uint32_t>(nb) * (kGroup * kRowB));
             const uint32_t voff_c = static_cast<uint32_t>(lane) * kRowB;
             // software pipeline: codes of the next tile and metadata of the next group are in flight
             uint4 cnext[kRowLoads];
 #pragma unroll
             for (int i = 0; i < kRowLoads; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(g0) * (kGroup * kRowB) + 16 * i);
-            const uint16_t* prs = rscale + plane * kPairs + lane;
-            const uint16_t* prm = rmn + plane * kPairs + lane;
-            const uint16_t* pts = tscale + plane * kPairs + lane;
-            const uint16_t* ptm = tmn + plane * kPairs + lane;
+            const uint16_t* prs = p.rscale + plane * kPairs + lane;
+            const uint16_t* prm = p.rmn + plane * kPairs + lane;
+            const uint16_t* pts = p.tscale + plane * kPairs + lane;
+            const uint16_t* ptm = p.tmn + plane * kPairs + lane;
             uint16_t mrs = prs[g0 * kPairs], mrm = prm[g0 * kPairs], mts = pts[g0 * kPairs], mtm = ptm[g0 * kPairs];
             // V operands are double-buffered by tile parity: tile t+1 is requested before tile t is scored
             VTile<V4> vv[2];
@@ -502,63 +494,61 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             if constexpr (V4) finish_v4<REPP>(st, lane);
         }
     }
-    // the residual keys go to the block that holds the last quantized group of the sequence
-    int last_split = 0;
-    {
-        int gps = (nb + n_splits - 1) / n_splits;
-        gps = gps < min_gps ? min_gps : gps;
-        last_split = nb > 0 ? (nb - 1) / gps : 0;
-    }
-    if (split == last_split && nres > 0) {
-        // ---------------- fp16 residual keys ----------------
+    if (do_resid && nres > 0) {
+        // ---------------- residual keys (model dtype) ----------------
+        // scores = K . q^T on the matrix cores, as the reference's half-precision matmul (:79): for 16 tokens
+        // at a time D[token][head] += K[token][16 dims] * q[head][16 dims], heads padded to the 16 columns.
+        // Lane (g,n) supplies, for step (kb, hf), dims 32 kb + 8 g + 4 hf .. +3 of key row n and of query head
+        // n: both operands use the same order of the contraction index, so one 16-byte load per lane feeds two
+        // MFMAs, and the four lanes of a row read 64 contiguous bytes.  All 16 loads of a 64-token tile are
+        // in flight at once.  The D tiles go through LDS (the table region) to the lane == token layout.
         asm volatile("" ::: "memory");
-        // q as fp32 in LDS: [REPP][128]
+        const int g = lane >> 4, n = lane & 15;
+        uint4 qv[4];
 #pragma unroll
-        for (int j = 0; j < REPP; j++) {
-            const bool ok = j < rep;
-            *lds_ptr<lds_f1>(lut + (j * kHeadDim + lane) * 4) = ok ? lo2f<T>(qb[j * kHeadDim + lane]) : 0.0f;
-            *lds_ptr<lds_f1>(lut + (j * kHeadDim + kWave + lane) * 4) = ok ? lo2f<T>(qb[j * kHeadDim + kWave + lane]) : 0.0f;
+        for (int kb = 0; kb < 4; kb++) {
+            qv[kb] = (n < rep) ? *reinterpret_cast<const uint4*>(qb + n * kHeadDim + 32 * kb + 8 * g) : make_uint4(0u, 0u, 0u, 0u);
         }
-        asm volatile("" ::: "memory");
-        const __amdgpu_buffer_rsrc_t rk = make_rsrc(k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(p.k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
                                                     static_cast<uint32_t>(nres) * (kHeadDim * 2));
+        const uint32_t voff_k = static_cast<uint32_t>(n) * (kHeadDim * 2) + static_cast<uint32_t>(g) * 16;
         const int n_tiles = (nres + kWave - 1) / kWave;
         for (int tt = 0; tt < n_tiles; tt++) {
             const int tok = tt * kWave + lane;
             const bool valid = tok < nres;
             const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
+            uint4 kk[4][4];
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+                for (int kb = 0; kb < 4; kb++)
+                    kk[tb][kb] = buf_load16(rk, voff_k, static_cast<uint32_t>(tt * kWave + 16 * tb) * (kHeadDim * 2) + 64 * kb);
             uint4 vv[4][4];
             load_v_tile(vv, rv, voff_v, (V4 ? static_cast<uint32_t>(tt * kWave) : arow) * (kHeadDim * 2));
-            float s[REPP];
 #pragma unroll
-            for (int j = 0; j < REPP; j++) s[j] = 0.0f;
-#pragma unroll 4
-            for (int c = 0; c < 16; c++) {
-                const uint4 kw = buf_load16(rk, static_cast<uint32_t>(tok) * (kHeadDim * 2), 16 * c);
-                const uint32_t w[4] = {kw.x, kw.y, kw.z, kw.w};
-                float kf[8];
+            for (int tb = 0; tb < 4; tb++) {
+                floatx4 d = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    kf[2 * i] = lo2f<T>(static_cast<uint16_t>(w[i] & 0xffffu));
-                    kf[2 * i + 1] = lo2f<T>(static_cast<uint16_t>(w[i] >> 16));
+                for (int kb = 0; kb < 4; kb++) {
+                    d = mfma16<T>(make_uint2(kk[tb][kb].x, kk[tb][kb].y), make_uint2(qv[kb].x, qv[kb].y), d);
+                    d = mfma16<T>(make_uint2(kk[tb][kb].z, kk[tb][kb].w), make_uint2(qv[kb].z, qv[kb].w), d);
                 }
-#pragma unroll
-                for (int j = 0; j < REPP; j++) {
-                    const lds_e4* qa = lds_ptr<lds_e4>(lut + (j * kHeadDim + 8 * c) * 4);
-                    const lds_e4* qc = lds_ptr<lds_e4>(lut + (j * kHeadDim + 8 * c + 4) * 4);
-                    s[j] = __builtin_fmaf(qa->x, kf[0], s[j]); s[j] = __builtin_fmaf(qa->y, kf[1], s[j]);
-                    s[j] = __builtin_fmaf(qa->z, kf[2], s[j]); s[j] = __builtin_fmaf(qa->w, kf[3], s[j]);
-                    s[j] = __builtin_fmaf(qc->x, kf[4], s[j]); s[j] = __builtin_fmaf(qc->y, kf[5], s[j]);
-                    s[j] = __builtin_fmaf(qc->z, kf[6], s[j]); s[j] = __builtin_fmaf(qc->w, kf[7], s[j]);
+                // d[i] = score of token 16 tb + 4 g + i for head n
+                if (n < REPP) {
+                    lds_e4* dst = lds_ptr<lds_e4>(lut + (n * kWave + 16 * tb + 4 * g) * 4);
+                    dst->x = d[0]; dst->y = d[1]; dst->z = d[2]; dst->w = d[3];
                 }
             }
+            asm volatile("" ::: "memory");
             const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(arow), 0) != 0) : true);
+            float s[REPP];
 #pragma unroll
             for (int j = 0; j < REPP; j++) {
                 // the reference multiplies q.K^T in the model dtype before promoting (:79)
-                const float sr = lo2f<T>(f2lo<T>(s[j]));
+                const float sr = lo2f<T>(f2lo<T>(*lds_ptr<lds_f1>(lut + (j * kWave + lane) * 4)));
                 s[j] = keep ? sr * scale_log2 : -INFINITY;
             }
+            asm volatile("" ::: "memory");
             softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
         }
     }
@@ -572,7 +562,7 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
         float mm = st.m[0], ll = lsum[0];
 #pragma unroll
         for (int j = 1; j < REPP; j++) { mm = (n == j) ? st.m[j] : mm; ll = (n == j) ? lsum[j] : ll; }
-        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * n_splits + split) * kPartialFloats;
+        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * n_splits + slot) * kPartialFloats;
         if (g == 0) { pw[0] = mm; pw[1] = ll; }
         float* pa = pw + 4 + 32 * g;
 #pragma unroll
@@ -580,6 +570,193 @@ void attn_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ cod
             *reinterpret_cast<float4*>(pa + 8 * i) = make_float4(st.acc[0][i], st.acc[1][i], st.acc[2][i], st.acc[3][i]);
             *reinterpret_cast<float4*>(pa + 8 * i + 4) = make_float4(st.acc[4][i], st.acc[5][i], st.acc[6][i], st.acc[7][i]);
         }
+    }
+}
+
+// Mark the partial slots [first, n_splits) of the `rep` query heads of (b, kvh) as holding nothing.
+// Both header words: the workspace is not cleared between calls, and the merge must not meet a
+// stale probability sum (0 * NaN) in a slot that holds nothing.
+__device__ __forceinline__ void mark_empty_slots(const AttnParams& p, int lane, int b, int kvh, int first) {
+    const int count = (p.n_splits - first) * p.rep;
+    for (int i = lane; i < count; i += kWave) {
+        const int j = i / (p.n_splits - first), s = first + i % (p.n_splits - first);
+        float* pw = p.ws + ((static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * p.rep + j) * p.n_splits + s) * kPartialFloats;
+        pw[0] = -INFINITY;
+        pw[1] = 0.0f;
+    }
+}
+
+#define PQ_ATTN_KERNEL_PARAMS                                                                                        \
+    const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes, const uint16_t* __restrict__ rscale,          \
+        const uint16_t* __restrict__ rmn, const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,     \
+        int group_capacity, int n_groups, const int32_t* __restrict__ n_groups_per_seq,                              \
+        const uint16_t* __restrict__ k_resid, int resid_capacity, int n_resid,                                       \
+        const int32_t* __restrict__ n_resid_per_seq, const uint16_t* __restrict__ v, int64_t v_capacity,             \
+        const uint8_t* __restrict__ mask, int64_t mask_stride, float scale_log2, int B, int N, int Nk, int rep,      \
+        int n_splits, int min_gps, float* __restrict__ ws, V4Args v4
+#define PQ_ATTN_KERNEL_PACK                                                                                          \
+    AttnParams p;                                                                                                    \
+    p.q = q; p.codes = codes; p.rscale = rscale; p.rmn = rmn; p.tscale = tscale; p.tmn = tmn;                        \
+    p.group_capacity = group_capacity; p.n_groups = n_groups; p.n_groups_per_seq = n_groups_per_seq;                 \
+    p.k_resid = k_resid; p.resid_capacity = resid_capacity; p.n_resid = n_resid; p.n_resid_per_seq = n_resid_per_seq; \
+    p.v = v; p.v_capacity = v_capacity; p.mask = mask; p.mask_stride = mask_stride; p.scale_log2 = scale_log2;      \
+    p.B = B; p.N = N; p.Nk = Nk; p.rep = rep; p.n_splits = n_splits; p.min_gps = min_gps; p.ws = ws
+
+// Even slices: block (plane bh, slice `split`) takes groups [split * gps, (split + 1) * gps) of its
+// sequence, gps = max(min_gps, ceil(groups / n_splits)); the block that holds the last group also
+// takes the residual keys.
+template <typename T, int TB, int REPP, bool V4, bool PK6>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
+void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
+    using L = Lut<TB, REPP>;
+    // the table region doubles as the staging buffer of the residual block's scores ([REPP][64] fp32)
+    constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
+    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
+    const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
+    PQ_ATTN_KERNEL_PACK;
+
+    const int lane = threadIdx.x;
+    // 1-D grid, (batch, KV head) index fastest.  Consecutive workgroup ids go to different XCDs, so
+    // every XCD receives whole (batch, KV head) planes with all their slices; with the slice index
+    // fastest an XCD would receive one slice index of every plane, and in a ragged batch the XCDs
+    // that own the high slice indices would sit idle (measured: 165 us instead of 120 us).
+    const int units = gridDim.x / n_splits;
+    const int bh = blockIdx.x % units;
+    const int split = blockIdx.x / units;
+    const int b = bh / Nk, kvh = bh - b * Nk;
+    const SeqCounts sc = seq_counts<V4>(p, v4, b);
+
+    // groups per slice: an even split of this sequence, but never fewer than min_gps (ragged
+    // batches: short sequences then use fewer slices, and the unused blocks return at once)
+    int gps = (sc.nb + n_splits - 1) / n_splits;
+    gps = gps < min_gps ? min_gps : gps;
+    // slices past the end of a short sequence have nothing to do: mark their partials empty and leave
+    if (split > 0 && split * gps >= sc.nb) {
+        if (lane < rep) {
+            float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats;
+            pw[0] = -INFINITY;
+            pw[1] = 0.0f;
+        }
+        return;
+    }
+    const int g0 = split * gps;
+    const int g1 = (g0 + gps) < sc.nb ? (g0 + gps) : sc.nb;
+    // the residual keys go to the block that holds the last quantized group of the sequence
+    const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
+    attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, b, kvh, sc, g0, g1, split == last_split, split);
+}
+
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// Balanced slices: the work of the whole batch is laid out as one line of units, plane after plane
+// (plane = (sequence, KV head), sequence-major); a sequence's plane holds one unit per quantized
+// group and one more for its residual keys if it has any (a sequence with nothing at all holds one
+// empty unit, so that somebody writes its partials).  The line is cut into segments of `seg` units,
+// the same for every wavefront; wavefront w works through segment w, which may end one plane and
+// begin the next: every piece of a plane it touches becomes one partial.  The piece of plane P cut
+// by segment w goes to slot w - floor(start of P / seg) of that plane's heads, and the piece that
+// ends P marks the slots behind it empty.
+//   seg = max(min_gps, ceil(line length / wavefronts), ceil((group_capacity + 1) / (n_splits - 1)))
+// the last term guarantees that no plane is cut into more than n_splits pieces (n_splits >= 2: a plane
+// shorter than a segment can still lie across one cut).  All of this is
+// computed from the per-sequence counts in device memory, by every wavefront alike, so the slices
+// follow the real lengths of a ragged or growing batch without the host knowing them.
+template <typename T, int TB, int REPP, bool V4, bool PK6>
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
+void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
+    using L = Lut<TB, REPP>;
+    constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
+    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
+    const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
+    PQ_ATTN_KERNEL_PACK;
+    const int lane = threadIdx.x;
+    const long long W = gridDim.x, w = blockIdx.x;
+
+    auto units_of = [&](int bb) {
+        const SeqCounts c = seq_counts<V4>(p, v4, bb);
+        const int u = c.nb + (c.nres > 0 ? 1 : 0);
+        return u > 0 ? u : 1;
+    };
+    // length of the line
+    int mine = 0;
+    for (int base = 0; base < B; base += kWave) mine += (base + lane < B) ? units_of(base + lane) : 0;
+    const long long per_head = wave_sum_i(mine);          // units of one KV head's planes, all sequences
+    const long long total = per_head * Nk;
+    long long seg = (total + W - 1) / W;
+    seg = seg < min_gps ? min_gps : seg;
+    const long long cap_units = static_cast<long long>(group_capacity) + 1;
+    const long long fit = (cap_units + n_splits - 2) / (n_splits - 1);      // n_splits >= 2 (checked on the host)
+    seg = seg < fit ? fit : seg;
+    const long long start = w * seg;
+    if (start >= total) return;
+    const long long end = (start + seg) < total ? (start + seg) : total;
+
+    // the sequence that holds unit `start`: units before sequence bb are Nk * (sum of u over earlier sequences)
+    int b = 0;
+    long long before = 0;                                  // units of one head's planes before sequence b
+    for (int base = 0; base < B; base += kWave) {
+        const int u = (base + lane < B) ? units_of(base + lane) : 0;
+        int incl = u;
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const int t = __shfl_up(incl, o);
+            incl += (lane >= o) ? t : 0;
+        }
+        const long long chunk = __shfl(incl, kWave - 1);
+        if (start < (before + chunk) * Nk) {
+            const unsigned long long past = __ballot((before + incl) * Nk > start);
+            const int l0 = __builtin_ctzll(past);
+            b = base + l0;
+            before += __shfl(incl - u, l0);
+            break;
+        }
+        before += chunk;
+    }
+    // The walk over the pieces of this segment keeps its state (6 integers) in LDS between pieces, so that
+    // nothing of it occupies registers inside a piece: the group loop already uses every scalar register.
+    __shared__ int walk[8];
+    {
+        const int u0 = units_of(b);
+        const long long seq_start = before * Nk;            // line position of plane (b, 0)
+        const int kvh0 = static_cast<int>((start - seq_start) / u0);
+        const long long plane_start = seq_start + static_cast<long long>(kvh0) * u0;
+        const long long span = end - start;
+        if (lane == 0) {
+            walk[0] = b; walk[1] = kvh0; walk[2] = static_cast<int>(start - plane_start); walk[3] = u0;
+            walk[4] = static_cast<int>(span < 0x7fffffffLL ? span : 0x7fffffffLL);          // units left in the segment
+            walk[5] = static_cast<int>(w - plane_start / seg);                               // slot of the first piece
+        }
+    }
+    for (;;) {
+        asm volatile("" ::: "memory");
+        const int cb = __builtin_amdgcn_readfirstlane(walk[0]), ckvh = __builtin_amdgcn_readfirstlane(walk[1]);
+        const int ua = __builtin_amdgcn_readfirstlane(walk[2]), u = __builtin_amdgcn_readfirstlane(walk[3]);
+        const int left = __builtin_amdgcn_readfirstlane(walk[4]), slot = __builtin_amdgcn_readfirstlane(walk[5]);
+        if (left <= 0 || cb >= B) break;
+        const int ub = (u - ua) < left ? u : ua + left;
+        asm volatile("" ::: "memory");
+        // the state of the next piece: a plane that begins inside this segment has its first piece here (slot 0)
+        {
+            int nb_ = cb, nk = ckvh, nu = u;
+            if (ub == u) {
+                if (++nk == Nk) { nk = 0; ++nb_; nu = nb_ < B ? units_of(nb_) : 1; }
+            }
+            if (lane == 0) {
+                walk[0] = nb_; walk[1] = nk; walk[2] = ub == u ? 0 : ub; walk[3] = nu;
+                walk[4] = left - (ub - ua); walk[5] = 0;
+            }
+        }
+        // the piece that ends its plane marks the slots behind its own as holding nothing
+        if (ub == u && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
+        const SeqCounts sc = seq_counts<V4>(p, v4, cb);
+        const int g0 = ua < sc.nb ? ua : sc.nb, g1 = ub < sc.nb ? ub : sc.nb;
+        attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, cb, ckvh, sc, g0, g1, ub > sc.nb, slot);
     }
 }
 #pragma clang diagnostic pop
@@ -653,20 +830,48 @@ __global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __rest
     out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : 0.0f);
 }
 
+// Wavefront slots of the current device for the balanced kernel: one wavefront per SIMD (4 per
+// compute unit), two for the 4-bit-value kernel with up to 4 query heads per KV head.
+static int device_compute_units() {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static int cus[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
 template <typename T, int TB>
 static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     const int rep = a.N / a.Nk;
     dim3 grid(static_cast<unsigned>(a.n_splits) * static_cast<unsigned>(a.B * a.Nk)), block(kWave);
+    if (a.balanced) {
+        // as many wavefronts as the device holds at once, but never more than there are partial slots
+        const long long slots = static_cast<long long>(device_compute_units()) * ((a.v4_codes && rep_pad(rep) <= 4) ? 8 : 4);
+        const long long most = static_cast<long long>(a.n_splits) * a.B * a.Nk;
+        grid = dim3(static_cast<unsigned>(slots < most ? slots : most));
+    }
     const float scale_log2 = a.sm_scale * kLog2e;
     V4Args v4{static_cast<const uint32_t*>(a.v4_codes), static_cast<const uint16_t*>(a.v4_scale),
               static_cast<const uint16_t*>(a.v4_zero), a.v4_capacity};
-#define PQ_LAUNCH_VP(REPP, V4, PK6)                                                                                  \
-    hipLaunchKernelGGL((attn_kernel<T, TB, REPP, V4, PK6>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,       \
+#define PQ_LAUNCH_K(KERNEL, REPP, V4, PK6)                                                                           \
+    hipLaunchKernelGGL((KERNEL<T, TB, REPP, V4, PK6>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,            \
                        (const uint16_t*)a.rscale, (const uint16_t*)a.rmn, (const uint16_t*)a.tscale,                 \
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
-                       (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.N, a.Nk, rep,        \
+                       (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
                        a.n_splits, a.min_groups_per_split, a.workspace, v4)
+#define PQ_LAUNCH_VP(REPP, V4, PK6)                                                                                  \
+    do {                                                                                                             \
+        if (a.balanced) PQ_LAUNCH_K(attn_balanced_kernel, REPP, V4, PK6);                                            \
+        else PQ_LAUNCH_K(attn_kernel, REPP, V4, PK6);                                                                \
+    } while (0)
     // packed 6-bit code rows exist for tbits == 3 only (the 3/3 configuration)
 #define PQ_LAUNCH_V(REPP, V4)                                                                                        \
     do {                                                                                                             \
@@ -691,6 +896,7 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
 #undef PQ_LAUNCH
 #undef PQ_LAUNCH_V
 #undef PQ_LAUNCH_VP
+#undef PQ_LAUNCH_K
     return static_cast<int>(hipGetLastError());
 }
 

@@ -15,8 +15,10 @@ int check_bits(int rbits, int tbits) {
 }
 
 // decode-side flags: only the packed 6-bit code layout, which exists for tbits == 3 (rbits <= 3)
-int check_decode_flags(unsigned flags, int rbits, int tbits) {
-    if (flags & ~static_cast<unsigned>(PQ_CODES_PACKED6)) return PQ_ERR_BAD_SHAPE;
+int check_decode_flags(unsigned flags, int rbits, int tbits, bool attention = false) {
+    // the score op has one slice per group; only the attention entry points cut the context
+    const unsigned known = PQ_CODES_PACKED6 | (attention ? PQ_BALANCED_SLICES : 0u);
+    if (flags & ~known) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && (tbits != 3 || rbits + tbits > 6)) return PQ_ERR_BAD_BITS;
     return PQ_OK;
 }
@@ -160,7 +162,7 @@ int pq_validate_decode_attn(const void* q,
                             int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
                             const void* out, unsigned flags) {
     if (!q || !v || !workspace || !out) return PQ_ERR_NULL_POINTER;
-    if (int rc = check_decode_flags(flags, rbits, tbits)) return rc;
+    if (int rc = check_decode_flags(flags, rbits, tbits, true)) return rc;
     if (int rc = check_heads(B, N, Nk)) return rc;
     if (static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
     if (int rc = check_bits(rbits, tbits)) return rc;
@@ -187,8 +189,11 @@ int pq_validate_decode_attn(const void* q,
         mask_stride < static_cast<int64_t>(n_groups) * PQ_GROUP + n_resid) return PQ_ERR_BAD_STRIDE;
     if (!(sm_scale == sm_scale)) return PQ_ERR_BAD_SHAPE;
     if (n_splits < 1 || n_splits > 65534 || min_groups_per_split < 0) return PQ_ERR_WORKSPACE;
+    // balanced slices: a plane shorter than a segment can still lie across one cut, i.e. two partials
+    if ((flags & PQ_BALANCED_SLICES) && n_splits < 2) return PQ_ERR_WORKSPACE;
     if (workspace_bytes < pq_decode_attn_workspace_bytes(B, N, n_splits)) return PQ_ERR_WORKSPACE;
-    if (!aligned(q, 2) || !aligned(v, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return PQ_ERR_MISALIGNED;
+    // q rows are read as 16-byte pieces (operands of the residual keys' matrix product)
+    if (!aligned(q, 16) || !aligned(v, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return PQ_ERR_MISALIGNED;
     if (codes && !aligned(codes, 16)) return PQ_ERR_MISALIGNED;
     if (k_resid && !aligned(k_resid, 16)) return PQ_ERR_MISALIGNED;
     return PQ_OK;
@@ -218,6 +223,7 @@ int pq_decode_attn_partials(const void* q,
     a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
     a.min_groups_per_split = min_groups_per_split;
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
+    a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
@@ -500,6 +506,7 @@ int pq_decode_attn_v4(const void* q,
     a.B = B; a.N = N; a.Nk = Nk; a.tbits = tbits; a.dtype = dtype; a.n_splits = n_splits;
     a.min_groups_per_split = min_groups_per_split;
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
+    a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     if (any_groups) {
         a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token

@@ -59,6 +59,7 @@ struct AttnArgs {
     float sm_scale;
     int B, N, Nk, tbits, dtype, n_splits, min_groups_per_split;
     bool packed6 = false;        // code rows are 48 bytes of packed 6-bit codes (tbits == 3 only)
+    bool balanced = false;       // slices cut on the device from the per-sequence counts (PQ_BALANCED_SLICES)
     float* workspace;
     void* out;
 };

@@ -33,6 +33,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--values4", action="store_true")
+    ap.add_argument("--even", action="store_true", help="ragged batches: even slices per sequence instead of balanced slices")
     args = ap.parse_args()
     if not os.path.exists(TIMERS_LIB):
         sys.exit("phase_timing: build the measuring library first: python -m polarquant_amd.build --phase-timers")
@@ -45,13 +46,15 @@ def main():
     sh = w["shape"]
     kw = dict(rbits=sh.rbits, tbits=sh.tbits)
     if w.get("groups_per_seq") is not None:
-        kw.update(n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=int(w["groups_per_seq"].sum()))
+        kw.update(n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=int(w["groups_per_seq"].sum()),
+                  balanced=not args.even)
     if args.values4:
         L = w["n_groups"] * 128
         vq = quantize_values(w["v"][:, :, :L])
         vres = torch.zeros(w["v"].shape[0], w["v"].shape[1], 128, 128, dtype=w["v"].dtype, device=dev)
         vres[:, :, :1] = w["v"][:, :, L:L + 1]
         kw.pop("total_groups", None)
+        kw.pop("balanced", None)
         call = lambda: polar_decode_attention_v4(w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], **kw)
     else:
         call = lambda: polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], **kw)
