@@ -54,9 +54,10 @@ def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.
 def balanced_slots(B: int, Nk: int, group_capacity: int, total_groups: Optional[int], wave_slots: int) -> int:
     """Partial slots per head for PQ_BALANCED_SLICES: enough for the segment length the device will pick
     when the batch holds `total_groups` groups per KV head (None: sequences half full on average)."""
-    units = (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + B
+    # in tiles of 64 tokens: two per group, and on average one per sequence for its residual keys
+    units = 2 * (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + B
     seg = max(1, -(-units * Nk // max(wave_slots, 1)))
-    return max(2, -(-(group_capacity + 1) // seg) + 1)
+    return max(2, -(-(2 * group_capacity + 2) // seg) + 1)
 
 
 def _pick_workspace(workspace: Optional[torch.Tensor], B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:

@@ -351,12 +351,14 @@ __device__ __forceinline__ SeqCounts seq_counts(const AttnParams& p, const V4Arg
     return c;
 }
 
-// One piece of work of a wavefront: quantized groups [g0, g1) of (sequence b, KV head kvh), then,
-// if do_resid, the half-precision residual keys of that sequence; the partial result (m, l, acc) of
-// each of the `rep` query heads goes to partial slot `slot` of its head.
+// One piece of work of a wavefront: the 64-token tiles [t0, t1) of the quantized part of (sequence b,
+// KV head kvh) (tile t = half t & 1 of group t >> 1; a piece may begin or end in the middle of a group,
+// whose table it then builds like any other), then the 64-key tiles [r0, r1) of that sequence's
+// half-precision residual keys; the partial result (m, l, acc) of each of the `rep` query heads goes
+// to partial slot `slot` of its head.
 template <typename T, int TB, int REPP, bool V4, bool PK6>
 __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4, uint32_t lut, uint32_t pbuf, int lane,
-                                           int b, int kvh, const SeqCounts& sc, int g0, int g1, bool do_resid, int slot) {
+                                           int b, int kvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot) {
     // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
     // residual window, row 0 = first residual token; otherwise `v` holds every row.
     const int N = p.N, Nk = p.Nk, rep = p.rep, n_splits = p.n_splits;
@@ -383,8 +385,9 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 
     {
-        // ---------------- quantized groups [g0, g1) ----------------
-        if (g0 < g1) {
+        // ---------------- quantized tiles [t0, t1) ----------------
+        if (t0 < t1) {
+            const int g0 = t0 >> 1, g1 = (t1 + 1) >> 1;
             float qx[REPP], qy[REPP];
 #pragma unroll
             for (int j = 0; j < REPP; j++) {
@@ -401,7 +404,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             // software pipeline: codes of the next tile and metadata of the next group are in flight
             uint4 cnext[kRowLoads];
 #pragma unroll
-            for (int i = 0; i < kRowLoads; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(g0) * (kGroup * kRowB) + 16 * i);
+            for (int i = 0; i < kRowLoads; i++) cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(t0) * (kWave * kRowB) + 16 * i);
             const uint16_t* prs = p.rscale + plane * kPairs + lane;
             const uint16_t* prm = p.rmn + plane * kPairs + lane;
             const uint16_t* pts = p.tscale + plane * kPairs + lane;
@@ -426,7 +429,8 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
                     load_v_tile(vv[buf].r, rv, voff_v, in_range ? tile_tok * (kHeadDim * 2) : 0xFFFF0000u);
                 }
             };
-            load_values(0, static_cast<uint32_t>(2 * g0) * kWave, true);
+            if (t0 & 1) load_values(1, static_cast<uint32_t>(t0) * kWave, true);
+            else load_values(0, static_cast<uint32_t>(t0) * kWave, true);
             PQ_T_DECL;
             for (int grp = g0; grp < g1; grp++) {
                 PQ_T_MARK();
@@ -443,11 +447,12 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
 #pragma unroll
                 for (int half = 0; half < 2; half++) {
                     const int tt = 2 * grp + half;
+                    if (tt < t0 || tt >= t1) continue;            // a piece may begin or end in the middle of a group
                     const uint32_t tok0 = static_cast<uint32_t>(tt) * kWave;
                     // past the last tile of this slice the loads run off the buffer's end and return zeros (the
                     // out-of-range offset leaves room for the 16 KiB of row offsets added to it: no 32-bit wrap)
                     PQ_T_MARK();
-                    load_values(half ^ 1, tok0 + kWave, half == 0 || grp + 1 < g1);
+                    load_values(half ^ 1, tok0 + kWave, tt + 1 < t1);
                     PQ_T_ADD(1);
                     uint32_t cw[16];
                     if constexpr (PK6) {
@@ -466,7 +471,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
                     PQ_T_KEEP(cw[0]);
                     PQ_T_KEEP(cw[15]);
                     PQ_T_ADD(2);
-                    if (half == 0 || grp + 1 < g1) {
+                    if (tt + 1 < t1) {
 #pragma unroll
                         for (int i = 0; i < kRowLoads; i++)
                             cnext[i] = buf_load16(rc, voff_c, static_cast<uint32_t>(tt + 1) * (kWave * kRowB) + 16 * i);
@@ -494,8 +499,8 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             if constexpr (V4) finish_v4<REPP>(st, lane);
         }
     }
-    if (do_resid && nres > 0) {
-        // ---------------- residual keys (model dtype) ----------------
+    if (r0 < r1) {
+        // ---------------- residual keys (model dtype), 64-key tiles [r0, r1) ----------------
         // scores = K . q^T on the matrix cores, as the reference's half-precision matmul (:79): for 16 tokens
         // at a time D[token][head] += K[token][16 dims] * q[head][16 dims], heads padded to the 16 columns.
         // Lane (g,n) supplies, for step (kb, hf), dims 32 kb + 8 g + 4 hf .. +3 of key row n and of query head
@@ -512,8 +517,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
         const __amdgpu_buffer_rsrc_t rk = make_rsrc(p.k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
                                                     static_cast<uint32_t>(nres) * (kHeadDim * 2));
         const uint32_t voff_k = static_cast<uint32_t>(n) * (kHeadDim * 2) + static_cast<uint32_t>(g) * 16;
-        const int n_tiles = (nres + kWave - 1) / kWave;
-        for (int tt = 0; tt < n_tiles; tt++) {
+        for (int tt = r0; tt < r1; tt++) {
             const int tok = tt * kWave + lane;
             const bool valid = tok < nres;
             const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
@@ -644,7 +648,8 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
     const int g1 = (g0 + gps) < sc.nb ? (g0 + gps) : sc.nb;
     // the residual keys go to the block that holds the last quantized group of the sequence
     const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
-    attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, b, kvh, sc, g0, g1, split == last_split, split);
+    attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, b, kvh, sc, 2 * g0, 2 * g1, 0,
+                                     split == last_split ? (sc.nres + kWave - 1) / kWave : 0, split);
 }
 
 __device__ __forceinline__ int wave_sum_i(int v) {
@@ -654,14 +659,14 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 }
 
 // Balanced slices: the work of the whole batch is laid out as one line of units, plane after plane
-// (plane = (sequence, KV head), sequence-major); a sequence's plane holds one unit per quantized
-// group and one more for its residual keys if it has any (a sequence with nothing at all holds one
-// empty unit, so that somebody writes its partials).  The line is cut into segments of `seg` units,
+// (plane = (sequence, KV head), sequence-major); a unit is a tile of 64 tokens: two per quantized
+// group, then one per 64 residual keys (a sequence with nothing at all holds one empty unit, so
+// that somebody writes its partials).  The line is cut into segments of `seg` units,
 // the same for every wavefront; wavefront w works through segment w, which may end one plane and
 // begin the next: every piece of a plane it touches becomes one partial.  The piece of plane P cut
 // by segment w goes to slot w - floor(start of P / seg) of that plane's heads, and the piece that
 // ends P marks the slots behind it empty.
-//   seg = max(min_gps, ceil(line length / wavefronts), ceil((group_capacity + 1) / (n_splits - 1)))
+//   seg = max(2 min_gps, ceil(line length / wavefronts), ceil((2 group_capacity + 2) / (n_splits - 1)))
 // the last term guarantees that no plane is cut into more than n_splits pieces (n_splits >= 2: a plane
 // shorter than a segment can still lie across one cut).  All of this is
 // computed from the per-sequence counts in device memory, by every wavefront alike, so the slices
@@ -680,7 +685,7 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
 
     auto units_of = [&](int bb) {
         const SeqCounts c = seq_counts<V4>(p, v4, bb);
-        const int u = c.nb + (c.nres > 0 ? 1 : 0);
+        const int u = 2 * c.nb + (c.nres + kWave - 1) / kWave;
         return u > 0 ? u : 1;
     };
     // length of the line
@@ -689,8 +694,8 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     const long long per_head = wave_sum_i(mine);          // units of one KV head's planes, all sequences
     const long long total = per_head * Nk;
     long long seg = (total + W - 1) / W;
-    seg = seg < min_gps ? min_gps : seg;
-    const long long cap_units = static_cast<long long>(group_capacity) + 1;
+    seg = seg < 2 * min_gps ? 2 * min_gps : seg;
+    const long long cap_units = 2 * static_cast<long long>(group_capacity) + 2;
     const long long fit = (cap_units + n_splits - 2) / (n_splits - 1);      // n_splits >= 2 (checked on the host)
     seg = seg < fit ? fit : seg;
     const long long start = w * seg;
@@ -755,8 +760,12 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
         // the piece that ends its plane marks the slots behind its own as holding nothing
         if (ub == u && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
         const SeqCounts sc = seq_counts<V4>(p, v4, cb);
-        const int g0 = ua < sc.nb ? ua : sc.nb, g1 = ub < sc.nb ? ub : sc.nb;
-        attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, cb, ckvh, sc, g0, g1, ub > sc.nb, slot);
+        const int qt = 2 * sc.nb;                              // tiles of the quantized part come first
+        const int t0 = ua < qt ? ua : qt, t1 = ub < qt ? ub : qt;
+        const int rt = (sc.nres + kWave - 1) / kWave;
+        int r0 = ua > qt ? ua - qt : 0, r1 = ub > qt ? ub - qt : 0;
+        r1 = r1 < rt ? r1 : rt;                                // (the empty unit of a sequence with nothing)
+        attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, cb, ckvh, sc, t0, t1, r0, r1, slot);
     }
 }
 #pragma clang diagnostic pop
