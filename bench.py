@@ -59,6 +59,8 @@ def bracketed_step_ms(first, second, steps, warmup=4):
     between and after them.  -> (ms per step over the region, mean ms of `first`, mean ms of `second`).
     All three come from the same events, so first + second <= step by construction; the gap between a
     step's end and the next step's start belongs to neither kernel."""
+    from polarquant_amd import workloads as wl
+    wl.ramp_clocks(lambda: (first(), second()))
     for _ in range(warmup):
         first()
         second()
@@ -378,7 +380,7 @@ def main():
     achieved = alg_bytes / (k_ms * 1e-3) / 1e9
     result = {
         "metric": METRIC, "value": round(ms * 1e3, 2), "unit": "us/step", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+        "steps": args.steps, "warmup": args.warmup, "clock_ramp_seconds_before_warmup": wl.RAMP_SECONDS, "ms_per_step": round(ms, 5),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: fused polar decode attention, Llama-3-8B shape (32 q heads / 8 KV heads, "

@@ -356,7 +356,7 @@ __device__ __forceinline__ SeqCounts seq_counts(const AttnParams& p, const V4Arg
 // whose table it then builds like any other), then the 64-key tiles [r0, r1) of that sequence's
 // half-precision residual keys; the partial result (m, l, acc) of each of the `rep` query heads goes
 // to partial slot `slot` of its head.
-template <typename T, int TB, int REPP, bool V4, bool PK6>
+template <typename T, int TB, int REPP, bool V4, bool PK6, bool RESID_FIRST>
 __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4, uint32_t lut, uint32_t pbuf, int lane,
                                            int b, int kvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot) {
     // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
@@ -383,6 +383,70 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
     for (int j = 0; j < REPP; j++) { st.m[j] = -INFINITY; st.l[j] = 0.0f; st.zp[j] = 0.0f; }
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // ---------------- residual keys (model dtype), 64-key tiles [r0, r1) ----------------
+    // RESID_FIRST: runs right after the first loads of the quantized part have been issued, so that its own
+    // loads and arithmetic overlap with their latency instead of standing alone at the end of the piece (the
+    // order of the tiles does not matter to the running softmax).  Measured: configs[1] 221.2 -> 219.2 us
+    // with even slices, where the wavefront that holds the residual keys is the last to finish; with balanced
+    // slices, where it is not, configs[2] 92.7 -> 94.2 us, so those keep the residual keys at the end.
+    auto residual_tiles = [&]() {
+        if (r0 >= r1) return;
+        // scores = K . q^T on the matrix cores, as the reference's half-precision matmul (:79): for 16 tokens
+        // at a time D[token][head] += K[token][16 dims] * q[head][16 dims], heads padded to the 16 columns.
+        // Lane (g,n) supplies, for step (kb, hf), dims 32 kb + 8 g + 4 hf .. +3 of key row n and of query head
+        // n: both operands use the same order of the contraction index, so one 16-byte load per lane feeds two
+        // MFMAs, and the four lanes of a row read 64 contiguous bytes.  All 16 loads of a 64-token tile are
+        // in flight at once.  The D tiles go through LDS (the table region) to the lane == token layout.
+        asm volatile("" ::: "memory");
+        const int g = lane >> 4, n = lane & 15;
+        uint4 qv[4];
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {
+            qv[kb] = (n < rep) ? *reinterpret_cast<const uint4*>(qb + n * kHeadDim + 32 * kb + 8 * g) : make_uint4(0u, 0u, 0u, 0u);
+        }
+        const __amdgpu_buffer_rsrc_t rk = make_rsrc(p.k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
+                                                    static_cast<uint32_t>(nres) * (kHeadDim * 2));
+        const uint32_t voff_k = static_cast<uint32_t>(n) * (kHeadDim * 2) + static_cast<uint32_t>(g) * 16;
+        for (int tt = r0; tt < r1; tt++) {
+            const int tok = tt * kWave + lane;
+            const bool valid = tok < nres;
+            const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
+            uint4 kk[4][4];
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+                for (int kb = 0; kb < 4; kb++)
+                    kk[tb][kb] = buf_load16(rk, voff_k, static_cast<uint32_t>(tt * kWave + 16 * tb) * (kHeadDim * 2) + 64 * kb);
+            uint4 vv[4][4];
+            load_v_tile(vv, rv, voff_v, (V4 ? static_cast<uint32_t>(tt * kWave) : arow) * (kHeadDim * 2));
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++) {
+                floatx4 d = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int kb = 0; kb < 4; kb++) {
+                    d = mfma16<T>(make_uint2(kk[tb][kb].x, kk[tb][kb].y), make_uint2(qv[kb].x, qv[kb].y), d);
+                    d = mfma16<T>(make_uint2(kk[tb][kb].z, kk[tb][kb].w), make_uint2(qv[kb].z, qv[kb].w), d);
+                }
+                // d[i] = score of token 16 tb + 4 g + i for head n
+                if (n < REPP) {
+                    lds_e4* dst = lds_ptr<lds_e4>(lut + (n * kWave + 16 * tb + 4 * g) * 4);
+                    dst->x = d[0]; dst->y = d[1]; dst->z = d[2]; dst->w = d[3];
+                }
+            }
+            asm volatile("" ::: "memory");
+            const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(arow), 0) != 0) : true);
+            float s[REPP];
+#pragma unroll
+            for (int j = 0; j < REPP; j++) {
+                // the reference multiplies q.K^T in the model dtype before promoting (:79)
+                const float sr = lo2f<T>(f2lo<T>(*lds_ptr<lds_f1>(lut + (j * kWave + lane) * 4)));
+                s[j] = keep ? sr * scale_log2 : -INFINITY;
+            }
+            asm volatile("" ::: "memory");
+            softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
+        }
+    };
 
     {
         // ---------------- quantized tiles [t0, t1) ----------------
@@ -431,6 +495,9 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             };
             if (t0 & 1) load_values(1, static_cast<uint32_t>(t0) * kWave, true);
             else load_values(0, static_cast<uint32_t>(t0) * kWave, true);
+            // (with 4-bit values the accumulators are in scaled units until finish_v4: the residual tiles, whose
+            // values are half precision, have to come after it)
+            if constexpr (!V4 && RESID_FIRST) residual_tiles();
             PQ_T_DECL;
             for (int grp = g0; grp < g1; grp++) {
                 PQ_T_MARK();
@@ -497,66 +564,11 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             }
             PQ_T_REPORT(g1 - g0);
             if constexpr (V4) finish_v4<REPP>(st, lane);
+            if constexpr (V4 || !RESID_FIRST) residual_tiles();
+        } else {
+            residual_tiles();
         }
     }
-    if (r0 < r1) {
-        // ---------------- residual keys (model dtype), 64-key tiles [r0, r1) ----------------
-        // scores = K . q^T on the matrix cores, as the reference's half-precision matmul (:79): for 16 tokens
-        // at a time D[token][head] += K[token][16 dims] * q[head][16 dims], heads padded to the 16 columns.
-        // Lane (g,n) supplies, for step (kb, hf), dims 32 kb + 8 g + 4 hf .. +3 of key row n and of query head
-        // n: both operands use the same order of the contraction index, so one 16-byte load per lane feeds two
-        // MFMAs, and the four lanes of a row read 64 contiguous bytes.  All 16 loads of a 64-token tile are
-        // in flight at once.  The D tiles go through LDS (the table region) to the lane == token layout.
-        asm volatile("" ::: "memory");
-        const int g = lane >> 4, n = lane & 15;
-        uint4 qv[4];
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++) {
-            qv[kb] = (n < rep) ? *reinterpret_cast<const uint4*>(qb + n * kHeadDim + 32 * kb + 8 * g) : make_uint4(0u, 0u, 0u, 0u);
-        }
-        const __amdgpu_buffer_rsrc_t rk = make_rsrc(p.k_resid + static_cast<size_t>(bh) * resid_capacity * kHeadDim,
-                                                    static_cast<uint32_t>(nres) * (kHeadDim * 2));
-        const uint32_t voff_k = static_cast<uint32_t>(n) * (kHeadDim * 2) + static_cast<uint32_t>(g) * 16;
-        for (int tt = r0; tt < r1; tt++) {
-            const int tok = tt * kWave + lane;
-            const bool valid = tok < nres;
-            const uint32_t arow = static_cast<uint32_t>(nb) * kGroup + tt * kWave;   // absolute row of lane 0
-            uint4 kk[4][4];
-#pragma unroll
-            for (int tb = 0; tb < 4; tb++)
-#pragma unroll
-                for (int kb = 0; kb < 4; kb++)
-                    kk[tb][kb] = buf_load16(rk, voff_k, static_cast<uint32_t>(tt * kWave + 16 * tb) * (kHeadDim * 2) + 64 * kb);
-            uint4 vv[4][4];
-            load_v_tile(vv, rv, voff_v, (V4 ? static_cast<uint32_t>(tt * kWave) : arow) * (kHeadDim * 2));
-#pragma unroll
-            for (int tb = 0; tb < 4; tb++) {
-                floatx4 d = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int kb = 0; kb < 4; kb++) {
-                    d = mfma16<T>(make_uint2(kk[tb][kb].x, kk[tb][kb].y), make_uint2(qv[kb].x, qv[kb].y), d);
-                    d = mfma16<T>(make_uint2(kk[tb][kb].z, kk[tb][kb].w), make_uint2(qv[kb].z, qv[kb].w), d);
-                }
-                // d[i] = score of token 16 tb + 4 g + i for head n
-                if (n < REPP) {
-                    lds_e4* dst = lds_ptr<lds_e4>(lut + (n * kWave + 16 * tb + 4 * g) * 4);
-                    dst->x = d[0]; dst->y = d[1]; dst->z = d[2]; dst->w = d[3];
-                }
-            }
-            asm volatile("" ::: "memory");
-            const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(arow), 0) != 0) : true);
-            float s[REPP];
-#pragma unroll
-            for (int j = 0; j < REPP; j++) {
-                // the reference multiplies q.K^T in the model dtype before promoting (:79)
-                const float sr = lo2f<T>(f2lo<T>(*lds_ptr<lds_f1>(lut + (j * kWave + lane) * 4)));
-                s[j] = keep ? sr * scale_log2 : -INFINITY;
-            }
-            asm volatile("" ::: "memory");
-            softmax_pv_tile<T, REPP>(st, s, vv, pbuf, lane);
-        }
-    }
-
     // ---------------- write the partial ----------------
     float lsum[REPP];
 #pragma unroll
@@ -648,7 +660,7 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
     const int g1 = (g0 + gps) < sc.nb ? (g0 + gps) : sc.nb;
     // the residual keys go to the block that holds the last quantized group of the sequence
     const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
-    attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, b, kvh, sc, 2 * g0, 2 * g1, 0,
+    attn_piece<T, TB, REPP, V4, PK6, true>(p, v4, lut, pbuf, lane, b, kvh, sc, 2 * g0, 2 * g1, 0,
                                      split == last_split ? (sc.nres + kWave - 1) / kWave : 0, split);
 }
 
@@ -765,7 +777,7 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
         const int rt = (sc.nres + kWave - 1) / kWave;
         int r0 = ua > qt ? ua - qt : 0, r1 = ub > qt ? ub - qt : 0;
         r1 = r1 < rt ? r1 : rt;                                // (the empty unit of a sequence with nothing)
-        attn_piece<T, TB, REPP, V4, PK6>(p, v4, lut, pbuf, lane, cb, ckvh, sc, t0, t1, r0, r1, slot);
+        attn_piece<T, TB, REPP, V4, PK6, false>(p, v4, lut, pbuf, lane, cb, ckvh, sc, t0, t1, r0, r1, slot);
     }
 }
 #pragma clang diagnostic pop
