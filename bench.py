@@ -272,6 +272,32 @@ def other_configs(dev, steps):
                               parity=dict(fl, sample="KV head 0, all 131072 keys, vs the CPU oracle's quantizer"))
     del w, quant, ref, got
     torch.cuda.empty_cache()
+
+    # configs[4] at reduced depth: the end-to-end greedy decode loop (random-init Llama-3-8B architecture, bf16,
+    # batch 8, prompt 16384) with 4 of its 32 decoder layers and 66 new tokens, the step replayed from a HIP graph;
+    # the full-depth run is `python -m polarquant_amd.e2e_bench --graph`.  Its parity is the test suite's
+    # (every step of toy models replayed through the oracle); nothing is checked here.
+    try:
+        from polarquant_amd import e2e_bench
+        r4 = e2e_bench.run(batch=8, prompt=16384, new=66, layers=4, graph=True)
+        r2 = e2e_bench.run(batch=8, prompt=16384, new=66, layers=2, graph=True)
+        per_layer = (r4["decode_ms_per_step"] - r2["decode_ms_per_step"]) / 2
+        head = r4["decode_ms_per_step"] - 4 * per_layer
+        full = 32 * per_layer + head
+        out["cfg4_e2e_reduced_depth"] = {
+            "workload": r4["workload"] + ", 4 and 2 of the 32 layers",
+            "decode_ms_per_step_4_layers": r4["decode_ms_per_step"], "decode_ms_per_step_2_layers": r2["decode_ms_per_step"],
+            "decode_ms_per_layer": round(per_layer, 4), "decode_ms_embedding_and_lm_head": round(head, 4),
+            "decode_ms_per_step_32_layers_extrapolated": round(full, 3),
+            "decode_tokens_per_s_32_layers_extrapolated": round(8 * 1e3 / full, 1),
+            "prefill_s_4_layers": r4["prefill_s"],
+            "kv_cache_bytes_per_token_32_layers": r4["kv_cache_bytes_per_token"] * 8,
+            "fp16_kv_cache_bytes_per_token_32_layers": r4["fp16_kv_cache_bytes_per_token"] * 8,
+            "note": "measured at reduced depth; the 32-layer figures are a linear extrapolation, not a measurement",
+        }
+    except Exception as e:                      # noqa: BLE001 - report, do not fail the bench
+        out["cfg4_e2e_reduced_depth"] = {"error": str(e)[:300]}
+    torch.cuda.empty_cache()
     return out
 
 
