@@ -28,8 +28,9 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # HBM bytes per launch of the dominant kernel at this workload, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
 # read for a copy kernel of known size; see profiles/attn_kernel_cfg1_pmc.md.
-MEASURED_TRAFFIC_BYTES = int(669602 * 2.0 * 1024 + 2176 * 1.0 * 1024)
-TRAFFIC_SOURCE = "constant, not read in this run: rocprofv3 --pmc runs of 2026-11-25 at commit 0b769ba (profiles/attn_kernel_cfg1_pmc.md)"
+MEASURED_TRAFFIC_BYTES = int(669351 * 2.0 * 1024 + 2112.16 * 1024)
+TRAFFIC_SOURCE = ("constant, not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of 2026-11-25 with the attention "
+                  "kernel as of the commit 'Residual keys right after the first loads of a piece' (profiles/attn_kernel_cfg1_pmc.md)")
 
 
 def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):
@@ -310,6 +311,7 @@ def main():
     ap.add_argument("--splits", type=int, default=0, help="override the context split count")
     ap.add_argument("--no-values4", action="store_true", help="skip the 4-bit-value (Mixed variant) measurement")
     ap.add_argument("--no-configs", action="store_true", help="skip configs[0], [2] and [3]")
+    ap.add_argument("--no-ramp", action="store_true", help="no clock ramp before the timed regions (counter-collection runs under the profiler)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run 3 plain 1 GiB device copies (torch clone): under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` "
                          "their counter values give the scale factor for the attention kernel's")
@@ -323,6 +325,8 @@ def main():
         sys.exit(1)
 
     from polarquant_amd import _ffi, workloads as wl
+    if args.no_ramp:
+        wl.RAMP_SECONDS = 0.0
     from polarquant_amd.attention import plan_splits, polar_decode_attention, workspace_for
     from polarquant_amd.kernel4group import _stream_ptr
 

@@ -115,7 +115,10 @@ def main():
     ap.add_argument("--values4", action="store_true")
     ap.add_argument("--packed", action="store_true", help="also run the 3/3-bit configuration with packed 6-bit code rows")
     ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--no-ramp", action="store_true", help="no clock ramp before the timed regions (counter-collection runs under the profiler)")
     args = ap.parse_args()
+    if args.no_ramp:
+        wl.RAMP_SECONDS = 0.0
     dev = torch.device("cuda:0")
     for idx in args.configs:
         run(idx, dev, args.values4, args.steps)

@@ -175,13 +175,14 @@ def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False,
 RAMP_SECONDS = 0.25
 
 
-def ramp_clocks(fn, seconds: float = RAMP_SECONDS) -> int:
+def ramp_clocks(fn, seconds: Optional[float] = None) -> int:
     """Run `fn` untimed for `seconds` of wall time.  After an idle stretch (input generation on the host, a CPU
     checker) the GPU sits in a low power state and takes some 30-50 ms of continuous work to reach its
     sustained clocks: a configs[1] step measures 280 -> 240 -> 226 us over its first 150 launches.  Timed
     regions are meant to show the sustained rate of a decode loop, so each one is preceded by this.
     -> number of calls made."""
     import time
+    seconds = RAMP_SECONDS if seconds is None else seconds
     n, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < seconds:
         for _ in range(10):
@@ -191,9 +192,10 @@ def ramp_clocks(fn, seconds: float = RAMP_SECONDS) -> int:
     return n
 
 
-def time_events(fn, steps, warmup, ramp_seconds: float = RAMP_SECONDS):
+def time_events(fn, steps, warmup, ramp_seconds: Optional[float] = None):
     """ms per call: clock ramp (untimed), `warmup` untimed calls, then exactly `steps` calls between one pair of
     events on the current stream, with a device synchronisation on both sides."""
+    ramp_seconds = RAMP_SECONDS if ramp_seconds is None else ramp_seconds
     if ramp_seconds > 0:
         ramp_clocks(fn, ramp_seconds)
     for _ in range(warmup):
