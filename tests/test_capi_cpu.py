@@ -135,6 +135,15 @@ def test_validate_decode_attn_and_plan(lib):
     assert max_rows * 256 == 0xFFFF0000
     assert bad(14, max_rows) == 0 and bad(14, max_rows + 1) == -2 and bad(14, 1 << 24) == -2
     assert bad(10, max_rows) == 0 and bad(10, max_rows + 1) == -2 and bad(10, 1 << 24) == -2
+    # slices cut on the device: a flag of the attention entry points only, and at least two partial slots per head
+    a = list(ok); a[29] = 16
+    assert lib.pq_validate_decode_attn(*a) == 0
+    a[24], a[27] = 1, lib.pq_decode_attn_workspace_bytes(B, N, 1)
+    assert lib.pq_validate_decode_attn(*a) == -7
+    a = list(ok); a[29] = 64
+    assert lib.pq_validate_decode_attn(*a) == -2                     # unknown flag bit
+    assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 16) == -2
+    assert bad(0, P + 8) == -5                                       # q rows are read as 16-byte pieces
     a = list(ok); a[15] = P; a[16] = 100          # mask row shorter than the context
     assert lib.pq_validate_decode_attn(*a) == -6
     # no quantized groups yet: codes may be NULL
