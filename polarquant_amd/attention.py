@@ -51,13 +51,15 @@ def workspace_for(B: int, N: int, n_splits: int, device: torch.device) -> torch.
     return ws
 
 
-def balanced_slots(B: int, Nk: int, group_capacity: int, total_groups: Optional[int], wave_slots: int) -> int:
+def balanced_slots(B: int, Nk: int, group_capacity: int, total_groups: Optional[int], wave_slots: int,
+                   resid_capacity: int = GROUP) -> int:
     """Partial slots per head for PQ_BALANCED_SLICES: enough for the segment length the device will pick
     when the batch holds `total_groups` groups per KV head (None: sequences half full on average)."""
-    # in tiles of 64 tokens: two per group, and on average one per sequence for its residual keys
-    units = 2 * (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + B
+    # in tiles of 64 tokens: two per group, and per sequence one for its residual keys (on average) and two that
+    # stand for a plane's start-up
+    units = 2 * (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + 3 * B
     seg = max(1, -(-units * Nk // max(wave_slots, 1)))
-    return max(2, -(-(2 * group_capacity + 2) // seg) + 1)
+    return max(2, -(-(2 * group_capacity + -(-resid_capacity // 64) + 2) // seg) + 1)
 
 
 def _pick_workspace(workspace: Optional[torch.Tensor], B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
@@ -135,7 +137,7 @@ def polar_decode_attention(
     if balanced:
         flags |= _ffi.PQ_BALANCED_SLICES
         if n_splits is None:
-            n_splits = balanced_slots(B, Nk, max_groups, total_groups, 4 * _num_cus(dev))
+            n_splits = balanced_slots(B, Nk, max_groups, total_groups, 4 * _num_cus(dev), r_cap)
     elif n_groups_per_seq is not None and n_splits is None and max_groups > 0:
         tot = total_groups if total_groups is not None else (B * max_groups + 1) // 2
         # one wavefront per SIMD; every (sequence, KV head) rounds its slice count up, so leave one
@@ -213,7 +215,7 @@ def polar_decode_attention_v4(
     if balanced:
         flags |= _ffi.PQ_BALANCED_SLICES
         if n_splits is None:
-            n_splits = balanced_slots(B, Nk, max_groups, total_groups, (8 if N // Nk <= 4 else 4) * _num_cus(dev))
+            n_splits = balanced_slots(B, Nk, max_groups, total_groups, (8 if N // Nk <= 4 else 4) * _num_cus(dev), r_cap)
     if n_splits is None:
         n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, N, Nk, max(max_groups, 1), _num_cus(dev))
     ws = _pick_workspace(workspace, B, N, n_splits, dev)

@@ -664,6 +664,9 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
                                      split == last_split ? (sc.nres + kWave - 1) / kWave : 0, split);
 }
 
+// Units a plane's start-up counts for when the balanced kernel cuts the line (query, first table, first loads, the
+// partial's write: measured at configs[2], 0 / 1 / 2 / 3 units: 92.8 / 89.6 / 87.9 / 88.6 us).
+constexpr int kStartUnits = 2;
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -672,13 +675,12 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 
 // Balanced slices: the work of the whole batch is laid out as one line of units, plane after plane
 // (plane = (sequence, KV head), sequence-major); a unit is a tile of 64 tokens: two per quantized
-// group, then one per 64 residual keys (a sequence with nothing at all holds one empty unit, so
-// that somebody writes its partials).  The line is cut into segments of `seg` units,
+// group, then one per 64 residual keys, behind kStartUnits units that stand for the plane's start-up.  The line is cut into segments of `seg` units,
 // the same for every wavefront; wavefront w works through segment w, which may end one plane and
 // begin the next: every piece of a plane it touches becomes one partial.  The piece of plane P cut
 // by segment w goes to slot w - floor(start of P / seg) of that plane's heads, and the piece that
 // ends P marks the slots behind it empty.
-//   seg = max(2 min_gps, ceil(line length / wavefronts), ceil((2 group_capacity + 2) / (n_splits - 1)))
+//   seg = max(2 min_gps, ceil(line length / wavefronts), ceil((2 group_capacity + ceil(resid_capacity / 64) + kStartUnits) / (n_splits - 1)))
 // the last term guarantees that no plane is cut into more than n_splits pieces (n_splits >= 2: a plane
 // shorter than a segment can still lie across one cut).  All of this is
 // computed from the per-sequence counts in device memory, by every wavefront alike, so the slices
@@ -695,10 +697,11 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     const int lane = threadIdx.x;
     const long long W = gridDim.x, w = blockIdx.x;
 
+    // units of one plane of sequence bb: kStartUnits for the plane's start-up (they also make a sequence with
+    // nothing at all a plane of its own, so that somebody writes its partials), then its tiles
     auto units_of = [&](int bb) {
         const SeqCounts c = seq_counts<V4>(p, v4, bb);
-        const int u = 2 * c.nb + (c.nres + kWave - 1) / kWave;
-        return u > 0 ? u : 1;
+        return kStartUnits + 2 * c.nb + (c.nres + kWave - 1) / kWave;
     };
     // length of the line
     int mine = 0;
@@ -707,7 +710,9 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     const long long total = per_head * Nk;
     long long seg = (total + W - 1) / W;
     seg = seg < 2 * min_gps ? 2 * min_gps : seg;
-    const long long cap_units = 2 * static_cast<long long>(group_capacity) + 2;
+    // the most units a plane can have (the residual window is 128 keys in the reference, but the interface takes
+    // any resid_capacity)
+    const long long cap_units = 2 * static_cast<long long>(group_capacity) + (resid_capacity + kWave - 1) / kWave + kStartUnits;
     const long long fit = (cap_units + n_splits - 2) / (n_splits - 1);      // n_splits >= 2 (checked on the host)
     seg = seg < fit ? fit : seg;
     const long long start = w * seg;
@@ -772,11 +777,11 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
         // the piece that ends its plane marks the slots behind its own as holding nothing
         if (ub == u && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
         const SeqCounts sc = seq_counts<V4>(p, v4, cb);
-        const int qt = 2 * sc.nb;                              // tiles of the quantized part come first
-        const int t0 = ua < qt ? ua : qt, t1 = ub < qt ? ub : qt;
-        const int rt = (sc.nres + kWave - 1) / kWave;
-        int r0 = ua > qt ? ua - qt : 0, r1 = ub > qt ? ub - qt : 0;
-        r1 = r1 < rt ? r1 : rt;                                // (the empty unit of a sequence with nothing)
+        // the first kStartUnits units of a plane stand for its start-up; then the tiles of the quantized part, then the residual keys'
+        const int ta = ua > kStartUnits ? ua - kStartUnits : 0, tb = ub > kStartUnits ? ub - kStartUnits : 0;
+        const int qt = 2 * sc.nb;
+        const int t0 = ta < qt ? ta : qt, t1 = tb < qt ? tb : qt;
+        const int r0 = ta > qt ? ta - qt : 0, r1 = tb > qt ? tb - qt : 0;
         attn_piece<T, TB, REPP, V4, PK6, false>(p, v4, lut, pbuf, lane, cb, ckvh, sc, t0, t1, r0, r1, slot);
     }
 }

@@ -151,3 +151,28 @@ def test_balanced_slices_random_batches(gpu, seed):
     assert torch.isfinite(got.float()).all()
     ok, err = _within(got, ref, literal=d["literal"])
     assert ok, err
+
+
+def test_balanced_slices_with_a_long_residual_window(gpu):
+    """The interface takes any residual capacity, not only the reference's 128: a window of 300 keys is five tiles of
+    a plane's line, and the slot bound has to count them (2 slots: every plane is cut at most once)."""
+    g = torch.Generator().manual_seed(35)
+    B, N, Nk, ng = 3, 8, 2, 2
+    lens_res = [300, 17, 129]
+    k = wl.make_keys(B, Nk, ng * 128 + 300, 5e5, g)
+    q = wl.make_half((B, N, 1, 128), g)
+    v = wl.make_half((B, Nk, ng * 128 + 300, 128), g)
+    quant = po.quantize_and_pack_nbit(k[:, :, :ng * 128].contiguous())
+    kres = torch.zeros(B, Nk, 300, 128, dtype=torch.float16)
+    refs = []
+    for b, nr in enumerate(lens_res):
+        kres[b, :, :nr] = k[b, :, ng * 128:ng * 128 + nr]
+        refs.append(po.decode_attention(q[b:b + 1], k[b:b + 1, :, ng * 128:ng * 128 + nr].contiguous(), *[t[b:b + 1] for t in quant],
+                                        v[b:b + 1, :, :ng * 128 + nr]).double())
+    ref = torch.cat(refs, 0)
+    for ns in (2, 3, 7):
+        got = polar_decode_attention(q.to(gpu), *[t.to(gpu) for t in quant], kres.to(gpu), v.to(gpu), 0, 0, balanced=True, n_splits=ns,
+                                     n_groups_per_seq=torch.full((B,), ng, dtype=torch.int32, device=gpu),
+                                     n_resid_per_seq=torch.tensor(lens_res, dtype=torch.int32, device=gpu)).cpu()
+        ok, err = _within(got, ref)
+        assert ok, (ns, err)
