@@ -33,22 +33,43 @@
 // Measuring build only (-DPQ_ATTN_PHASE_TIMERS, `python -m polarquant_amd.build --phase-timers`): wall-clock
 // (100 MHz) time of each phase of the group loop, summed per wavefront and printed by a few of them.
 #ifdef PQ_ATTN_PHASE_TIMERS
-#define PQ_T_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}, pt_mark_ = 0; const long long pt_begin_ = wall_clock64()
+#define PQ_T_ENTRY const long long pt_entry_ = wall_clock64(); long long pt_loop0_ = pt_entry_, pt_first_ = 0, pt_loop1_ = pt_entry_, pt_sum_[6] = {0, 0, 0, 0, 0, 0}; int pt_groups_ = 0
+#define PQ_T_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}, pt_mark_ = 0; pt_loop0_ = wall_clock64()
 #define PQ_T_MARK() pt_mark_ = wall_clock64()
 #define PQ_T_ADD(i) do { const long long pt_now_ = wall_clock64(); pt_[i] += pt_now_ - pt_mark_; pt_mark_ = pt_now_; } while (0)
 #define PQ_T_KEEP(x) asm volatile("" ::"v"(x))
+#define PQ_T_FIRST_GROUP_DONE() do { if (pt_first_ == 0) pt_first_ = wall_clock64() - pt_loop0_; } while (0)
 #define PQ_T_REPORT(n_groups)                                                                                        \
     do {                                                                                                             \
-        if (threadIdx.x == 0 && blockIdx.x % 97 == 0)                                                                \
+        pt_loop1_ = wall_clock64();                                                                                  \
+        pt_groups_ = n_groups;                                                                                       \
+        for (int i_ = 0; i_ < 6; i_++) pt_sum_[i_] = pt_[i_];                                                        \
+    } while (0)
+// Printed once per piece, after its partial has been handed to the memory system (a device printf takes
+// milliseconds, so none may sit inside what is timed): the phase sums of the group loop, then the absolute entry
+// and exit clocks (the 100 MHz counter is common to the chip, so the spread of entries and exits over the
+// wavefronts can be read off), entry -> loop, the first group, the loop, loop -> exit.
+#define PQ_T_EXIT()                                                                                                  \
+    do {                                                                                                             \
+        const long long pt_exit_ = wall_clock64();                                                                   \
+        if (threadIdx.x == 0 && blockIdx.x % 97 == 0) {                                                              \
             printf("pq_phase block %d groups %d total %lld table %lld value_issue %lld code_wait %lld code_issue %lld score %lld softmax_pv %lld\n", \
-                   static_cast<int>(blockIdx.x), n_groups, wall_clock64() - pt_begin_, pt_[0], pt_[1], pt_[2], pt_[3], pt_[4], pt_[5]); \
+                   static_cast<int>(blockIdx.x), pt_groups_, pt_loop1_ - pt_loop0_, pt_sum_[0], pt_sum_[1], pt_sum_[2], \
+                   pt_sum_[3], pt_sum_[4], pt_sum_[5]);                                                              \
+            printf("pq_piece block %d groups %d entry %lld exit %lld before_loop %lld first_group %lld loop %lld after_loop %lld\n", \
+                   static_cast<int>(blockIdx.x), pt_groups_, pt_entry_, pt_exit_, pt_loop0_ - pt_entry_, pt_first_,   \
+                   pt_loop1_ - pt_loop0_, pt_exit_ - pt_loop1_);                                                     \
+        }                                                                                                            \
     } while (0)
 #else
+#define PQ_T_ENTRY
 #define PQ_T_DECL
 #define PQ_T_MARK()
 #define PQ_T_ADD(i)
 #define PQ_T_KEEP(x)
+#define PQ_T_FIRST_GROUP_DONE()
 #define PQ_T_REPORT(n_groups)
+#define PQ_T_EXIT()
 #endif
 
 namespace pq {
@@ -361,6 +382,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
                                            int b, int kvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot) {
     // V4: the values of the quantized groups are 4-bit (v4), and `v` holds only the rows of the
     // residual window, row 0 = first residual token; otherwise `v` holds every row.
+    PQ_T_ENTRY;
     const int N = p.N, Nk = p.Nk, rep = p.rep, n_splits = p.n_splits;
     const int bh = b * Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
@@ -452,12 +474,15 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
         // ---------------- quantized tiles [t0, t1) ----------------
         if (t0 < t1) {
             const int g0 = t0 >> 1, g1 = (t1 + 1) >> 1;
-            float qx[REPP], qy[REPP];
+            // the query rows of all heads are requested at once, and nothing waits for them before the table is
+            // built: a load under `j < rep` would be a branch with its own wait, one memory round trip per head
+            // before the first codes are even requested (a padded head re-reads row 0 and is zeroed afterwards)
+            uint16_t qraw[REPP][2];
 #pragma unroll
             for (int j = 0; j < REPP; j++) {
-                const bool ok = j < rep;
-                qx[j] = ok ? lo2f<T>(qb[j * kHeadDim + lane]) : 0.0f;
-                qy[j] = ok ? lo2f<T>(qb[j * kHeadDim + kPairs + lane]) : 0.0f;
+                const uint16_t* qrow = qb + (j < rep ? j : 0) * kHeadDim + lane;
+                qraw[j][0] = qrow[0];
+                qraw[j][1] = qrow[kPairs];
             }
             const size_t plane = static_cast<size_t>(bh) * group_capacity;
             // a token's code row: 64 bytes, or 48 when the 6-bit codes are stored packed
@@ -498,6 +523,12 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             // (with 4-bit values the accumulators are in scaled units until finish_v4: the residual tiles, whose
             // values are half precision, have to come after it)
             if constexpr (!V4 && RESID_FIRST) residual_tiles();
+            float qx[REPP], qy[REPP];
+#pragma unroll
+            for (int j = 0; j < REPP; j++) {
+                qx[j] = j < rep ? lo2f<T>(qraw[j][0]) : 0.0f;
+                qy[j] = j < rep ? lo2f<T>(qraw[j][1]) : 0.0f;
+            }
             PQ_T_DECL;
             for (int grp = g0; grp < g1; grp++) {
                 PQ_T_MARK();
@@ -561,6 +592,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
                     PQ_T_KEEP(st.acc[0][0]);
                     PQ_T_ADD(5);
                 }
+                PQ_T_FIRST_GROUP_DONE();
             }
             PQ_T_REPORT(g1 - g0);
             if constexpr (V4) finish_v4<REPP>(st, lane);
@@ -587,6 +619,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             *reinterpret_cast<float4*>(pa + 8 * i + 4) = make_float4(st.acc[4][i], st.acc[5][i], st.acc[6][i], st.acc[7][i]);
         }
     }
+    PQ_T_EXIT();
 }
 
 // Mark the partial slots [first, n_splits) of the `rep` query heads of (b, kvh) as holding nothing.

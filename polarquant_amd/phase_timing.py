@@ -34,6 +34,7 @@ def main():
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--values4", action="store_true")
     ap.add_argument("--even", action="store_true", help="ragged batches: even slices per sequence instead of balanced slices")
+    ap.add_argument("--pieces", action="store_true", help="also list every reporting piece: block, groups, us from the first entry to its entry and exit")
     args = ap.parse_args()
     if not os.path.exists(TIMERS_LIB):
         sys.exit("phase_timing: build the measuring library first: python -m polarquant_amd.build --phase-timers")
@@ -77,6 +78,11 @@ def main():
         m = re.match(r"pq_phase block (\d+) groups (\d+) total (\d+) " + " ".join(p + r" (\d+)" for p in PHASES), line)
         if m:
             rows.append([int(v) for v in m.groups()])
+    pieces = []
+    for line in text.splitlines():
+        m = re.match(r"pq_piece block (\d+) groups (\d+) entry (\d+) exit (\d+) before_loop (\d+) first_group (\d+) loop (\d+) after_loop (\d+)", line)
+        if m:
+            pieces.append([int(v) for v in m.groups()])
     rows = [r for r in rows if r[1] > 0]
     if not rows:
         sys.exit("phase_timing: no wavefront reported (is this the measuring build?)")
@@ -85,9 +91,36 @@ def main():
     for i, p in enumerate(PHASES):
         per_group[p] = sum(r[3 + i] for r in rows) / groups * 0.01
     per_group["other"] = per_group["total"] - sum(per_group[p] for p in PHASES)
-    print(json.dumps({"config": args.config, "values4": bool(args.values4), "wavefronts_reporting": len(rows),
-                      "groups_per_wavefront": round(groups / len(rows), 2),
-                      "us_per_group": {k: round(v, 3) for k, v in per_group.items()}}))
+    out = {"config": args.config, "values4": bool(args.values4), "wavefronts_reporting": len(rows),
+           "groups_per_wavefront": round(groups / len(rows), 2),
+           "us_per_group": {k: round(v, 3) for k, v in per_group.items()}}
+    with_loop = [r for r in pieces if r[1] > 0]
+    if with_loop:
+        # the life of a piece outside its steady state (clock ticks of 10 ns -> us)
+        n = len(with_loop)
+        mean = lambda i: sum(r[i] for r in with_loop) / n * 0.01
+        # absolute clocks: only a block's first piece (a later piece of the same wavefront starts after the print)
+        seen, firsts = set(), []
+        for r in pieces:
+            if r[0] not in seen:
+                seen.add(r[0])
+                firsts.append(r)
+        first = min(r[2] for r in firsts)
+        out["piece_us"] = {
+            "pieces_reporting": n,
+            "entry_to_loop (addresses, first loads issued, residual keys if they come first)": round(mean(4), 2),
+            "first_group (waits for the query, the first metadata and codes)": round(mean(5), 2),
+            "loop": round(mean(6), 2),
+            "loop_to_exit (4-bit values' rescale, residual keys if they come last, partial written)": round(mean(7), 2),
+            "entry_spread_over_wavefronts": round((max(r[2] for r in firsts) - first) * 0.01, 2),
+            "first_entry_to_exit_of_first_pieces_min_mean_max": [round((min(r[3] for r in firsts) - first) * 0.01, 2),
+                                                                 round((sum(r[3] for r in firsts) / len(firsts) - first) * 0.01, 2),
+                                                                 round((max(r[3] for r in firsts) - first) * 0.01, 2)],
+        }
+        if args.pieces:
+            out["pieces (block, groups, entry us, exit us)"] = [[r[0], r[1], round((r[2] - first) * 0.01, 2), round((r[3] - first) * 0.01, 2)]
+                                                                for r in pieces]
+    print(json.dumps(out))
 
 
 if __name__ == "__main__":
