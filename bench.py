@@ -274,30 +274,28 @@ def other_configs(dev, steps):
     del w, quant, ref, got
     torch.cuda.empty_cache()
 
-    # configs[4] at reduced depth: the end-to-end greedy decode loop (random-init Llama-3-8B architecture, bf16,
-    # batch 8, prompt 16384) with 4 of its 32 decoder layers and 66 new tokens, the step replayed from a HIP graph;
-    # the full-depth run is `python -m polarquant_amd.e2e_bench --graph`.  Its parity is the test suite's
-    # (every step of toy models replayed through the oracle); nothing is checked here.
+    # configs[4]: the end-to-end greedy decode loop (random-init Llama-3-8B architecture, bf16, all 32 layers, batch 8,
+    # prompt 16384, 256 new tokens), the step replayed from a HIP graph; a 2-layer run of the same loop splits the step
+    # into its per-layer part and the embedding / lm_head part.  Its parity is the test suite's (every step of toy
+    # models replayed through the oracle); nothing is checked here.
     try:
         from polarquant_amd import e2e_bench
-        r4 = e2e_bench.run(batch=8, prompt=16384, new=66, layers=4, graph=True)
+        r32 = e2e_bench.run(batch=8, prompt=16384, new=256, layers=32, graph=True)
+        torch.cuda.empty_cache()
         r2 = e2e_bench.run(batch=8, prompt=16384, new=66, layers=2, graph=True)
-        per_layer = (r4["decode_ms_per_step"] - r2["decode_ms_per_step"]) / 2
-        head = r4["decode_ms_per_step"] - 4 * per_layer
-        full = 32 * per_layer + head
-        out["cfg4_e2e_reduced_depth"] = {
-            "workload": r4["workload"] + ", 4 and 2 of the 32 layers",
-            "decode_ms_per_step_4_layers": r4["decode_ms_per_step"], "decode_ms_per_step_2_layers": r2["decode_ms_per_step"],
-            "decode_ms_per_layer": round(per_layer, 4), "decode_ms_embedding_and_lm_head": round(head, 4),
-            "decode_ms_per_step_32_layers_extrapolated": round(full, 3),
-            "decode_tokens_per_s_32_layers_extrapolated": round(8 * 1e3 / full, 1),
-            "prefill_s_4_layers": r4["prefill_s"],
-            "kv_cache_bytes_per_token_32_layers": r4["kv_cache_bytes_per_token"] * 8,
-            "fp16_kv_cache_bytes_per_token_32_layers": r4["fp16_kv_cache_bytes_per_token"] * 8,
-            "note": "measured at reduced depth; the 32-layer figures are a linear extrapolation, not a measurement",
+        per_layer = (r32["decode_ms_per_step"] - r2["decode_ms_per_step"]) / 30
+        out["cfg4_e2e"] = {
+            "workload": r32["workload"], "layers": 32,
+            "prefill_s": r32["prefill_s"], "decode_ms_per_step": r32["decode_ms_per_step"],
+            "decode_tokens_per_s": r32["decode_tokens_per_s"],
+            "decode_ms_per_layer": round(per_layer, 4),
+            "decode_ms_embedding_and_lm_head": round(r32["decode_ms_per_step"] - 32 * per_layer, 4),
+            "kv_cache_bytes_per_token": r32["kv_cache_bytes_per_token"],
+            "fp16_kv_cache_bytes_per_token": r32["fp16_kv_cache_bytes_per_token"],
+            "peak_memory_GiB": r32["peak_memory_GiB"],
         }
     except Exception as e:                      # noqa: BLE001 - report, do not fail the bench
-        out["cfg4_e2e_reduced_depth"] = {"error": str(e)[:300]}
+        out["cfg4_e2e"] = {"error": str(e)[:300]}
     torch.cuda.empty_cache()
     return out
 
@@ -310,7 +308,7 @@ def main():
     ap.add_argument("--no-baselines", action="store_true", help="skip the CPU and fp16 baselines")
     ap.add_argument("--splits", type=int, default=0, help="override the context split count")
     ap.add_argument("--no-values4", action="store_true", help="skip the 4-bit-value (Mixed variant) measurement")
-    ap.add_argument("--no-configs", action="store_true", help="skip configs[0], [2] and [3]")
+    ap.add_argument("--no-configs", action="store_true", help="skip configs[0], [2], [3] and [4]")
     ap.add_argument("--no-ramp", action="store_true", help="no clock ramp before the timed regions (counter-collection runs under the profiler)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run 3 plain 1 GiB device copies (torch clone): under `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` "
