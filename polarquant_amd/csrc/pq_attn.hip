@@ -700,6 +700,7 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
 // Units a plane's start-up counts for when the balanced kernel cuts the line (query, first table, first loads, the
 // partial's write: measured at configs[2], 0 / 1 / 2 / 3 units: 92.8 / 89.6 / 87.9 / 88.6 us).
 constexpr int kStartUnits = 2;
+
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -707,17 +708,19 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 }
 
 // Balanced slices: the work of the whole batch is laid out as one line of units, plane after plane
-// (plane = (sequence, KV head), sequence-major); a unit is a tile of 64 tokens: two per quantized
-// group, then one per 64 residual keys, behind kStartUnits units that stand for the plane's start-up.  The line is cut into segments of `seg` units,
-// the same for every wavefront; wavefront w works through segment w, which may end one plane and
-// begin the next: every piece of a plane it touches becomes one partial.  The piece of plane P cut
-// by segment w goes to slot w - floor(start of P / seg) of that plane's heads, and the piece that
-// ends P marks the slots behind it empty.
-//   seg = max(2 min_gps, ceil(line length / wavefronts), ceil((2 group_capacity + ceil(resid_capacity / 64) + kStartUnits) / (n_splits - 1)))
-// the last term guarantees that no plane is cut into more than n_splits pieces (n_splits >= 2: a plane
-// shorter than a segment can still lie across one cut).  All of this is
-// computed from the per-sequence counts in device memory, by every wavefront alike, so the slices
-// follow the real lengths of a ragged or growing batch without the host knowing them.
+// (plane = (sequence, KV head), sequence-major).  A plane is kStartUnits units that stand for its
+// start-up, then one unit per tile of 64 tokens: two per quantized group, then one per 64 residual
+// keys.  The line is cut into segments of `seg` units, the same for every wavefront; wavefront w
+// works through segment w, which may end one plane and begin the next: every piece of a plane it
+// touches becomes one partial.  The piece of plane P cut by segment w goes to slot
+// w - floor(start of P / seg) of that plane's heads, and the piece that ends P marks the slots
+// behind it empty.
+//   seg = max(2 min_gps, ceil(line length / wavefronts),
+//             ceil((2 group_capacity + ceil(resid_capacity / 64) + kStartUnits) / (n_splits - 1)))
+// The last term guarantees that no plane is cut into more than n_splits pieces (n_splits >= 2: a
+// plane shorter than a segment can still lie across one cut).  All of this is computed from the
+// per-sequence counts in device memory, by every wavefront alike, so the slices follow the real
+// lengths of a ragged or growing batch without the host knowing them.
 template <typename T, int TB, int REPP, bool V4, bool PK6>
 __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
 void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
@@ -810,7 +813,8 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
         // the piece that ends its plane marks the slots behind its own as holding nothing
         if (ub == u && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
         const SeqCounts sc = seq_counts<V4>(p, v4, cb);
-        // the first kStartUnits units of a plane stand for its start-up; then the tiles of the quantized part, then the residual keys'
+        // the first kStartUnits units of a plane stand for its start-up; then the tiles of the quantized part,
+        // then the residual keys'
         const int ta = ua > kStartUnits ? ua - kStartUnits : 0, tb = ub > kStartUnits ? ub - kStartUnits : 0;
         const int qt = 2 * sc.nb;
         const int t0 = ta < qt ? ta : qt, t1 = tb < qt ? tb : qt;
