@@ -48,6 +48,7 @@ class PolarConfig:
     vocab_size: int = 128256
     rms_norm_eps: float = 1e-5
     rope_theta: float = 500000.0
+    rope_scaling: Optional[dict] = None  # HF's dict ("rope_type": "linear" | "llama3", ...), None: plain RoPE
     head_dim: int = 128
     attention_bias: bool = False        # q/k/v bias (Qwen2: True)
     mlp_bias: bool = False
@@ -679,6 +680,13 @@ class PolarForCausalLM(nn.Module):
     @property
     def device(self):
         return next(self.parameters()).device
+
+    @classmethod
+    def from_pretrained(cls, path, torch_dtype=torch.bfloat16, device="cuda:0", **polar_options):
+        """The model of a Hugging Face checkpoint directory (config.json + safetensors), as the reference's
+        evaluation scripts obtain it (test4long.py:46-47); `polar_options`: PolarConfig's cache fields."""
+        from .checkpoint import load_pretrained
+        return load_pretrained(path, torch_dtype, device, model_class=cls, **polar_options)
 
     def forward(self, input_ids=None, attention_mask=None, past_key_values=None, num_logits_to_keep=0,
                 return_dict=True):
