@@ -41,6 +41,14 @@ def config_from_hf(hf: Dict, **polar_options) -> PolarConfig:
     if hf.get("sliding_window") and hf.get("use_sliding_window", kind == "mistral"):
         raise NotImplementedError("polarquant_amd: sliding-window attention is not implemented")
     fields = {k: hf[k] for k in _ARCH_FIELDS if hf.get(k) is not None}
+    rp = hf.get("rope_parameters")                          # transformers 5 writes one dict instead of theta + scaling
+    if isinstance(rp, dict):
+        if rp.get("rope_theta") is not None:
+            fields["rope_theta"] = rp["rope_theta"]
+        fields["rope_scaling"] = {k: v for k, v in rp.items() if k != "rope_theta"}
+    sc = fields.get("rope_scaling")
+    if isinstance(sc, dict) and sc.get("rope_type", sc.get("type", "default")) == "default":
+        fields.pop("rope_scaling")
     fields.setdefault("num_key_value_heads", fields["num_attention_heads"])
     fields.setdefault("head_dim", fields["hidden_size"] // fields["num_attention_heads"])
     if fields["head_dim"] != 128:

@@ -107,3 +107,38 @@ def test_wrong_checkpoints_are_refused(tmp_path):
     (tmp_path / "pytorch_model.bin").write_bytes(b"")
     with pytest.raises(FileNotFoundError):
         ck.load_pretrained(str(tmp_path), torch.float32, "cpu")
+
+
+@pytest.mark.parametrize("family", ["llama", "qwen2"])
+def test_directories_written_by_transformers_load(tmp_path, family):
+    """A checkpoint directory as Hugging Face's own `save_pretrained` writes it (a library, not the reference)."""
+    transformers = pytest.importorskip("transformers")
+    kw = dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, num_hidden_layers=2, intermediate_size=128,
+              vocab_size=96, max_position_embeddings=4096, eos_token_id=5)
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 8192}
+    torch.manual_seed(3)
+    if family == "llama":
+        try:
+            cfg = transformers.LlamaConfig(rope_parameters=dict(scaling, rope_theta=5e5), head_dim=128, **kw)
+            if getattr(cfg, "rope_parameters", None) is None:
+                raise TypeError
+        except TypeError:
+            cfg = transformers.LlamaConfig(rope_theta=5e5, rope_scaling=scaling, head_dim=128, **kw)
+        hf = transformers.LlamaForCausalLM(cfg)
+    else:
+        hf = transformers.Qwen2ForCausalLM(transformers.Qwen2Config(**kw))
+    hf.save_pretrained(str(tmp_path), safe_serialization=True)
+    got = ck.load_pretrained(str(tmp_path), torch.float32, "cpu")
+    assert type(got).__name__ == ("LlamaPolarForCausalLM" if family == "llama" else "Qwen2PolarForCausalLM")
+    want = dict(hf.named_parameters())
+    mine = dict(got.named_parameters())
+    assert set(mine) == set(want)
+    for name, p in mine.items():
+        assert torch.equal(p, want[name]), name
+    assert got.config.eos_token_id == [5]
+    if family == "llama":
+        from polarquant_amd.modeling_common import rope_parameters
+        theta, sc = rope_parameters(got.config)
+        assert theta == 5e5 and sc["rope_type"] == "llama3" and sc["factor"] == 8.0
+        assert torch.allclose(got.model.rotary_emb.inv_freq, hf.model.rotary_emb.inv_freq, rtol=1e-6, atol=0)
