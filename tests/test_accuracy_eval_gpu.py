@@ -101,3 +101,35 @@ def test_gsm8k_run(toy, tmp_path):
         assert r["score"] == metrics.judge_gsm8k(r["output_text"], r["answers"])
     assert ae.run_gsm8k(model, tok, gen, str(data), str(out), chat="none", max_new_tokens=12, limit=1) in (0.0, 1.0)
     assert len(out.read_text().splitlines()) == 1
+
+
+def test_command_line_with_a_tokenizer_directory(tmp_path, gpu, capsys):
+    """`python -m polarquant_amd.accuracy_eval ...` as a user runs it: the checkpoint directory also holds the
+    tokenizer files (here a byte-level tokenizer without merges, written with the `tokenizers` library)."""
+    transformers = pytest.importorskip("transformers")
+    from tokenizers import Tokenizer, decoders, models, pre_tokenizers
+    vocab = {ch: i for i, ch in enumerate(sorted(pre_tokenizers.ByteLevel.alphabet()))}
+    vocab["<|eot|>"] = 256
+    tk = Tokenizer(models.BPE(vocab=vocab, merges=[]))
+    tk.pre_tokenizer = pre_tokenizers.ByteLevel(add_prefix_space=False, use_regex=False)
+    tk.decoder = decoders.ByteLevel()
+    ckpt = tmp_path / "ckpt"
+    transformers.PreTrainedTokenizerFast(tokenizer_object=tk, eos_token="<|eot|>").save_pretrained(str(ckpt))
+    torch.manual_seed(12)
+    cfg = PolarConfig(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, num_hidden_layers=1,
+                      intermediate_size=128, vocab_size=257, eos_token_id=[256])
+    ck.save_pretrained(LlamaPolarForCausalLM(cfg), str(ckpt))
+    data = _longbench_dir(tmp_path)
+    ae.main(["longbench", "--model", str(ckpt), "--data", str(data), "--out", str(tmp_path / "o"), "--datasets", "lcc",
+             "--max-length", "300", "--limit", "1", "--rbits", "3", "--tbits", "3", "--variant", "mixed"])
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line["task"] == "longbench" and set(line["scores_x100"]) == {"lcc"} and 0 <= line["scores_x100"]["lcc"] <= 100
+    assert len((tmp_path / "o" / "lcc.jsonl").read_text().splitlines()) == 1
+    gs = tmp_path / "g.json"
+    gs.write_text(json.dumps({"conversations": [{"value": "1+1?"}, {"value": "The answer is 2"}]}) + "\n")
+    shots = tmp_path / "shots.txt"
+    shots.write_text("Question: 2+2?\nLet's think step by step\n2+2=4\nThe answer is 4\n")
+    ae.main(["gsm8k", "--model", str(ckpt), "--data", str(gs), "--out", str(tmp_path / "g.jsonl"), "--shots", str(shots),
+             "--chat", "none", "--variant", "snapkv"])
+    line = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert line["task"] == "gsm8k" and line["accuracy_x100"] in (0.0, 100.0)
