@@ -32,7 +32,7 @@ def _inputs(gpu, B, N, Nk, n_groups, n_resid, seed):
     return dev, ref64
 
 
-def _call(static, dev, B, N, Nk, n_groups, n_resid, n_splits, gpu):
+def _call(static, dev, B, N, Nk, n_groups, n_resid, n_splits, gpu, flags=0):
     q, codes, rs, rm, ts, tm, kres, v = dev
     out = torch.full((B, N, 128), float("nan"), dtype=torch.float16, device=gpu)
     head = [q.data_ptr(), codes.data_ptr(), rs.data_ptr(), rm.data_ptr(), ts.data_ptr(), tm.data_ptr(), n_groups,
@@ -40,11 +40,11 @@ def _call(static, dev, B, N, Nk, n_groups, n_resid, n_splits, gpu):
             1.0 / math.sqrt(128), B, N, Nk, 4, 4, _ffi.PQ_F16, n_splits, 0]
     lib = _ffi.lib()
     if static:
-        rc = lib.pq_decode_attn_static(*head, out.data_ptr(), 0, _stream_ptr(gpu))
+        rc = lib.pq_decode_attn_static(*head, out.data_ptr(), flags, _stream_ptr(gpu))
     else:
         nbytes = lib.pq_decode_attn_workspace_bytes(B, N, n_splits)
         ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device=gpu)
-        rc = lib.pq_decode_attn(*head, ws.data_ptr(), nbytes, out.data_ptr(), 0, _stream_ptr(gpu))
+        rc = lib.pq_decode_attn(*head, ws.data_ptr(), nbytes, out.data_ptr(), flags, _stream_ptr(gpu))
     assert rc == 0, _ffi.STATUS_NAMES.get(rc, rc)
     torch.cuda.synchronize()
     return out.cpu()
@@ -61,6 +61,20 @@ def test_static_entry_point_matches_workspace_entry_point(gpu):
         got = _call(True, dev, gpu=gpu, **shape)
         want = _call(False, dev, gpu=gpu, **shape)
         assert torch.isfinite(got.float()).all()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "call %d: outputs differ" % i
+        err = (got.double().reshape(ref64.shape) - ref64).abs()
+        assert bool((err <= 1e-3 + 1e-2 * ref64.abs()).all()), "call %d: off the oracle by %g" % (i, err.max().item())
+
+
+def test_static_entry_point_with_balanced_slices(gpu):
+    """The flags pass through: slices cut on the device (PQ_BALANCED_SLICES) leave some partial slots of the library's
+    buffer unused, which the second, smaller call must not read as results of the first."""
+    for i, (shape, seed) in enumerate(((dict(B=3, N=32, Nk=8, n_groups=9, n_resid=100, n_splits=6), 14),
+                                       (dict(B=1, N=32, Nk=8, n_groups=2, n_resid=0, n_splits=3), 15))):
+        print("pq_decode_attn_static balanced call", i, shape, flush=True)
+        dev, ref64 = _inputs(gpu, shape["B"], shape["N"], shape["Nk"], shape["n_groups"], shape["n_resid"], seed)
+        got = _call(True, dev, gpu=gpu, flags=_ffi.PQ_BALANCED_SLICES, **shape)
+        want = _call(False, dev, gpu=gpu, flags=_ffi.PQ_BALANCED_SLICES, **shape)
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "call %d: outputs differ" % i
         err = (got.double().reshape(ref64.shape) - ref64).abs()
         assert bool((err <= 1e-3 + 1e-2 * ref64.abs()).all()), "call %d: off the oracle by %g" % (i, err.max().item())
