@@ -191,3 +191,54 @@ def test_cfg1_full_size_with_4bit_values(gpu):
     for ns in (3, 8, 64):
         ok, err = _ok(attn(n_splits=ns).cpu(), out.cpu())
         assert ok, (ns, err)
+
+
+def test_cfg4_attention_layer_at_full_width(gpu):
+    """configs[4]'s shape for ONE attention layer of the drop-in class (hidden 4096, 32 query / 8 KV heads, bf16,
+    batch 8, prompt 16384, then decode steps across nothing but the residual window): the post-RoPE q / k / v the layer
+    saw are replayed through the oracle for sequence 0, cache contents bit for bit, outputs within the bf16 band of
+    the model test; the other sequences are held to batch invariance (sequence 5 alone == sequence 5 in the batch)."""
+    from polarquant_amd.modeling_common import PolarConfig
+    from polarquant_amd.modeling_llama_polar import LlamaPolarGroupAttention
+    torch.manual_seed(4)
+    cfg = PolarConfig.llama3_8b(num_hidden_layers=1)
+    att = LlamaPolarGroupAttention(cfg, 0).to(torch.bfloat16).to(gpu)
+    att.capture = []
+    B, L, steps = 8, 16384, 3
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+
+    def rope(start, n):
+        ang = torch.arange(start, start + n, dtype=torch.float32)[:, None] * inv[None]
+        emb = torch.cat([ang, ang], -1)[None]
+        return emb.cos().to(torch.bfloat16).to(gpu), emb.sin().to(torch.bfloat16).to(gpu)
+
+    g = torch.Generator(device=gpu).manual_seed(44)
+    x = torch.randn(B, L + steps, cfg.hidden_size, generator=g, device=gpu).mul_(0.5).to(torch.bfloat16)
+    with torch.no_grad():
+        _, cache = att(x[:, :L], attention_mask=None, past_key_value=None, position_embeddings=rope(0, L))
+        q, k, v = [t[:1].cpu() for t in att.capture[-1]]
+        ref_cache = po.prefill_cache(k, v, 4, 4)
+        assert cache[-1] == L and cache[1].shape[2] >= L // 128
+        for j in (1, 2, 3, 4, 5):                                       # codes and the four metadata tensors of sequence 0
+            got, ref = cache[j][:1, :, :L // 128].cpu(), ref_cache[j]
+            assert got.shape == ref.shape, j
+            assert torch.equal(got, ref) if got.dtype == torch.uint8 else bool((got.float() == ref.float()).all()), "tuple element %d" % j
+        o_proj = att.o_proj.weight.detach().float().cpu()
+        solo_cache = None
+        for i in range(steps):
+            out, cache = att(x[:, L + i:L + i + 1], attention_mask=None, past_key_value=cache, position_embeddings=rope(L + i, 1))
+            q, k, v = [t[:1].cpu() for t in att.capture[-1]]
+            ref_attn, ref_cache = po.decode_step(q, k, v, ref_cache, None, 4, 4)
+            ref_out = ref_attn.reshape(1, 1, -1).float() @ o_proj.T
+            err = (out[:1].float().cpu() - ref_out).abs().max().item()
+            assert err < 2e-2 * max(1.0, ref_out.abs().max().item()), (i, err)
+        assert cache[-1] == L + steps
+        # batch invariance: sequence 5 on its own gives the bits it gave inside the batch
+        att.capture = []
+        _, solo_cache = att(x[5:6, :L], attention_mask=None, past_key_value=None, position_embeddings=rope(0, L))
+        solo, _ = att(x[5:6, L:L + 1], attention_mask=None, past_key_value=solo_cache, position_embeddings=rope(L, 1))
+        _, again = att(x[:, :L], attention_mask=None, past_key_value=None, position_embeddings=rope(0, L))
+        batched, _ = att(x[:, L:L + 1], attention_mask=None, past_key_value=again, position_embeddings=rope(L, 1))
+        assert torch.equal(solo_cache[1][0, :, :L // 128], again[1][5, :, :L // 128])
+        close = (solo[0].float() - batched[5].float()).abs().max().item()
+        assert close <= 2e-2 * max(1.0, batched[5].float().abs().max().item()), close
