@@ -87,6 +87,15 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * the context at all). */
 #define PQ_BALANCED_SLICES 16u
 
+/* flag for the attention entry points with half-precision values: one wavefront per slice does everything
+ * (codes, tables, scores, then values, softmax, P.V in turn), as the kernels for 4-bit values do.  Without it
+ * (the default) a slice is shared by the two wavefronts that sit on one SIMD: a scorer (codes, tables, scores)
+ * and an accumulator (values, mask, softmax, P.V) that hand 64-token tiles of scores over through LDS, so the
+ * two halves of the work overlap; the results differ only as two split counts differ (fp32 summation order
+ * is the same: the tiles are accumulated in the same order).  Kept for comparison and as the fall-back.
+ * No reference counterpart. */
+#define PQ_SINGLE_WAVEFRONT 32u
+
 /* Linear layer of a decode step: y[M, N] = x[M, K] . w[N, K]^T (+ bias[N]), M <= 16 rows (one new
  * token per sequence), fp32 accumulation, one rounding to the dtype.  Replaces the q/k/v, o and MLP
  * projections (`nn.Linear`) the decode step calls around the attention
@@ -232,7 +241,8 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
  *   out      [B,N,128] half words
  *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48) and / or
- *            PQ_BALANCED_SLICES (slices cut on the device from the per-sequence counts, see above)
+ *            PQ_BALANCED_SLICES (slices cut on the device from the per-sequence counts, see above) and / or
+ *            PQ_SINGLE_WAVEFRONT (one wavefront per slice instead of a scorer / accumulator pair)
  * Limits: v_capacity <= PQ_MAX_PLANE_TOKENS tokens and group_capacity <= 2^17 groups per (batch, KV head)
  * plane (32-bit byte sizes and offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */

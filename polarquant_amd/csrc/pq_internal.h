@@ -60,6 +60,7 @@ struct AttnArgs {
     int B, N, Nk, tbits, dtype, n_splits, min_groups_per_split;
     bool packed6 = false;        // code rows are 48 bytes of packed 6-bit codes (tbits == 3 only)
     bool balanced = false;       // slices cut on the device from the per-sequence counts (PQ_BALANCED_SLICES)
+    bool single_wave = false;    // one wavefront per slice instead of a scorer / accumulator pair (PQ_SINGLE_WAVEFRONT)
     float* workspace;
     void* out;
 };
