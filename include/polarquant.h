@@ -77,10 +77,10 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * the device from the per-sequence counts, so that every wavefront gets the same amount of work
  * whatever the lengths are (ragged batches; batches that grow under a replayed graph).  All planes
  * ((sequence, KV head) pairs) are laid end to end in tiles of 64 tokens (two per quantized group, then
- * one per 64 residual keys, behind two units that stand for a plane's start-up), and the line is cut into equal segments, one per wavefront the device holds
+ * one per 64 residual keys, behind three units that stand for a plane's start-up), and the line is cut into equal segments, one per wavefront the device holds
  * at once; a segment may end one plane and begin the next, and may cut a group in half.  n_splits is
  * then the number of partial slots per query head (>= 2): no plane is cut into more pieces than that (the
- * segment length is raised to ceil((2 group_capacity + ceil(resid_capacity / 64) + 2) / (n_splits - 1)) tiles if it has
+ * segment length is raised to ceil((2 group_capacity + ceil(resid_capacity / 64) + 3) / (n_splits - 1)) tiles if it has
  * to be),
  * min_groups_per_split a lower bound on the segment length in groups.  Results do not depend on how the
  * line is cut beyond fp32 summation order.  No reference counterpart (the reference has no split over

@@ -55,11 +55,11 @@ def balanced_slots(B: int, Nk: int, group_capacity: int, total_groups: Optional[
                    resid_capacity: int = GROUP) -> int:
     """Partial slots per head for PQ_BALANCED_SLICES: enough for the segment length the device will pick
     when the batch holds `total_groups` groups per KV head (None: sequences half full on average)."""
-    # in tiles of 64 tokens: two per group, and per sequence one for its residual keys (on average) and two that
+    # in tiles of 64 tokens: two per group, and per sequence one for its residual keys (on average) and three that
     # stand for a plane's start-up
-    units = 2 * (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + 3 * B
+    units = 2 * (total_groups if total_groups is not None else (B * group_capacity + 1) // 2) + 4 * B
     seg = max(1, -(-units * Nk // max(wave_slots, 1)))
-    return max(2, -(-(2 * group_capacity + -(-resid_capacity // 64) + 2) // seg) + 1)
+    return max(2, -(-(2 * group_capacity + -(-resid_capacity // 64) + 3) // seg) + 1)
 
 
 def _pick_workspace(workspace: Optional[torch.Tensor], B: int, N: int, n_splits: int, device: torch.device) -> torch.Tensor:
@@ -85,7 +85,7 @@ def polar_decode_attention(
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
     total_groups: Optional[int] = None, min_groups_per_split: Optional[int] = None,
-    workspace: Optional[torch.Tensor] = None, balanced: Optional[bool] = None,
+    workspace: Optional[torch.Tensor] = None, balanced: Optional[bool] = None, single_wavefront: bool = False,
 ) -> torch.Tensor:
     """-> attention output [B,N,1,128] in the query dtype.
 
@@ -97,7 +97,9 @@ def polar_decode_attention(
     device from the actual counts so that all wavefronts get equal work (PQ_BALANCED_SLICES);
     `n_splits` is then the number of partial slots per head.
     `workspace`: a buffer from `new_workspace` that the caller owns (needed under graph capture);
-    by default the cached buffer of the current stream is used."""
+    by default the cached buffer of the current stream is used.
+    `single_wavefront`: the earlier kernels, in which one wavefront does all the work of a slice
+    (PQ_SINGLE_WAVEFRONT), instead of the scorer / accumulator pairs; for comparison."""
     if not query_states.is_cuda:
         raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
     dev = query_states.device
@@ -134,6 +136,8 @@ def polar_decode_attention(
     min_gps = 0
     if balanced is None:
         balanced = n_groups_per_seq is not None and n_splits is None and min_groups_per_split is None
+    if single_wavefront:
+        flags |= _ffi.PQ_SINGLE_WAVEFRONT
     if balanced:
         flags |= _ffi.PQ_BALANCED_SLICES
         if n_splits is None:

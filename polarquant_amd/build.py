@@ -18,7 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libpolarquant_hip.so")
-SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_attn.hip"]
+SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_attn.hip", "pq_attn_pair.hip"]
 # measurement aids (a plain streaming read, the attention kernel's loads without its arithmetic): a library of
 # their own, loaded by bench.py and its tests only
 BENCH_LIB = os.path.join(HERE, "libpolarquant_bench.so")
@@ -66,7 +66,7 @@ def build(verbose: bool = True, phase_timers: bool = False) -> str:
     os.makedirs(OBJ, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     lib, defines, tag = (TIMERS_LIB, ("PQ_ATTN_PHASE_TIMERS",), ".timers") if phase_timers else (LIB, (), "")
-    with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         objs = list(ex.map(lambda s_: _compile(s_, defines, tag), srcs))
     _link(objs, lib)
     if not phase_timers:

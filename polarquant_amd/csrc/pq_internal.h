@@ -65,6 +65,8 @@ struct AttnArgs {
     void* out;
 };
 int launch_attn_partials(const AttnArgs& a, hipStream_t st);
+// the default kernels for half-precision values (pq_attn_pair.hip); called by launch_attn_partials
+int launch_attn_pair(const AttnArgs& a, int total, hipStream_t st);
 int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st);
 
 // Device address, on the current device, of the library's own buffer for split partials

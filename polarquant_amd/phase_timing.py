@@ -1,4 +1,6 @@
-"""Where a wavefront of the fused decode-attention kernel spends its time, phase by phase.
+"""Where a wavefront of the one-wavefront-per-slice decode-attention kernel (PQ_SINGLE_WAVEFRONT, and the form the
+kernels for 4-bit values have) spends its time, phase by phase: the measurement that led to the scorer / accumulator
+pairs of the default kernels, whose two wavefronts overlap what is added up here.
 
 Needs the measuring build of the library (`python -m polarquant_amd.build --phase-timers`), whose attention
 kernel brackets its phases with the 100 MHz wall clock and lets every 97th wavefront print its sums.  The
@@ -58,7 +60,8 @@ def main():
         kw.pop("balanced", None)
         call = lambda: polar_decode_attention_v4(w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], **kw)
     else:
-        call = lambda: polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], **kw)
+        call = lambda: polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"],
+                                              single_wavefront=True, **kw)
     torch.cuda.synchronize()
     sys.stdout.flush()
     # the kernel prints from the device: collect the process's stdout of one launch in a file

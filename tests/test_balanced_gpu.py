@@ -9,9 +9,26 @@ import torch
 from oracle import polar_oracle as po
 from polarquant_amd import attention
 from polarquant_amd import workloads as wl
-from polarquant_amd.attention import polar_decode_attention, polar_decode_attention_v4
+from polarquant_amd.attention import polar_decode_attention as _polar_decode_attention
+from polarquant_amd.attention import polar_decode_attention_v4
 
 pytestmark = pytest.mark.gpu
+
+
+# Every test of this file runs twice: with the default kernels (a scorer / accumulator pair of wavefronts per slice)
+# and with one wavefront per slice (PQ_SINGLE_WAVEFRONT).
+_FORM = {"single": False}
+
+
+@pytest.fixture(autouse=True, params=[False, True], ids=["pairs", "single"])
+def _kernel_form(request):
+    _FORM["single"] = request.param
+    yield
+    _FORM["single"] = False
+
+
+def polar_decode_attention(*args, **kwargs):
+    return _polar_decode_attention(*args, single_wavefront=_FORM["single"], **kwargs)
 
 
 def _ragged(gpu, B, N, Nk, lens, rb, tb, dtype, seed, gcap_extra=0, mask=False):

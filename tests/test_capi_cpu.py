@@ -140,6 +140,11 @@ def test_validate_decode_attn_and_plan(lib):
     assert lib.pq_validate_decode_attn(*a) == 0
     a[24], a[27] = 1, lib.pq_decode_attn_workspace_bytes(B, N, 1)
     assert lib.pq_validate_decode_attn(*a) == -7
+    a = list(ok); a[29] = 32
+    assert lib.pq_validate_decode_attn(*a) == 0                      # PQ_SINGLE_WAVEFRONT, alone or with balanced slices
+    a[29] = 32 | 16
+    assert lib.pq_validate_decode_attn(*a) == 0
+    assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 32) == -2
     a = list(ok); a[29] = 64
     assert lib.pq_validate_decode_attn(*a) == -2                     # unknown flag bit
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 16) == -2

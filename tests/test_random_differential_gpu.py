@@ -98,7 +98,8 @@ def test_random_decode_attention_case(gpu, seed):
         vq_d = [dev(vcodes)] + [dev(m) for m in vmeta] if have_groups else [None] * 3
         out = polar_decode_attention_v4(dev(q), *cq, dev(kres), dev(vres), *vq_d, ng, nr, **kw)
     else:
-        out = polar_decode_attention(dev(q), *cq, dev(kres), dev(vfull), ng, nr, **kw)
+        # one case in four takes the one-wavefront-per-slice kernels instead of the scorer / accumulator pairs
+        out = polar_decode_attention(dev(q), *cq, dev(kres), dev(vfull), ng, nr, single_wavefront=seed % 4 == 3, **kw)
     out = out.cpu()
     assert torch.isfinite(out.float()).all()
     # the band is centred on the fp64 value and widened, element by element, by the distance of the
