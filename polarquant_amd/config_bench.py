@@ -34,7 +34,7 @@ def _entry(op, ms, nbytes, **extra):
                 frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)
 
 
-def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool = False):
+def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool = False, single_wavefront: bool = False):
     """Time configs[idx] -> (list of measurement dicts, the workload).  The workload keeps what a caller
     needs to check the timed calls' results against a CPU checker: w["scores"] (configs[0]), w["out"] (decode
     attention output), w["append_out"] (configs[3]: codes and metadata the timed quantizer calls wrote) and
@@ -77,8 +77,10 @@ def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool
     out = torch.empty(B, N, 1, 128, dtype=w["q"].dtype, device=dev)
     ms = wl.time_events(lambda: polar_decode_attention(
         w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
-        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups, out=out), steps, 10)
-    res.append(_entry("decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else ""), ms, nbytes,
+        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups, out=out,
+        single_wavefront=single_wavefront), steps, 10)
+    res.append(_entry("decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else "")
+                      + (", one wavefront per slice" if single_wavefront else ""), ms, nbytes,
                       tokens=int(sum(lq) + sum(rs))))
     w["out"] = out
     if values4 and not sh.ragged:
@@ -103,8 +105,8 @@ def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool
     return res, w
 
 
-def run(idx: int, dev, values4: bool, steps: int, packed: bool = False):
-    res, _ = measure(idx, dev, values4, steps, packed)
+def run(idx: int, dev, values4: bool, steps: int, packed: bool = False, single_wavefront: bool = False):
+    res, _ = measure(idx, dev, values4, steps, packed, single_wavefront)
     for r in res:
         print(json.dumps(dict(config=idx, **r)), flush=True)
 
@@ -115,16 +117,17 @@ def main():
     ap.add_argument("--values4", action="store_true")
     ap.add_argument("--packed", action="store_true", help="also run the 3/3-bit configuration with packed 6-bit code rows")
     ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--single-wavefront", action="store_true", help="decode attention with one wavefront per slice (PQ_SINGLE_WAVEFRONT) instead of the scorer / accumulator pairs")
     ap.add_argument("--no-ramp", action="store_true", help="no clock ramp before the timed regions (counter-collection runs under the profiler)")
     args = ap.parse_args()
     if args.no_ramp:
         wl.RAMP_SECONDS = 0.0
     dev = torch.device("cuda:0")
     for idx in args.configs:
-        run(idx, dev, args.values4, args.steps)
+        run(idx, dev, args.values4, args.steps, single_wavefront=args.single_wavefront)
         torch.cuda.empty_cache()
         if args.packed and wl.CONFIGS[idx].rbits + wl.CONFIGS[idx].tbits <= 6:
-            run(idx, dev, False, args.steps, packed=True)
+            run(idx, dev, False, args.steps, packed=True, single_wavefront=args.single_wavefront)
             torch.cuda.empty_cache()
 
 
