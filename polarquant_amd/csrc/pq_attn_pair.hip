@@ -32,6 +32,23 @@ struct PairMem {
 
 typedef __attribute__((address_space(3))) volatile int lds_vi;
 
+// Measuring build only (-DPQ_ATTN_PHASE_TIMERS): every wavefront adds up the wall-clock time (100 MHz) it spends in
+// pair_wait, and the wavefronts of every 97th workgroup print it with their role when their kernel ends.
+#ifdef PQ_ATTN_PHASE_TIMERS
+#define PQ_PAIR_T_DECL long long pw_total_ = 0; const long long pw_entry_ = wall_clock64()
+#define PQ_PAIR_T_WAIT(call) [&]() { const long long t0_ = wall_clock64(); const bool r_ = (call); pw_total_ += wall_clock64() - t0_; return r_; }()
+#define PQ_PAIR_T_REPORT(role, tiles)                                                                                \
+    do {                                                                                                             \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x % 97 == 0)                                                         \
+            printf("pq_pair block %d wave %d role %d tiles %d life %lld waited %lld\n", static_cast<int>(blockIdx.x),  \
+                   static_cast<int>(threadIdx.x >> 6), role, tiles, wall_clock64() - pw_entry_, pw_total_);          \
+    } while (0)
+#else
+#define PQ_PAIR_T_DECL
+#define PQ_PAIR_T_WAIT(call) (call)
+#define PQ_PAIR_T_REPORT(role, tiles)
+#endif
+
 __device__ __forceinline__ bool pair_wait(uint32_t addr, int want) {
     bool seen = false;
     for (int i = 0; i < kSpinLimit; i++) {
@@ -70,14 +87,14 @@ __device__ __forceinline__ void pair_roles(int* simd_of, int* flags, int wave, i
 // has handed over since the kernel began.  -> false if the partner stopped answering.
 template <typename T, int TB, int REPP, bool PK6>
 __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& pm, int lane, int b, int kvh, const SeqCounts& sc,
-                                            int t0, int t1, int r0, int r1, int& k) {
+                                            int t0, int t1, int r0, int r1, int& k, long long& pw_total_) {
     const int rep = p.rep;
     const int bh = b * p.Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
     const uint16_t* qb = p.q + (static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * rep) * kHeadDim;
     bool ok = true;
     auto publish_begin = [&]() {            // the buffer of tile k is free once tile k - 2 has been consumed
-        if (k >= 2) ok = ok && pair_wait(pm.flags + 4, k - 1);
+        if (k >= 2) ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1));
         return pm.sbuf + (k & 1) * (REPP * kWave * 4);
     };
     auto publish_end = [&]() {
@@ -201,7 +218,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
 // Accumulator: the same tiles in the same order; writes the partial of the piece to `slot`.
 template <typename T, int REPP>
 __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const PairMem& pm, int lane, int b, int kvh, const SeqCounts& sc,
-                                                 int t0, int t1, int r0, int r1, int slot, int& k) {
+                                                 int t0, int t1, int r0, int r1, int slot, int& k, long long& pw_total_) {
     const int N = p.N, rep = p.rep;
     const int bh = b * p.Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
@@ -229,7 +246,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         const bool resid = i >= nq;
         const bool valid = resid ? (r0 + i - nq) * kWave + lane < nres : true;
         const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, row, 0) != 0) : true);
-        ok = ok && pair_wait(pm.flags, k + 1);
+        ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags, k + 1));
         const uint32_t src = pm.sbuf + (k & 1) * (REPP * kWave * 4);
         float s[REPP];
 #pragma unroll
@@ -313,8 +330,14 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
     const int r1 = split == last_split ? (sc.nres + kWave - 1) / kWave : 0;
     int k = 0;
-    if (role == 0) pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k);
-    else           pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k);
+    long long waited = 0;
+    PQ_PAIR_T_DECL;
+    if (role == 0) pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited);
+    else           pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited);
+#ifdef PQ_ATTN_PHASE_TIMERS
+    pw_total_ = waited;
+#endif
+    PQ_PAIR_T_REPORT(role, k);
 }
 
 
@@ -341,16 +364,22 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     if (w >= n_pairs_total) return;
     int k = 0;
     bool ok = true;
+    long long waited = 0;
+    PQ_PAIR_T_DECL;
     walk_segment<false>(p, v4, n_pairs_total, w, lane, lds_addr(walk_mem[wave]),
                         [&](int cb, int ckvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot, bool ends_plane) {
                             if (!ok) return;         // the partner stopped answering: run out without touching anything
                             if (role == 0) {
-                                ok = pair_scorer<T, TB, REPP, PK6>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, k);
+                                ok = pair_scorer<T, TB, REPP, PK6>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, k, waited);
                             } else {
                                 if (ends_plane && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
-                                ok = pair_accumulator<T, REPP>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, slot, k);
+                                ok = pair_accumulator<T, REPP>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, slot, k, waited);
                             }
                         });
+#ifdef PQ_ATTN_PHASE_TIMERS
+    pw_total_ = waited;
+#endif
+    PQ_PAIR_T_REPORT(role, k);
 }
 
 #pragma clang diagnostic pop

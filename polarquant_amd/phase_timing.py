@@ -36,6 +36,8 @@ def main():
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--values4", action="store_true")
     ap.add_argument("--even", action="store_true", help="ragged batches: even slices per sequence instead of balanced slices")
+    ap.add_argument("--pairs", action="store_true", help="the default kernels instead (a scorer / accumulator pair of wavefronts per slice): "
+                    "how long each role waits for the other")
     ap.add_argument("--pieces", action="store_true", help="also list every reporting piece: block, groups, us from the first entry to its entry and exit")
     args = ap.parse_args()
     if not os.path.exists(TIMERS_LIB):
@@ -61,7 +63,7 @@ def main():
         call = lambda: polar_decode_attention_v4(w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], **kw)
     else:
         call = lambda: polar_decode_attention(w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"],
-                                              single_wavefront=True, **kw)
+                                              single_wavefront=not args.pairs, **kw)
     torch.cuda.synchronize()
     sys.stdout.flush()
     # the kernel prints from the device: collect the process's stdout of one launch in a file
@@ -76,6 +78,23 @@ def main():
             os.close(saved)
         tmp.seek(0)
         text = tmp.read().decode(errors="replace")
+    if args.pairs:
+        roles = {0: [], 1: []}
+        for line in text.splitlines():
+            m = re.match(r"pq_pair block (\d+) wave (\d+) role (\d+) tiles (\d+) life (\d+) waited (\d+)", line)
+            if m and int(m.group(4)) > 0:
+                roles[int(m.group(3))].append((int(m.group(4)), int(m.group(5)) * 0.01, int(m.group(6)) * 0.01))
+        if not roles[0] or not roles[1]:
+            sys.exit("phase_timing: no pair reported (is this the measuring build?)")
+        out = {"config": args.config, "kernels": "scorer / accumulator pairs"}
+        for r, name in ((0, "scorer"), (1, "accumulator")):
+            v = roles[r]
+            out[name] = {"wavefronts_reporting": len(v), "tiles": round(sum(t for t, _, _ in v) / len(v), 1),
+                         "life_us": round(sum(l for _, l, _ in v) / len(v), 2),
+                         "waiting_for_the_partner_us": round(sum(x for _, _, x in v) / len(v), 2),
+                         "waiting_share": round(sum(x for _, _, x in v) / sum(l for _, l, _ in v), 3)}
+        print(json.dumps(out))
+        return
     rows = []
     for line in text.splitlines():
         m = re.match(r"pq_phase block (\d+) groups (\d+) total (\d+) " + " ".join(p + r" (\d+)" for p in PHASES), line)
