@@ -96,6 +96,11 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * No reference counterpart. */
 #define PQ_SINGLE_WAVEFRONT 32u
 
+/* test hook of the same entry points (default kernels only): the scorers publish nothing, and the bounded waits of
+ * the hand-over give up after 1000 polls instead of 2^22.  Every kernel still ends normally; every output of the
+ * call is NaN.  For the test that a hand-over which fails can neither hang the GPU nor pass for a result. */
+#define PQ_TEST_SILENT_SCORER 0x40000000u
+
 /* Linear layer of a decode step: y[M, N] = x[M, K] . w[N, K]^T (+ bias[N]), M <= 16 rows (one new
  * token per sequence), fp32 accumulation, one rounding to the dtype.  Replaces the q/k/v, o and MLP
  * projections (`nn.Linear`) the decode step calls around the attention

@@ -20,6 +20,7 @@ PQ_CODES_PACKED6 = 4
 PQ_DEVICE_ATAN2 = 8
 PQ_BALANCED_SLICES = 16
 PQ_SINGLE_WAVEFRONT = 32
+PQ_TEST_SILENT_SCORER = 0x40000000
 PQ_EAGER_GPU = PQ_WRAP_FP32 | PQ_DEVICE_ATAN2
 
 STATUS_NAMES = {

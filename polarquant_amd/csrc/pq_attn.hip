@@ -459,7 +459,8 @@ __global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __rest
     for (int i = 1; i < NW; i++) den += red[1][i];
 #pragma unroll
     for (int i = 1; i < G; i++) num += part[i][d];
-    out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : 0.0f);
+    // nothing to attend to (den == 0) gives zeros; a NaN among the partials (a poisoned slice) must stay visible
+    out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : (den == den ? 0.0f : den));
 }
 
 // Wavefront slots of the current device for the balanced kernel: one wavefront per SIMD (4 per

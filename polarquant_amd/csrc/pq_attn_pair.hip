@@ -12,7 +12,9 @@
 // The two hand tiles over through two counters in LDS (tiles published / tiles consumed); a wait
 // gives up after kSpinLimit polls (about half a second), after which both wavefronts run out
 // without waiting again and the accumulator writes NaN into the piece's partial: a failed hand-over
-// cannot pass for a result, and no wavefront can wait for ever.
+// cannot pass for a result, and no wavefront can wait for ever.  PQ_TEST_SILENT_SCORER makes the
+// scorers publish nothing and the waits give up after 1000 polls, so that a test can see exactly
+// that: every kernel ends, every output is NaN.
 #include "pq_attn_device.h"
 
 namespace pq {
@@ -22,12 +24,15 @@ namespace pq {
 
 constexpr int kPairsPerBlock = 4;
 constexpr int kSpinLimit = 1 << 22;
+constexpr int kSpinLimitSilent = 1000;      // with PQ_TEST_SILENT_SCORER: the waits' time-out is what is being tested
 
 struct PairMem {
     uint32_t lut;      // the scorer's table
     uint32_t sbuf;     // [2][REPP][64] fp32 scores
     uint32_t pbuf;     // the accumulator's probability staging
     uint32_t flags;    // int[4]: tiles published by the scorer, tiles consumed by the accumulator, -, -
+    int spin_limit;    // polls after which a wait gives up
+    bool silent;       // PQ_TEST_SILENT_SCORER: the scorer publishes nothing
 };
 
 typedef __attribute__((address_space(3))) volatile int lds_vi;
@@ -49,9 +54,9 @@ typedef __attribute__((address_space(3))) volatile int lds_vi;
 #define PQ_PAIR_T_REPORT(role, tiles)
 #endif
 
-__device__ __forceinline__ bool pair_wait(uint32_t addr, int want) {
+__device__ __forceinline__ bool pair_wait(uint32_t addr, int want, int spin_limit) {
     bool seen = false;
-    for (int i = 0; i < kSpinLimit; i++) {
+    for (int i = 0; i < spin_limit; i++) {
         if (*lds_ptr<lds_vi>(addr) >= want) { seen = true; break; }
         __builtin_amdgcn_s_sleep(1);
     }
@@ -94,13 +99,13 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
     const uint16_t* qb = p.q + (static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * rep) * kHeadDim;
     bool ok = true;
     auto publish_begin = [&]() {            // the buffer of tile k is free once tile k - 2 has been consumed
-        if (k >= 2) ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1));
+        if (k >= 2) ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1, pm.spin_limit));
         return pm.sbuf + (k & 1) * (REPP * kWave * 4);
     };
     auto publish_end = [&]() {
         asm volatile("" ::: "memory");
         k++;
-        if (lane == 0) *lds_ptr<lds_vi>(pm.flags) = k;
+        if (lane == 0 && !pm.silent) *lds_ptr<lds_vi>(pm.flags) = k;
         asm volatile("" ::: "memory");
     };
     if (t0 < t1) {
@@ -246,7 +251,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         const bool resid = i >= nq;
         const bool valid = resid ? (r0 + i - nq) * kWave + lane < nres : true;
         const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, row, 0) != 0) : true);
-        ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags, k + 1));
+        ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags, k + 1, pm.spin_limit));
         const uint32_t src = pm.sbuf + (k & 1) * (REPP * kWave * 4);
         float s[REPP];
 #pragma unroll
@@ -291,7 +296,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
 // Even slices, one slice per pair: pair index = 4 * blockIdx.x + (pair within the block), laid out as attn_kernel's
 // block index (plane fastest).
 template <typename T, int TB, int REPP, bool PK6>
-__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total) {
+__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer) {
     using L = Lut<TB, REPP>;
     __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
@@ -307,6 +312,8 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     pm.sbuf = lds_addr(s_mem[pair]);
     pm.pbuf = lds_addr(p_mem[pair]);
     pm.flags = lds_addr(flag_mem[pair]);
+    pm.silent = silent_scorer != 0;
+    pm.spin_limit = pm.silent ? kSpinLimitSilent : kSpinLimit;
 
     const int slice = blockIdx.x * kPairsPerBlock + pair;
     if (slice >= n_slices_total) return;
@@ -343,7 +350,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
 
 // Balanced slices for pairs: both wavefronts of a pair walk the same segment and meet tile by tile.
 template <typename T, int TB, int REPP, bool PK6>
-__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total) {
+__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total, int silent_scorer) {
     using L = Lut<TB, REPP>;
     __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
@@ -360,6 +367,8 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     pm.sbuf = lds_addr(s_mem[pair]);
     pm.pbuf = lds_addr(p_mem[pair]);
     pm.flags = lds_addr(flag_mem[pair]);
+    pm.silent = silent_scorer != 0;
+    pm.spin_limit = pm.silent ? kSpinLimitSilent : kSpinLimit;
     const int w = blockIdx.x * kPairsPerBlock + pair;
     if (w >= n_pairs_total) return;
     int k = 0;
@@ -398,7 +407,7 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
-                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0)
 #define PQ_LAUNCH_PAIR_P(REPP, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_PAIR_K(attn_pair_balanced_kernel, REPP, PK6);                                      \

@@ -17,7 +17,7 @@ int check_bits(int rbits, int tbits) {
 // decode-side flags: only the packed 6-bit code layout, which exists for tbits == 3 (rbits <= 3)
 int check_decode_flags(unsigned flags, int rbits, int tbits, bool attention = false) {
     // the score op has one slice per group; only the attention entry points cut the context
-    const unsigned known = PQ_CODES_PACKED6 | (attention ? (PQ_BALANCED_SLICES | PQ_SINGLE_WAVEFRONT) : 0u);
+    const unsigned known = PQ_CODES_PACKED6 | (attention ? (PQ_BALANCED_SLICES | PQ_SINGLE_WAVEFRONT | PQ_TEST_SILENT_SCORER) : 0u);
     if (flags & ~known) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && (tbits != 3 || rbits + tbits > 6)) return PQ_ERR_BAD_BITS;
     return PQ_OK;
@@ -225,6 +225,7 @@ int pq_decode_attn_partials(const void* q,
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
+    a.silent_scorer = (flags & PQ_TEST_SILENT_SCORER) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
@@ -509,6 +510,7 @@ int pq_decode_attn_v4(const void* q,
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
+    a.silent_scorer = (flags & PQ_TEST_SILENT_SCORER) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     if (any_groups) {
         a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token

@@ -145,6 +145,8 @@ def test_validate_decode_attn_and_plan(lib):
     a[29] = 32 | 16
     assert lib.pq_validate_decode_attn(*a) == 0
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 32) == -2
+    a = list(ok); a[29] = 0x40000000
+    assert lib.pq_validate_decode_attn(*a) == 0                      # PQ_TEST_SILENT_SCORER (test hook of the hand-over)
     a = list(ok); a[29] = 64
     assert lib.pq_validate_decode_attn(*a) == -2                     # unknown flag bit
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 16) == -2
