@@ -1,16 +1,18 @@
-// Fused polar-key decode attention: quantized-key scores, fp16 residual-key
-// scores, 1/sqrt(d), mask, softmax and P.V in one pass over HBM
-// (reference decode branch: models/modeling_llama_polar.py:66-99), split over
-// the context, followed by a small merge kernel.
+// Fused polar-key decode attention, the kernels with ONE wavefront per slice: quantized-key scores,
+// half-precision residual-key scores, 1/sqrt(d), mask, softmax and P.V in one pass over HBM
+// (reference decode branch: models/modeling_llama_polar.py:66-99), split over the context; and the
+// small merge kernel that follows every attention kernel.  These kernels serve the 4-bit values of the
+// Mixed variant and PQ_SINGLE_WAVEFRONT; with half-precision values the default kernels are the
+// scorer / accumulator pairs of pq_attn_pair.hip, which share the device code of pq_attn_device.h.
 //
 // attn_kernel: grid n_splits * B*Nk (plane index fastest), one wavefront per block: a block works
 // through one slice of its sequence's quantized groups; the last block of
-// a (batch, KV head) then also takes the fp16 residual keys (0..128 tokens).
+// a (batch, KV head) then also takes the residual keys (0..128 tokens).
 // The kernel is built for ONE resident wavefront per SIMD (4 per CU) with deep
 // software prefetch instead of many wavefronts: V operands are double-buffered
 // a whole 64-token tile ahead, which keeps ~40 KiB of loads in flight per
 // wavefront; pq_decode_attn_plan sizes n_splits so that B*Nk*n_splits fills
-// those slots exactly once.
+// those slots exactly once.  (With 4-bit values at up to 4 heads per KV head: two per SIMD.)
 // Each wavefront walks its tokens in 64-token tiles, lane == token, and keeps
 // flash-style running state (m, l, acc) for the `rep` query heads of its KV
 // head.  P.V runs on the matrix cores: for 16 tokens at a time
