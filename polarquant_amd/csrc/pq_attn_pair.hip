@@ -223,7 +223,8 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
 // Accumulator: the same tiles in the same order; writes the partial of the piece to `slot`.
 template <typename T, int REPP>
 __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const PairMem& pm, int lane, int b, int kvh, const SeqCounts& sc,
-                                                 int t0, int t1, int r0, int r1, int slot, int& k, long long& pw_total_) {
+                                                 int t0, int t1, int r0, int r1, int slot, int& k, long long& pw_total_,
+                                                 uint16_t* direct_out = nullptr) {
     const int N = p.N, rep = p.rep;
     const int bh = b * p.Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
@@ -281,6 +282,24 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
 #pragma unroll
         for (int j = 1; j < REPP; j++) { mm = (n == j) ? st.m[j] : mm; ll = (n == j) ? lsum[j] : ll; }
         if (!ok) mm = __builtin_nanf("");            // the scorer stopped answering: poison the result
+        if (direct_out) {
+            // the only slice of its plane: what the merge kernel would make of this one partial, written directly
+            // (weight exp2(m - m) = 1, so out = acc / l; no token to attend to -> zeros; a poisoned slice -> NaN)
+            const float den = (mm != mm) ? mm : ll;
+            uint16_t* po = direct_out + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * kHeadDim + 32 * g;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    const float lo = den > 0.0f ? st.acc[e][i] / den : (den == den ? 0.0f : den);
+                    const float hi = den > 0.0f ? st.acc[e + 1][i] / den : (den == den ? 0.0f : den);
+                    w[e >> 1] = static_cast<uint32_t>(f2lo<T>(lo)) | (static_cast<uint32_t>(f2lo<T>(hi)) << 16);
+                }
+                *reinterpret_cast<uint4*>(po + 8 * i) = make_uint4(w[0], w[1], w[2], w[3]);
+            }
+            return ok;
+        }
         float* pw = p.ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * p.n_splits + slot) * kPartialFloats;
         if (g == 0) { pw[0] = mm; pw[1] = ll; }
         float* pa = pw + 4 + 32 * g;
@@ -296,7 +315,8 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
 // Even slices, one slice per pair: pair index = 4 * blockIdx.x + (pair within the block), laid out as attn_kernel's
 // block index (plane fastest).
 template <typename T, int TB, int REPP, bool PK6>
-__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer) {
+__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer,
+                                                                              uint16_t* __restrict__ direct_out) {
     using L = Lut<TB, REPP>;
     __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
@@ -340,7 +360,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     long long waited = 0;
     PQ_PAIR_T_DECL;
     if (role == 0) pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited);
-    else           pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited);
+    else           pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
 #ifdef PQ_ATTN_PHASE_TIMERS
     pw_total_ = waited;
 #endif
@@ -401,17 +421,17 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
     const float scale_log2 = a.sm_scale * kLog2e;
     const V4Args v4{nullptr, nullptr, nullptr, 0};
     const dim3 grid((total + kPairsPerBlock - 1) / kPairsPerBlock), block(kPairsPerBlock * 2 * kWave);
-#define PQ_LAUNCH_PAIR_K(KERNEL, REPP, PK6)                                                                          \
+#define PQ_LAUNCH_PAIR_K(KERNEL, REPP, PK6, ...)                                                                     \
     hipLaunchKernelGGL((KERNEL<T, TB, REPP, PK6>), grid, block, 0, st, (const uint16_t*)a.q, a.codes,                \
                        (const uint16_t*)a.rscale, (const uint16_t*)a.rmn, (const uint16_t*)a.tscale,                 \
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
-                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0, ##__VA_ARGS__)
 #define PQ_LAUNCH_PAIR_P(REPP, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_PAIR_K(attn_pair_balanced_kernel, REPP, PK6);                                      \
-        else PQ_LAUNCH_PAIR_K(attn_pair_kernel, REPP, PK6);                                                          \
+        else PQ_LAUNCH_PAIR_K(attn_pair_kernel, REPP, PK6, static_cast<uint16_t*>(a.out));                           \
     } while (0)
     // packed 6-bit code rows exist for tbits == 3 only (the 3/3 configuration)
 #define PQ_LAUNCH_PAIR(REPP)                                                                                         \

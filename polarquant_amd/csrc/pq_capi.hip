@@ -199,17 +199,20 @@ int pq_validate_decode_attn(const void* q,
     return PQ_OK;
 }
 
-int pq_decode_attn_partials(const void* q,
-                            const uint8_t* codes, const void* rscale, const void* rmn,
-                            const void* tscale, const void* tmn, int group_capacity,
-                            int n_groups, const int32_t* n_groups_per_seq,
-                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
-                            const void* v, int64_t v_capacity,
-                            const uint8_t* mask, int64_t mask_stride,
-                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                            unsigned flags, void* stream) {
-    // `out` is not touched by this half: validate with a stand-in non-null, aligned pointer
+namespace {
+// The attention launch of pq_decode_attn_partials.  direct_out != nullptr (one slice per plane, default kernels): the
+// kernel writes the finished output there and no partial, so that no merge has to follow.
+int run_attn_partials(const void* q,
+                      const uint8_t* codes, const void* rscale, const void* rmn,
+                      const void* tscale, const void* tmn, int group_capacity,
+                      int n_groups, const int32_t* n_groups_per_seq,
+                      const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                      const void* v, int64_t v_capacity,
+                      const uint8_t* mask, int64_t mask_stride,
+                      float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                      int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
+                      unsigned flags, void* stream, void* direct_out) {
+    // `out` is not touched by the partials: validate with a stand-in non-null, aligned pointer
     if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                          mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
@@ -226,9 +229,26 @@ int pq_decode_attn_partials(const void* q,
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
     a.silent_scorer = (flags & PQ_TEST_SILENT_SCORER) != 0;
-    a.workspace = static_cast<float*>(workspace); a.out = nullptr;
+    a.workspace = static_cast<float*>(workspace); a.out = direct_out;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
+}
+}  // namespace
+
+int pq_decode_attn_partials(const void* q,
+                            const uint8_t* codes, const void* rscale, const void* rmn,
+                            const void* tscale, const void* tmn, int group_capacity,
+                            int n_groups, const int32_t* n_groups_per_seq,
+                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                            const void* v, int64_t v_capacity,
+                            const uint8_t* mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
+                            unsigned flags, void* stream) {
+    return run_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq, k_resid,
+                             resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask, mask_stride, sm_scale, B, N, Nk,
+                             rbits, tbits, dtype, n_splits, min_groups_per_split, workspace, workspace_bytes, flags, stream,
+                             nullptr);
 }
 
 int pq_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
@@ -255,11 +275,16 @@ int pq_decode_attn(const void* q,
                    int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
                    void* out, unsigned flags, void* stream) {
     if (!out) return PQ_ERR_NULL_POINTER;
-    if (int rc = pq_decode_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
-                                         k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
-                                         mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
-                                         workspace, workspace_bytes, flags, stream))
+    if (!aligned(out, 2)) return PQ_ERR_MISALIGNED;
+    // one slice per plane (a batch large enough to fill the device by itself): the default kernels write the output
+    // themselves and the merge launch is saved
+    const bool direct = n_splits == 1 && !(flags & (PQ_SINGLE_WAVEFRONT | PQ_BALANCED_SLICES)) && aligned(out, 16);
+    if (int rc = run_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+                                   k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
+                                   mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
+                                   workspace, workspace_bytes, flags, stream, direct ? out : nullptr))
         return rc;
+    if (direct) return PQ_OK;
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
 }
 

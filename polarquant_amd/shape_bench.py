@@ -26,6 +26,8 @@ SHAPES = [
     (16, 64, 8, 32768, 4, 4, torch.float16),       # 8 heads per KV head, 16 angle bins: the largest table
     (8, 32, 8, 4096, 4, 4, torch.float16),         # short contexts
     (64, 32, 8, 2048, 4, 4, torch.float16),
+    (128, 32, 8, 2048, 4, 4, torch.float16),       # one slice per plane: the default kernels write the output, no merge
+    (256, 32, 8, 1024, 4, 4, torch.float16),
 ]
 
 

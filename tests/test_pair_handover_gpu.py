@@ -37,7 +37,7 @@ def _call(dev, B, N, Nk, n_groups, n_resid, n_splits, gpu, flags, counts=None):
     ws = torch.zeros((nbytes // 4,), dtype=torch.float32, device=gpu)
     gp, rp = (None, None) if counts is None else (counts[0].data_ptr(), counts[1].data_ptr())
     rc = lib.pq_decode_attn(q.data_ptr(), codes.data_ptr(), rs.data_ptr(), rm.data_ptr(), ts.data_ptr(), tm.data_ptr(),
-                            n_groups, n_groups, gp, kres.data_ptr(), kres.shape[2], n_resid, rp, v.data_ptr(), v.shape[2],
+                            max(n_groups, 1), n_groups, gp, kres.data_ptr(), kres.shape[2], n_resid, rp, v.data_ptr(), v.shape[2],
                             None, 0, 1.0 / math.sqrt(128), B, N, Nk, 4, 4, _ffi.PQ_F16, n_splits, 0, ws.data_ptr(), nbytes,
                             out.data_ptr(), flags, _stream_ptr(gpu))
     assert rc == 0, _ffi.STATUS_NAMES.get(rc, rc)
@@ -69,3 +69,45 @@ def test_the_hook_is_refused_where_it_means_nothing(gpu):
     # the score op has no hand-over
     P = 4096
     assert _ffi.lib().pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, _ffi.PQ_TEST_SILENT_SCORER) == -2
+
+
+@pytest.mark.parametrize("N,Nk,n_groups,n_resid", [(32, 8, 6, 37), (28, 4, 3, 0), (8, 8, 0, 5), (16, 8, 2, 128)])
+def test_one_slice_per_plane_writes_the_output_without_a_merge(gpu, N, Nk, n_groups, n_resid):
+    """With n_splits == 1 the default kernels of pq_decode_attn write the finished output themselves.  It must be, bit
+    for bit, what the two-step form (pq_decode_attn_partials, then pq_decode_attn_merge) makes of the same call."""
+    B = 3
+    dev, ref64 = _inputs(gpu, B, N, Nk, max(n_groups, 1), n_resid, 31)
+    q, codes, rs, rm, ts, tm, kres, v = dev
+    if n_groups == 0:                                   # no quantized groups: only the residual window
+        v = v[:, :, 128:].contiguous()
+        g = torch.Generator().manual_seed(32)
+        kres_cpu, v_cpu = kres.cpu(), v.cpu()
+        ref64 = po.decode_attention_exact(q.cpu().reshape(B, N, 1, 128), kres_cpu, None, None, None, None, None, v_cpu, None, 4, 4)
+        dev = [q, codes, rs, rm, ts, tm, kres, v]
+    if n_resid == 0:
+        dev[6] = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=gpu)
+    direct = _call(dev, B=B, N=N, Nk=Nk, n_groups=n_groups, n_resid=n_resid, n_splits=1, gpu=gpu, flags=0)
+    # the same call in two steps
+    q, codes, rs, rm, ts, tm, kres, v = dev
+    lib = _ffi.lib()
+    nbytes = lib.pq_decode_attn_workspace_bytes(B, N, 1)
+    ws = torch.zeros((nbytes // 4,), dtype=torch.float32, device=gpu)
+    out = torch.zeros((B, N, 128), dtype=torch.float16, device=gpu)
+    rc = lib.pq_decode_attn_partials(q.data_ptr(), codes.data_ptr(), rs.data_ptr(), rm.data_ptr(), ts.data_ptr(), tm.data_ptr(),
+                                     max(n_groups, 1), n_groups, None, kres.data_ptr(), kres.shape[2], n_resid, None, v.data_ptr(),
+                                     v.shape[2], None, 0, 1.0 / math.sqrt(128), B, N, Nk, 4, 4, _ffi.PQ_F16, 1, 0, ws.data_ptr(),
+                                     nbytes, 0, _stream_ptr(gpu))
+    assert rc == 0
+    rc = lib.pq_decode_attn_merge(ws.data_ptr(), nbytes, B, N, 1, _ffi.PQ_F16, out.data_ptr(), _stream_ptr(gpu))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(direct.view(torch.int16), out.cpu().view(torch.int16))
+    err = (direct.double().reshape(ref64.shape) - ref64).abs()
+    assert bool((err <= 1e-3 + 1e-2 * ref64.abs()).all()), float(err.max())
+
+
+def test_a_silent_scorer_poisons_the_directly_written_output_too(gpu):
+    shape = dict(B=2, N=32, Nk=8, n_groups=3, n_resid=9, n_splits=1)
+    dev, _ = _inputs(gpu, 2, 32, 8, 3, 9, 33)
+    bad = _call(dev, gpu=gpu, flags=_ffi.PQ_TEST_SILENT_SCORER, **shape)
+    assert bool(torch.isnan(bad.float()).all())
