@@ -111,3 +111,35 @@ def test_a_silent_scorer_poisons_the_directly_written_output_too(gpu):
     dev, _ = _inputs(gpu, 2, 32, 8, 3, 9, 33)
     bad = _call(dev, gpu=gpu, flags=_ffi.PQ_TEST_SILENT_SCORER, **shape)
     assert bool(torch.isnan(bad.float()).all())
+
+
+def test_directly_written_output_under_a_replayed_graph(gpu):
+    """One slice per plane inside a captured HIP graph: replays, with the inputs changed in place between them, must give
+    what the eager call gives for the same inputs."""
+    from polarquant_amd.attention import new_workspace, polar_decode_attention
+    B, N, Nk, ng, nr = 2, 32, 8, 3, 9
+    dev, _ = _inputs(gpu, B, N, Nk, ng, nr, 41)
+    q, codes, rs, rm, ts, tm, kres, v = dev
+    q = q.reshape(B, N, 1, 128).contiguous()
+    ws = new_workspace(B, N, 1, gpu)
+    out = torch.zeros(B, N, 1, 128, dtype=torch.float16, device=gpu)
+    call = lambda o: polar_decode_attention(q, codes, rs, rm, ts, tm, kres, v, ng, nr, n_splits=1, out=o, workspace=ws)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(out)                                            # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(out)
+    g = torch.Generator(device=gpu).manual_seed(42)
+    for i in range(3):
+        q.copy_(torch.randn(q.shape, generator=g, device=gpu).half())
+        v.mul_(0.5 + i)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.zeros_like(out)
+        call(eager)
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), i
