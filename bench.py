@@ -228,20 +228,43 @@ def other_configs(dev, steps):
     HBM), each with its algorithmic bytes, fraction of the 8 TB/s peak, and a check of the timed calls' own
     results against the CPU oracle on a sampled plane."""
     from oracle import polar_oracle as po            # the checker, after the timing
-    from polarquant_amd import config_bench as cb
+    from polarquant_amd.benchmarks import config_bench as cb
     out = {}
 
     res, w = cb.measure(0, dev, steps=steps)
     sh = w["shape"]
     quant = [w["codes"].cpu()] + [m.cpu() for m in w["meta"]]
-    ref = po.decode_scores(w["q"].cpu(), *quant, sh.rbits, sh.tbits, dtype=torch.float64)
-    rel = ((w["scores"].cpu().double() - ref).abs() / ref.abs().amax(-1, keepdim=True)).max()
+    qc = w["q"].cpu()
+    ref = po.decode_scores(qc, *quant, sh.rbits, sh.tbits, dtype=torch.float64)
+    got = w["scores"].cpu().double()
+    adiff = (got - ref).abs()
+    rel = (adiff / ref.abs().amax(-1, keepdim=True)).max()
+    # element by element: scores that are off by more than 1e-3 of THEIR OWN magnitude (only scores near zero, where the
+    # terms of the sum cancel, can be), how large the largest of them is, and the absolute error there
+    off = adiff > 1e-3 * ref.abs()
+    elementwise = {"scores": ref.numel(), "off_by_more_than_1e-3_of_own_magnitude": int(off.sum()),
+                   "largest_abs_score_among_them": float(ref.abs()[off].max()) if bool(off.any()) else 0.0,
+                   "largest_abs_err_among_them": float(adiff[off].max()) if bool(off.any()) else 0.0,
+                   "row_max_abs_score_median": float(ref.abs().amax(-1).median()),
+                   "max_abs_err": float(adiff.max())}
     fl = _flips(quant, po.quantize_and_pack_nbit(w["keys"].cpu(), sh.rbits, sh.tbits))
+    # the reference's CPU-runnable case on the host cores: dequantize-then-matmul scores in fp32
+    # (models/kernel4group.py:151-155 restated by the oracle), median of 5 runs
+    po.decode_scores(qc, *quant, sh.rbits, sh.tbits)
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        po.decode_scores(qc, *quant, sh.rbits, sh.tbits)
+        times.append(time.perf_counter() - t0)
+    cpu0 = {"value": round(sorted(times)[2] * 1e6, 1), "unit": "us/call", "cores": torch.get_num_threads(), "cpu": cpu_model(),
+            "kind": "port", "sample": "the whole configuration (1 x 32 heads x 4096 tokens), median of 5 runs: the torch-CPU "
+                                      "restatement of the reference's dequantize-then-matmul score path"}
     out["cfg0_scores"] = dict(res[0], workload="configs[0]: score op, batch 1, 32 heads (MHA), context 4096, 4/4 bits",
-                              roofline=_roof(res[0]),
+                              roofline=_roof(res[0]), cpu_baseline=cpu0,
                               parity={"scores_max_err_rel_to_row_max_vs_fp64_oracle": float(rel), "within_1e-3": bool(rel < 1e-3),
+                                      "elementwise_vs_fp64_oracle": elementwise,
                                       "quantizer_vs_cpu_oracle": fl, "sample": "all 32 heads x 4096 tokens"})
-    del w, quant, ref
+    del w, quant, ref, got, adiff, off
     torch.cuda.empty_cache()
 
     res, w = cb.measure(2, dev, steps=steps)
@@ -258,7 +281,7 @@ def other_configs(dev, steps):
     del w, quant, ref
     torch.cuda.empty_cache()
 
-    res, w = cb.measure(3, dev, steps=steps)
+    res, w = cb.measure(3, dev, steps=steps, eager_gpu_append=True)
     sh = w["shape"]
     quant = [w["codes"][:, :1].cpu()] + [m[:, :1].cpu() for m in w["meta"]]
     rep = sh.n_heads // sh.n_kv_heads
@@ -271,16 +294,33 @@ def other_configs(dev, steps):
     out["cfg3_append"] = dict(res[1], workload="configs[3]: prompt quantization of 131072 fp16 post-RoPE keys x 8 KV heads (read keys, write codes and metadata)",
                               roofline=_roof(res[1]),
                               parity=dict(fl, sample="KV head 0, all 131072 keys, vs the CPU oracle's quantizer"))
+    # the same append in PQ_EAGER_GPU mode, against the reference's lines evaluated by eager torch ON THE DEVICE (all 8 KV
+    # heads, one at a time to bound the temporaries); and the default mode's distance from that evaluation, for the record
+    from oracle.device_eager import quantize_and_pack_nbit_eager
+    fe = {"codes": 0, "flips": 0, "metadata_words": 0, "metadata_words_differing": 0}
+    fd = dict(fe)
+    for h in range(sh.n_kv_heads):
+        dref = [t.cpu() for t in quantize_and_pack_nbit_eager(w["keys"][:, h:h + 1].contiguous(), sh.rbits, sh.tbits)]
+        for acc, src in ((fe, w["append_out_eager_gpu"]), (fd, w["append_out"])):
+            one = _flips([t[:, h:h + 1].cpu() for t in src], dref)
+            for key in acc:
+                acc[key] += one[key]
+    out["cfg3_append_eager_gpu"] = dict(res[2], workload="configs[3]'s prompt quantization in PQ_EAGER_GPU mode (fp32 wrap, the device "
+                                                         "library's atan2f): codes as the reference's lines give them when they run on GPU tensors",
+                                        roofline=_roof(res[2]),
+                                        parity=dict(fe, sample="all 8 KV heads x 131072 keys, vs the reference's lines as eager torch ops on device tensors",
+                                                    default_mode_vs_the_same=fd))
     del w, quant, ref, got
     torch.cuda.empty_cache()
 
     # configs[4]: the end-to-end greedy decode loop (random-init Llama-3-8B architecture, bf16, all 32 layers, batch 8,
     # prompt 16384, 256 new tokens), the step replayed from a HIP graph; a 2-layer run of the same loop splits the step
-    # into its per-layer part and the embedding / lm_head part.  Its parity is the test suite's (every step of toy
-    # models replayed through the oracle); nothing is checked here.
+    # into its per-layer part and the embedding / lm_head part.  Sanity of the timed run itself: its first 8 greedy steps
+    # against the eager model.  Beside it the un-quantized model (same shells and graph, bf16 K and V caches), as the
+    # reference's throughput script has it (benchmark/benchmark_throughput.py:93-113).
     try:
-        from polarquant_amd import e2e_bench
-        r32 = e2e_bench.run(batch=8, prompt=16384, new=256, layers=32, graph=True)
+        from polarquant_amd.benchmarks import e2e_bench
+        r32 = e2e_bench.run(batch=8, prompt=16384, new=256, layers=32, graph=True, check_tokens=8)
         torch.cuda.empty_cache()
         r2 = e2e_bench.run(batch=8, prompt=16384, new=66, layers=2, graph=True)
         per_layer = (r32["decode_ms_per_step"] - r2["decode_ms_per_step"]) / 30
@@ -293,7 +333,18 @@ def other_configs(dev, steps):
             "kv_cache_bytes_per_token": r32["kv_cache_bytes_per_token"],
             "fp16_kv_cache_bytes_per_token": r32["fp16_kv_cache_bytes_per_token"],
             "peak_memory_GiB": r32["peak_memory_GiB"],
+            "sanity": r32.get("sanity"),
         }
+        for mode in ("same_kernel", "sdpa_splitk"):
+            torch.cuda.empty_cache()
+            try:
+                rb = e2e_bench.run(batch=8, prompt=16384, new=256, layers=32, fp16_kv=mode)
+                out["cfg4_e2e"]["fp16_kv_" + mode] = {
+                    "workload": rb["workload"], "decode_ms_per_step": rb["decode_ms_per_step"],
+                    "decode_tokens_per_s": rb["decode_tokens_per_s"], "peak_memory_GiB": rb["peak_memory_GiB"],
+                    "polar_speedup": round(rb["decode_ms_per_step"] / r32["decode_ms_per_step"], 3)}
+            except Exception as e:              # noqa: BLE001 - report, do not fail the bench
+                out["cfg4_e2e"]["fp16_kv_" + mode] = {"error": str(e)[:300]}
     except Exception as e:                      # noqa: BLE001 - report, do not fail the bench
         out["cfg4_e2e"] = {"error": str(e)[:300]}
     torch.cuda.empty_cache()
@@ -357,7 +408,7 @@ def main():
                 n_splits, 0, ws.data_ptr(), ws.numel() * 4, 0] for x in sets]
 
     def partials_only():
-        rc = lib.pq_decode_attn_partials(*commons[turn[0] & 1], _stream_ptr(dev))
+        rc = lib.pq_decode_attn_partials(*commons[turn[0] & 1], None, _stream_ptr(dev))
         turn[0] += 1
         assert rc == 0, rc
 

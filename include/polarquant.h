@@ -96,9 +96,17 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
  * No reference counterpart. */
 #define PQ_SINGLE_WAVEFRONT 32u
 
-/* test hook of the same entry points (default kernels only): the scorers publish nothing, and the bounded waits of
- * the hand-over give up after 1000 polls instead of 2^22.  Every kernel still ends normally; every output of the
- * call is NaN.  For the test that a hand-over which fails can neither hang the GPU nor pass for a result. */
+/* What the optional `status` word of the attention entry points can hold after the call's kernels have run. */
+#define PQ_STATUS_HANDOVER_TIMEOUT 1 /* a scorer / accumulator hand-over gave up waiting; the output rows of every plane
+                                        the failing pair worked on are NaN */
+
+/* Test hook of pq_decode_attn / _partials / _static (scorer / accumulator kernels only; refused together with
+ * PQ_SINGLE_WAVEFRONT and by the 4-bit-value entry point, whose kernels have no hand-over): the scorers publish nothing,
+ * and the bounded waits of the hand-over give up after 1000 polls instead of 2^22.  Every kernel still ends normally;
+ * every output of the call is NaN and the status word is set.  For the test that a hand-over which fails can neither
+ * hang the GPU nor pass for a result.  ONLY the test build of the library (compiled with -DPQ_TEST_HOOKS:
+ * libpolarquant_hip_testhooks.so, which the package never loads) honours it; the shipping library refuses the flag with
+ * PQ_ERR_BAD_SHAPE like any unknown flag, and its kernels contain no such switch. */
 #define PQ_TEST_SILENT_SCORER 0x40000000u
 
 /* Linear layer of a decode step: y[M, N] = x[M, K] . w[N, K]^T (+ bias[N]), M <= 16 rows (one new
@@ -250,6 +258,12 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48) and / or
  *            PQ_BALANCED_SLICES (slices cut on the device from the per-sequence counts, see above) and / or
  *            PQ_SINGLE_WAVEFRONT (one wavefront per slice instead of a scorer / accumulator pair)
+ *   status   NULL, or one device int32 that the CALLER has set to 0 (the library never clears it): the kernels with a
+ *            scorer / accumulator pair per slice store PQ_STATUS_HANDOVER_TIMEOUT there when a hand-over between the
+ *            two wavefronts gives up (2^22 polls, about half a second, without an answer: a wavefront that never got
+ *            to run, which no correct execution produces).  The affected output rows are NaN as well; the word lets a
+ *            host learn of it, after synchronizing with the stream, without scanning the output.  It stays untouched
+ *            by the one-wavefront kernels, which have no hand-over.
  * Limits: v_capacity <= PQ_MAX_PLANE_TOKENS tokens and group_capacity <= 2^17 groups per (batch, KV head)
  * plane (32-bit byte sizes and offsets inside a plane), B*Nk <= 65535, N/Nk <= 8.
  * ------------------------------------------------------------------------- */
@@ -262,7 +276,7 @@ int pq_decode_attn(const void *q,
                    const uint8_t *mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                    int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
-                   void *out, unsigned flags, void *stream);
+                   void *out, unsigned flags, int32_t *status, void *stream);
 
 int pq_validate_decode_attn(const void *q,
                             const uint8_t *codes, const void *rscale, const void *rmn,
@@ -291,7 +305,7 @@ int pq_decode_attn_partials(const void *q,
                             const uint8_t *mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                             int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
-                            unsigned flags, void *stream);
+                            unsigned flags, int32_t *status, void *stream);
 
 int pq_decode_attn_merge(const void *workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
                          void *out, void *stream);
@@ -314,7 +328,8 @@ int pq_decode_attn_static(const void *q,
                           const void *v, int64_t v_capacity,
                           const uint8_t *mask, int64_t mask_stride,
                           float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                          int n_splits, int min_groups_per_split, void *out, unsigned flags, void *stream);
+                          int n_splits, int min_groups_per_split, void *out, unsigned flags, int32_t *status,
+                          void *stream);
 
 /* ---------------------------------------------------------------------------
  * 4-bit values: the reference's Mixed variant (LlamaPolarMixedGroupAttention,

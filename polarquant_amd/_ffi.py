@@ -20,7 +20,8 @@ PQ_CODES_PACKED6 = 4
 PQ_DEVICE_ATAN2 = 8
 PQ_BALANCED_SLICES = 16
 PQ_SINGLE_WAVEFRONT = 32
-PQ_TEST_SILENT_SCORER = 0x40000000
+PQ_TEST_SILENT_SCORER = 0x40000000      # honoured by the test build of the library only; the one loaded here refuses it
+PQ_STATUS_HANDOVER_TIMEOUT = 1
 PQ_EAGER_GPU = PQ_WRAP_FP32 | PQ_DEVICE_ATAN2
 
 STATUS_NAMES = {
@@ -42,16 +43,16 @@ SIGNATURES = {
     "pq_selftest_quantizer_math": (c_int, [c_int, c_void_p, c_void_p]),
     "pq_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                 c_void_p, c_int64, c_void_p, c_int64, c_float]
-                       + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p]),
+                       + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p, c_void_p]),
     "pq_decode_attn_static": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                        c_void_p, c_int64, c_void_p, c_int64, c_float]
-                              + [c_int] * 8 + [c_void_p, c_uint, c_void_p]),
+                              + [c_int] * 8 + [c_void_p, c_uint, c_void_p, c_void_p]),
     "pq_validate_decode_attn": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
                                 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint]),
     "pq_decode_attn_partials": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                          c_void_p, c_int64, c_void_p, c_int64, c_float]
-                                + [c_int] * 8 + [c_void_p, c_size_t, c_uint, c_void_p]),
+                                + [c_int] * 8 + [c_void_p, c_size_t, c_uint, c_void_p, c_void_p]),
     "pq_decode_attn_merge": (c_int, [c_void_p, c_size_t, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "pq_quantize_values": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_int64, c_void_p]),

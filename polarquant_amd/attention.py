@@ -86,6 +86,7 @@ def polar_decode_attention(
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
     total_groups: Optional[int] = None, min_groups_per_split: Optional[int] = None,
     workspace: Optional[torch.Tensor] = None, balanced: Optional[bool] = None, single_wavefront: bool = False,
+    status: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """-> attention output [B,N,1,128] in the query dtype.
 
@@ -99,7 +100,11 @@ def polar_decode_attention(
     `workspace`: a buffer from `new_workspace` that the caller owns (needed under graph capture);
     by default the cached buffer of the current stream is used.
     `single_wavefront`: the earlier kernels, in which one wavefront does all the work of a slice
-    (PQ_SINGLE_WAVEFRONT), instead of the scorer / accumulator pairs; for comparison."""
+    (PQ_SINGLE_WAVEFRONT), instead of the scorer / accumulator pairs; for comparison.
+    `status`: an int32 tensor of one element on the same device that the caller has zeroed.  The default
+    kernels set it to PQ_STATUS_HANDOVER_TIMEOUT (1) if a hand-over between a scorer and its accumulator
+    gives up (the affected output rows are NaN too); nothing here reads it back, so no synchronisation
+    is added: `int(status)` after the call is the caller's."""
     if not query_states.is_cuda:
         raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
     dev = query_states.device
@@ -158,11 +163,16 @@ def polar_decode_attention(
         out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
     gps = n_groups_per_seq.data_ptr() if n_groups_per_seq is not None else None
     rps = n_resid_per_seq.data_ptr() if n_resid_per_seq is not None else None
+    sptr = None
+    if status is not None:
+        if status.dtype != torch.int32 or status.device != dev or status.numel() != 1:
+            raise ValueError("polarquant_amd: status must be one int32 on %s" % dev)
+        sptr = status.data_ptr()
     with torch.cuda.device(dev):
         rc = _ffi.lib().pq_decode_attn(
             q.data_ptr(), *cptr, g_cap, n_groups, gps, kptr, r_cap, n_resid, rps,
             value_states.data_ptr(), v_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
-            n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, _stream_ptr(dev))
+            n_splits, min_gps, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, sptr, _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn")
     return out
 

@@ -5,7 +5,7 @@
   configs[2]  ragged continuous-batch decode attention, Qwen2.5-7B shape (batch 64, GQA 7, 3/3 bits)
   configs[3]  prompt quantization (append) of 131072 keys x 8 KV heads, then one decode step over them
 
-    python -m polarquant_amd.config_bench [--configs 0 2 3] [--values4] [--packed]
+    python -m polarquant_amd.benchmarks.config_bench [--configs 0 2 3] [--values4] [--packed]
 
 Prints one JSON line per measurement: µs per call, algorithmic bytes, GB/s and fraction of the
 8 TB/s HBM peak.  --values4 adds the decode step with 4-bit values (Mixed variant) for the
@@ -19,11 +19,11 @@ import time
 
 import torch
 
-from . import workloads as wl
-from .attention import polar_decode_attention, polar_decode_attention_v4
-from .kernel4group import attention_decode_forward_triton_impl
-from .quantize import quantize_and_pack_nbit
-from .values import quantize_values
+from .. import workloads as wl
+from ..attention import polar_decode_attention, polar_decode_attention_v4
+from ..kernel4group import attention_decode_forward_triton_impl
+from ..quantize import quantize_and_pack_nbit
+from ..values import quantize_values
 
 HBM_PEAK_GBPS = 8000.0
 
@@ -34,11 +34,18 @@ def _entry(op, ms, nbytes, **extra):
                 frac_of_hbm_peak=round(gbps / HBM_PEAK_GBPS, 4), **extra)
 
 
-def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool = False, single_wavefront: bool = False):
+def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool = False, single_wavefront: bool = False,
+            n_sets: int = 2, eager_gpu_append: bool = False):
     """Time configs[idx] -> (list of measurement dicts, the workload).  The workload keeps what a caller
     needs to check the timed calls' results against a CPU checker: w["scores"] (configs[0]), w["out"] (decode
     attention output), w["append_out"] (configs[3]: codes and metadata the timed quantizer calls wrote) and
-    w["keys"] (configs[0] and configs[3])."""
+    w["keys"] (configs[0] and configs[3]); all of them belong to input set 0.
+    n_sets: independent input sets the timed calls rotate over (configs[2] and [3]; configs[0] always uses 8):
+    one set of these configurations is 340-390 MB, not much more than the 256 MB Infinity Cache, so a loop over a
+    single set could be served partly from that cache.
+    eager_gpu_append (configs[3]): the prompt quantization is timed a second time in PQ_EAGER_GPU mode, the
+    arithmetic eager torch applies to the reference's lines on device tensors; its output is kept in
+    w["append_out_eager_gpu"]."""
     w = wl.build_workload(idx, dev, keep_keys=(idx in (0, 3)), packed=packed)
     sh = w["shape"]
     B, N, Nk = sh.batch, sh.n_heads, sh.n_kv_heads
@@ -67,6 +74,14 @@ def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool
                           input_sets_rotated=8))
         w["scores"] = attention_decode_forward_triton_impl(w["q"], w["codes"], *w["meta"], rbits=sh.rbits, tbits=sh.tbits)
         return res, w
+    n_sets = max(1, n_sets)
+    sets = [w] + [wl.build_workload(idx, dev, keep_keys=(idx == 3), packed=packed, variant=i) for i in range(1, n_sets)]
+    turn = [0]
+
+    def next_set():
+        x = sets[turn[0] % n_sets]
+        turn[0] += 1
+        return x
     if sh.ragged:
         lens = w["lengths"]
         lq, rs = ((lens // 128) * 128).tolist(), (lens % 128).tolist()
@@ -75,33 +90,62 @@ def measure(idx: int, dev, values4: bool = False, steps: int = 100, packed: bool
         lq, rs, total_groups = [w["n_groups"] * 128] * B, [w["n_resid"]] * B, None
     nbytes = wl.algorithmic_bytes(Nk, N, lq, rs, sh.rbits, sh.tbits, code_bytes_per_pair=0.75 if packed else 1.0)
     out = torch.empty(B, N, 1, 128, dtype=w["q"].dtype, device=dev)
-    ms = wl.time_events(lambda: polar_decode_attention(
-        w["q"], w["codes"], *w["meta"], w["kres"], w["v"], w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
-        n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=total_groups, out=out,
-        single_wavefront=single_wavefront), steps, 10)
+
+    def attend(x=None, o=out):
+        x = x or next_set()
+        polar_decode_attention(
+            x["q"], x["codes"], *x["meta"], x["kres"], x["v"], x["n_groups"], x["n_resid"], rbits=sh.rbits, tbits=sh.tbits,
+            n_groups_per_seq=x["groups_per_seq"], n_resid_per_seq=x["resid_per_seq"], total_groups=total_groups, out=o,
+            single_wavefront=single_wavefront)
+    ms = wl.time_events(attend, steps, 10)
     res.append(_entry("decode attention (pq_decode_attn)" + (", packed 6-bit codes" if packed else "")
                       + (", one wavefront per slice" if single_wavefront else ""), ms, nbytes,
-                      tokens=int(sum(lq) + sum(rs))))
+                      tokens=int(sum(lq) + sum(rs)), input_sets_rotated=n_sets))
+    attend(w)                                   # leave set 0's result in `out` for the caller's check
     w["out"] = out
     if values4 and not sh.ragged:
         L = w["n_groups"] * 128
-        vq = quantize_values(w["v"][:, :, :L])
-        vres = torch.zeros(B, Nk, 128, 128, dtype=w["v"].dtype, device=dev)
-        vres[:, :, :w["n_resid"]] = w["v"][:, :, L:L + w["n_resid"]]
-        ms4 = wl.time_events(lambda: polar_decode_attention_v4(
-            w["q"], w["codes"], *w["meta"], w["kres"], vres, *vq, w["n_groups"], w["n_resid"], rbits=sh.rbits, tbits=sh.tbits), steps, 10)
+        v4 = []
+        for x in sets:
+            vq = quantize_values(x["v"][:, :, :L])
+            vres = torch.zeros(B, Nk, 128, 128, dtype=x["v"].dtype, device=dev)
+            vres[:, :, :x["n_resid"]] = x["v"][:, :, L:L + x["n_resid"]]
+            v4.append((x, vq, vres))
+
+        def attend4():
+            x, vq, vres = v4[turn[0] % n_sets]
+            turn[0] += 1
+            polar_decode_attention_v4(x["q"], x["codes"], *x["meta"], x["kres"], vres, *vq, x["n_groups"], x["n_resid"],
+                                      rbits=sh.rbits, tbits=sh.tbits)
+        ms4 = wl.time_events(attend4, steps, 10)
         res.append(_entry("decode attention, 4-bit values (pq_decode_attn_v4)", ms4,
-                          wl.algorithmic_bytes(Nk, N, lq, rs, sh.rbits, sh.tbits, value_bits=4)))
-        msq = wl.time_events(lambda: quantize_values(w["v"][:, :, :L], out=vq), max(steps // 2, 5), 3)
-        res.append(_entry("value quantization (pq_quantize_values)", msq, B * Nk * L * (256 + 64 + 4)))
-        del vq, vres
+                          wl.algorithmic_bytes(Nk, N, lq, rs, sh.rbits, sh.tbits, value_bits=4), input_sets_rotated=n_sets))
+
+        def quant4():
+            x, vq, _ = v4[turn[0] % n_sets]
+            turn[0] += 1
+            quantize_values(x["v"][:, :, :L], out=vq)
+        msq = wl.time_events(quant4, max(steps // 2, 5), 3)
+        res.append(_entry("value quantization (pq_quantize_values)", msq, B * Nk * L * (256 + 64 + 4), input_sets_rotated=n_sets))
+        del v4
     if idx == 3:
+        aouts = [(torch.empty_like(x["codes"]), *[torch.empty_like(m) for m in x["meta"]]) for x in sets]
+
+        def append(eager_gpu=False):
+            i = turn[0] % n_sets
+            turn[0] += 1
+            quantize_and_pack_nbit(sets[i]["keys"], sh.rbits, sh.tbits, out=aouts[i], eager_gpu=eager_gpu)
         k = w["keys"]
-        aout = (torch.empty_like(w["codes"]), *[torch.empty_like(m) for m in w["meta"]])
-        ms = wl.time_events(lambda: quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=aout), max(steps // 2, 5), 5)
-        res.append(_entry("append / prompt quantization (pq_quantize_groups)", ms,
-                          k.numel() * 2 + aout[0].numel() + 4 * aout[1].numel() * 2))
-        w["append_out"] = aout
+        append_bytes = k.numel() * 2 + aouts[0][0].numel() + 4 * aouts[0][1].numel() * 2
+        ms = wl.time_events(append, max(steps // 2, 6), 6)
+        res.append(_entry("append / prompt quantization (pq_quantize_groups)", ms, append_bytes, input_sets_rotated=n_sets))
+        if eager_gpu_append:
+            ms = wl.time_events(lambda: append(True), max(steps // 2, 6), 6)
+            res.append(_entry("append / prompt quantization, PQ_EAGER_GPU (the reference's lines as eager torch evaluates them on "
+                              "device tensors)", ms, append_bytes, input_sets_rotated=n_sets))
+            w["append_out_eager_gpu"] = quantize_and_pack_nbit(k, sh.rbits, sh.tbits, eager_gpu=True)
+        quantize_and_pack_nbit(k, sh.rbits, sh.tbits, out=aouts[0])       # set 0, default mode, for the caller's check
+        w["append_out"] = aouts[0]
     return res, w
 
 

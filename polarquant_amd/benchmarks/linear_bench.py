@@ -3,7 +3,7 @@
 distinct weight matrices (more than the 256 MB of last-level cache in total), the way the decode step
 meets them: every layer has its own weights and nothing is re-read between layers.
 
-    python -m polarquant_amd.linear_bench [--rows 8]
+    python -m polarquant_amd.benchmarks.linear_bench [--rows 8]
 """
 from __future__ import annotations
 
@@ -13,7 +13,7 @@ import json
 import torch
 import torch.nn.functional as F
 
-from .decode_ops import linear_small_m
+from ..decode_ops import linear_small_m
 
 SHAPES = (("q|k|v", 6144, 4096, False), ("o_proj", 4096, 4096, False), ("gate, up, silu*up", 14336, 4096, True),
           ("down_proj", 4096, 14336, False))

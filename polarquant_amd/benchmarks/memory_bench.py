@@ -3,7 +3,7 @@ random ids, `output_length` greedily generated tokens with the stop token made u
 allocator over prompt pass + generation, in GB (1e9 bytes), per batch size.  The model is the random-init Llama-3-8B
 architecture in fp16 (no weights can be fetched here; memory does not depend on their values).
 
-    python -m polarquant_amd.memory_bench [--batch_size 1 4 16] [--input_length 256] [--output_length 4096]
+    python -m polarquant_amd.benchmarks.memory_bench [--batch_size 1 4 16] [--input_length 256] [--output_length 4096]
                                           [--layers 32] [--values4] [--eager]
 
 One JSON line per batch size: peak memory, the part of it that is weights, and the cache's size by the per-token
@@ -19,7 +19,7 @@ import time
 import torch
 
 from .e2e_bench import build_model
-from .modeling_common import GenerationConfig, PolarConfig, generate
+from ..modeling_common import GenerationConfig, PolarConfig, generate
 
 
 def run(batch_size: int, input_length: int, output_length: int, layers: int = 32, values4: bool = False, eager: bool = False):

@@ -3,7 +3,7 @@
 heads, random codes and randn metadata, B in {1,2,4,8}, L in {4k..128k}; prints ms per call
 of the polar score op next to an fp16 torch.matmul QK^T on the same GPU.
 
-    python -m polarquant_amd.microbench [--iters 50]
+    python -m polarquant_amd.benchmarks.microbench [--iters 50]
 """
 from __future__ import annotations
 
@@ -12,7 +12,7 @@ import json
 
 import torch
 
-from .kernel4group import attention_decode_forward_triton_impl
+from ..kernel4group import attention_decode_forward_triton_impl
 
 LENGTHS = (4096, 8192, 16384, 32768, 65536, 131072)
 BATCHES = (1, 2, 4, 8)

@@ -6,7 +6,7 @@ Needs the measuring build of the library (`python -m polarquant_amd.build --phas
 kernel brackets its phases with the 100 MHz wall clock and lets every 97th wavefront print its sums.  The
 instrumentation costs a few percent, so totals are a little above the real kernel's; the split is what matters.
 
-    python -m polarquant_amd.phase_timing [--config 1] [--values4]
+    python -m polarquant_amd.benchmarks.phase_timing [--config 1] [--values4]
 
 Phases of one 128-token group: table = build of the per-group angle table in LDS; value_issue = issue of the
 next tile's value loads (16 buffer loads; the time is spent in the issue itself when the compute unit's miss
@@ -25,8 +25,8 @@ import tempfile
 
 import torch
 
-from . import _ffi
-from .build import TIMERS_LIB
+from .. import _ffi
+from ..build import TIMERS_LIB
 
 PHASES = ("table", "value_issue", "code_wait", "code_issue", "score", "softmax_pv")
 
@@ -43,9 +43,9 @@ def main():
     if not os.path.exists(TIMERS_LIB):
         sys.exit("phase_timing: build the measuring library first: python -m polarquant_amd.build --phase-timers")
     _ffi.LIB_PATH = TIMERS_LIB
-    from . import workloads as wl
-    from .attention import polar_decode_attention, polar_decode_attention_v4
-    from .values import quantize_values
+    from .. import workloads as wl
+    from ..attention import polar_decode_attention, polar_decode_attention_v4
+    from ..values import quantize_values
     dev = torch.device("cuda:0")
     w = wl.build_workload(args.config, dev)
     sh = w["shape"]

@@ -1,7 +1,7 @@
 """Fused decode attention at head layouts and sizes other than the benchmark configurations: the default kernels (a
 scorer / accumulator pair of wavefronts per slice) beside the kernels with one wavefront per slice.
 
-    python -m polarquant_amd.shape_bench
+    python -m polarquant_amd.benchmarks.shape_bench
 
 One JSON line per shape: batch, query heads, KV heads, context, bits, dtype -> us per step (attention + merge) of
 both forms and their fractions of the 8 TB/s HBM peak on algorithmic bytes.  Uniform batches, one residual key,
@@ -13,9 +13,9 @@ import json
 
 import torch
 
-from . import workloads as wl
-from .attention import polar_decode_attention
-from .quantize import quantize_and_pack_nbit
+from .. import workloads as wl
+from ..attention import polar_decode_attention
+from ..quantize import quantize_and_pack_nbit
 
 SHAPES = [
     # B, N, Nk, L, rbits, tbits, dtype

@@ -36,6 +36,10 @@ def _hipcc() -> str:
 
 
 TIMERS_LIB = os.path.join(HERE, "libpolarquant_hip_timers.so")
+# the test build: the same library with -DPQ_TEST_HOOKS, which alone honours PQ_TEST_SILENT_SCORER (a hook that turns
+# the output into NaN on purpose).  Loaded by tests/test_pair_handover_gpu.py only, never by the package.
+HOOKS_LIB = os.path.join(HERE, "libpolarquant_hip_testhooks.so")
+HOOKS_SOURCES = ["pq_capi.hip", "pq_attn_pair.hip"]          # the sources that read the define
 
 
 def _compile(src: str, defines=(), tag: str = "") -> str:
@@ -62,16 +66,24 @@ def _link(objs, lib: str) -> None:
 def build(verbose: bool = True, phase_timers: bool = False) -> str:
     """The library the package loads; or, with phase_timers, a second library (same ABI, not loaded by default)
     whose attention kernel times its phases with the wall clock and prints them: a measuring build for
-    `python -m polarquant_amd.phase_timing`, a few percent slower than the real one."""
+    `python -m polarquant_amd.benchmarks.phase_timing`, a few percent slower than the real one."""
     os.makedirs(OBJ, exist_ok=True)
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
     lib, defines, tag = (TIMERS_LIB, ("PQ_ATTN_PHASE_TIMERS",), ".timers") if phase_timers else (LIB, (), "")
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(lambda s_: _compile(s_, defines, tag), srcs))
+    jobs = [(s_, defines, tag) for s_ in srcs]
+    if not phase_timers:
+        jobs += [(s_, ("PQ_TEST_HOOKS",), ".hooks") for s_ in HOOKS_SOURCES] + [(s_, (), "") for s_ in BENCH_SOURCES]
+    # the longest compilations first, so that they do not start last
+    jobs.sort(key=lambda j: -os.path.getsize(os.path.join(CSRC, j[0])) if "attn" not in j[0] else -1 << 30)
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
+        built = dict(zip([(j[0], j[2]) for j in jobs], ex.map(lambda j: _compile(*j), jobs)))
+    objs = [built[(s_, tag)] for s_ in srcs]
     _link(objs, lib)
     if not phase_timers:
-        _link([_compile(s_) for s_ in BENCH_SOURCES], BENCH_LIB)
+        _link([built[(s_, ".hooks" if s_ in HOOKS_SOURCES else "")] for s_ in srcs], HOOKS_LIB)
+        _link([built[(s_, "")] for s_ in BENCH_SOURCES], BENCH_LIB)
         if verbose:
+            print("built", HOOKS_LIB)
             print("built", BENCH_LIB)
     if verbose:
         print("built", lib)

@@ -31,47 +31,7 @@
 #include "pq_attn_device.h"
 #include <mutex>
 
-// Measuring build only (-DPQ_ATTN_PHASE_TIMERS, `python -m polarquant_amd.build --phase-timers`): wall-clock
-// (100 MHz) time of each phase of the group loop, summed per wavefront and printed by a few of them.
-#ifdef PQ_ATTN_PHASE_TIMERS
-#define PQ_T_ENTRY const long long pt_entry_ = wall_clock64(); long long pt_loop0_ = pt_entry_, pt_first_ = 0, pt_loop1_ = pt_entry_, pt_sum_[6] = {0, 0, 0, 0, 0, 0}; int pt_groups_ = 0
-#define PQ_T_DECL long long pt_[6] = {0, 0, 0, 0, 0, 0}, pt_mark_ = 0; pt_loop0_ = wall_clock64()
-#define PQ_T_MARK() pt_mark_ = wall_clock64()
-#define PQ_T_ADD(i) do { const long long pt_now_ = wall_clock64(); pt_[i] += pt_now_ - pt_mark_; pt_mark_ = pt_now_; } while (0)
-#define PQ_T_KEEP(x) asm volatile("" ::"v"(x))
-#define PQ_T_FIRST_GROUP_DONE() do { if (pt_first_ == 0) pt_first_ = wall_clock64() - pt_loop0_; } while (0)
-#define PQ_T_REPORT(n_groups)                                                                                        \
-    do {                                                                                                             \
-        pt_loop1_ = wall_clock64();                                                                                  \
-        pt_groups_ = n_groups;                                                                                       \
-        for (int i_ = 0; i_ < 6; i_++) pt_sum_[i_] = pt_[i_];                                                        \
-    } while (0)
-// Printed once per piece, after its partial has been handed to the memory system (a device printf takes
-// milliseconds, so none may sit inside what is timed): the phase sums of the group loop, then the absolute entry
-// and exit clocks (the 100 MHz counter is common to the chip, so the spread of entries and exits over the
-// wavefronts can be read off), entry -> loop, the first group, the loop, loop -> exit.
-#define PQ_T_EXIT()                                                                                                  \
-    do {                                                                                                             \
-        const long long pt_exit_ = wall_clock64();                                                                   \
-        if (threadIdx.x == 0 && blockIdx.x % 97 == 0) {                                                              \
-            printf("pq_phase block %d groups %d total %lld table %lld value_issue %lld code_wait %lld code_issue %lld score %lld softmax_pv %lld\n", \
-                   static_cast<int>(blockIdx.x), pt_groups_, pt_loop1_ - pt_loop0_, pt_sum_[0], pt_sum_[1], pt_sum_[2], \
-                   pt_sum_[3], pt_sum_[4], pt_sum_[5]);                                                              \
-            printf("pq_piece block %d groups %d entry %lld exit %lld before_loop %lld first_group %lld loop %lld after_loop %lld\n", \
-                   static_cast<int>(blockIdx.x), pt_groups_, pt_entry_, pt_exit_, pt_loop0_ - pt_entry_, pt_first_,   \
-                   pt_loop1_ - pt_loop0_, pt_exit_ - pt_loop1_);                                                     \
-        }                                                                                                            \
-    } while (0)
-#else
-#define PQ_T_ENTRY
-#define PQ_T_DECL
-#define PQ_T_MARK()
-#define PQ_T_ADD(i)
-#define PQ_T_KEEP(x)
-#define PQ_T_FIRST_GROUP_DONE()
-#define PQ_T_REPORT(n_groups)
-#define PQ_T_EXIT()
-#endif
+#include "pq_phase_timers.h"
 
 namespace pq {
 

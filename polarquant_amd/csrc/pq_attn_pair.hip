@@ -11,11 +11,16 @@
 // pairs the wavefronts are paired as (w, w + 4): the results are the same, only the overlap is lost.
 // The two hand tiles over through two counters in LDS (tiles published / tiles consumed); a wait
 // gives up after kSpinLimit polls (about half a second), after which both wavefronts run out
-// without waiting again and the accumulator writes NaN into the piece's partial: a failed hand-over
-// cannot pass for a result, and no wavefront can wait for ever.  PQ_TEST_SILENT_SCORER makes the
+// without waiting again, the accumulator writes NaN into the partial of this piece and of every
+// later piece of its segment, and both set the caller's status word (if one was passed) with a plain
+// vector store: a failed hand-over cannot pass for a result, the host can learn of it without
+// scanning the output, and no wavefront can wait for ever.
+// Test build only (-DPQ_TEST_HOOKS, libpolarquant_hip_testhooks.so): PQ_TEST_SILENT_SCORER makes the
 // scorers publish nothing and the waits give up after 1000 polls, so that a test can see exactly
-// that: every kernel ends, every output is NaN.
+// that: every kernel ends, every output is NaN, the status word is set.  The shipping library
+// refuses the flag and its kernels hold no such switch.
 #include "pq_attn_device.h"
+#include "pq_phase_timers.h"
 
 namespace pq {
 
@@ -25,6 +30,12 @@ namespace pq {
 constexpr int kPairsPerBlock = 4;
 constexpr int kSpinLimit = 1 << 22;
 constexpr int kSpinLimitSilent = 1000;      // with PQ_TEST_SILENT_SCORER: the waits' time-out is what is being tested
+#ifdef PQ_TEST_HOOKS
+constexpr bool kTestHooks = true;
+#else
+constexpr bool kTestHooks = false;
+#endif
+constexpr int kStatusHandoverTimeout = 1;   // == PQ_STATUS_HANDOVER_TIMEOUT
 
 struct PairMem {
     uint32_t lut;      // the scorer's table
@@ -32,27 +43,34 @@ struct PairMem {
     uint32_t pbuf;     // the accumulator's probability staging
     uint32_t flags;    // int[4]: tiles published by the scorer, tiles consumed by the accumulator, -, -
     int spin_limit;    // polls after which a wait gives up
-    bool silent;       // PQ_TEST_SILENT_SCORER: the scorer publishes nothing
+    bool silent;       // PQ_TEST_SILENT_SCORER (test build only): the scorer publishes nothing
 };
 
-typedef __attribute__((address_space(3))) volatile int lds_vi;
+__device__ __forceinline__ PairMem pair_mem(uint32_t lut, uint32_t sbuf, uint32_t pbuf, uint32_t flags, int silent_scorer) {
+    PairMem pm;
+    pm.lut = lut; pm.sbuf = sbuf; pm.pbuf = pbuf; pm.flags = flags;
+    pm.silent = kTestHooks && silent_scorer != 0;
+    pm.spin_limit = pm.silent ? kSpinLimitSilent : kSpinLimit;
+    return pm;
+}
 
-// Measuring build only (-DPQ_ATTN_PHASE_TIMERS): every wavefront adds up the wall-clock time (100 MHz) it spends in
-// pair_wait, and the wavefronts of every 97th workgroup print it with their role when their kernel ends.
-#ifdef PQ_ATTN_PHASE_TIMERS
-#define PQ_PAIR_T_DECL long long pw_total_ = 0; const long long pw_entry_ = wall_clock64()
-#define PQ_PAIR_T_WAIT(call) [&]() { const long long t0_ = wall_clock64(); const bool r_ = (call); pw_total_ += wall_clock64() - t0_; return r_; }()
-#define PQ_PAIR_T_REPORT(role, tiles)                                                                                \
-    do {                                                                                                             \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x % 97 == 0)                                                         \
-            printf("pq_pair block %d wave %d role %d tiles %d life %lld waited %lld\n", static_cast<int>(blockIdx.x),  \
-                   static_cast<int>(threadIdx.x >> 6), role, tiles, wall_clock64() - pw_entry_, pw_total_);          \
-    } while (0)
-#else
-#define PQ_PAIR_T_DECL
-#define PQ_PAIR_T_WAIT(call) (call)
-#define PQ_PAIR_T_REPORT(role, tiles)
-#endif
+// A hand-over gave up: tell the host, if it passed a status word.  One lane, an ordinary vector store of a constant
+// (every wavefront that fails writes the same value, so no atomic is needed).
+__device__ __forceinline__ void report_timeout(int* status, int lane) {
+    if (status != nullptr && lane == 0) *status = kStatusHandoverTimeout;
+}
+
+// The partial of a piece whose pair has already failed: a NaN maximum for every head, which the merge turns into a NaN
+// output row whatever the body of the partial holds.
+__device__ __forceinline__ void poison_slot(const AttnParams& p, int lane, int b, int kvh, int slot) {
+    if (lane < p.rep) {
+        float* pw = p.ws + ((static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * p.rep + lane) * p.n_splits + slot) * kPartialFloats;
+        pw[0] = __builtin_nanf("");
+        pw[1] = 0.0f;
+    }
+}
+
+typedef __attribute__((address_space(3))) volatile int lds_vi;
 
 __device__ __forceinline__ bool pair_wait(uint32_t addr, int want, int spin_limit) {
     bool seen = false;
@@ -316,7 +334,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
 // block index (plane fastest).
 template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer,
-                                                                              uint16_t* __restrict__ direct_out) {
+                                                                              int* __restrict__ status, uint16_t* __restrict__ direct_out) {
     using L = Lut<TB, REPP>;
     __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
@@ -327,13 +345,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int pair, role;
     pair_roles(simd_of, &flag_mem[0][0], wave, lane, pair, role);
-    PairMem pm;
-    pm.lut = lds_addr(lut_mem[pair]);
-    pm.sbuf = lds_addr(s_mem[pair]);
-    pm.pbuf = lds_addr(p_mem[pair]);
-    pm.flags = lds_addr(flag_mem[pair]);
-    pm.silent = silent_scorer != 0;
-    pm.spin_limit = pm.silent ? kSpinLimitSilent : kSpinLimit;
+    const PairMem pm = pair_mem(lds_addr(lut_mem[pair]), lds_addr(s_mem[pair]), lds_addr(p_mem[pair]), lds_addr(flag_mem[pair]), silent_scorer);
 
     const int slice = blockIdx.x * kPairsPerBlock + pair;
     if (slice >= n_slices_total) return;
@@ -359,8 +371,9 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     int k = 0;
     long long waited = 0;
     PQ_PAIR_T_DECL;
-    if (role == 0) pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited);
-    else           pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
+    const bool ok = role == 0 ? pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited)
+                              : pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
+    if (!ok) report_timeout(status, lane);
 #ifdef PQ_ATTN_PHASE_TIMERS
     pw_total_ = waited;
 #endif
@@ -370,7 +383,8 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
 
 // Balanced slices for pairs: both wavefronts of a pair walk the same segment and meet tile by tile.
 template <typename T, int TB, int REPP, bool PK6>
-__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total, int silent_scorer) {
+__global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total, int silent_scorer,
+                                                                                       int* __restrict__ status) {
     using L = Lut<TB, REPP>;
     __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
@@ -382,13 +396,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int pair, role;
     pair_roles(simd_of, &flag_mem[0][0], wave, lane, pair, role);
-    PairMem pm;
-    pm.lut = lds_addr(lut_mem[pair]);
-    pm.sbuf = lds_addr(s_mem[pair]);
-    pm.pbuf = lds_addr(p_mem[pair]);
-    pm.flags = lds_addr(flag_mem[pair]);
-    pm.silent = silent_scorer != 0;
-    pm.spin_limit = pm.silent ? kSpinLimitSilent : kSpinLimit;
+    const PairMem pm = pair_mem(lds_addr(lut_mem[pair]), lds_addr(s_mem[pair]), lds_addr(p_mem[pair]), lds_addr(flag_mem[pair]), silent_scorer);
     const int w = blockIdx.x * kPairsPerBlock + pair;
     if (w >= n_pairs_total) return;
     int k = 0;
@@ -397,14 +405,19 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     PQ_PAIR_T_DECL;
     walk_segment<false>(p, v4, n_pairs_total, w, lane, lds_addr(walk_mem[wave]),
                         [&](int cb, int ckvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot, bool ends_plane) {
-                            if (!ok) return;         // the partner stopped answering: run out without touching anything
+                            // once the partner has stopped answering, the pair runs out without loads, waits or
+                            // arithmetic; the accumulator still owns the partial of every remaining piece of the
+                            // segment (a NaN header) and the empty slots behind a plane's last piece, so that the merge
+                            // never meets what an earlier call left in the workspace
                             if (role == 0) {
-                                ok = pair_scorer<T, TB, REPP, PK6>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, k, waited);
+                                if (ok) ok = pair_scorer<T, TB, REPP, PK6>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, k, waited);
                             } else {
                                 if (ends_plane && slot + 1 < n_splits) mark_empty_slots(p, lane, cb, ckvh, slot + 1);
-                                ok = pair_accumulator<T, REPP>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, slot, k, waited);
+                                if (ok) ok = pair_accumulator<T, REPP>(p, pm, lane, cb, ckvh, sc, t0, t1, r0, r1, slot, k, waited);
+                                else poison_slot(p, lane, cb, ckvh, slot);
                             }
                         });
+    if (!ok) report_timeout(status, lane);
 #ifdef PQ_ATTN_PHASE_TIMERS
     pw_total_ = waited;
 #endif
@@ -427,7 +440,7 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
-                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0, ##__VA_ARGS__)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0, a.status, ##__VA_ARGS__)
 #define PQ_LAUNCH_PAIR_P(REPP, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_PAIR_K(attn_pair_balanced_kernel, REPP, PK6);                                      \

@@ -14,10 +14,20 @@ int check_bits(int rbits, int tbits) {
     return PQ_OK;
 }
 
-// decode-side flags: only the packed 6-bit code layout, which exists for tbits == 3 (rbits <= 3)
-int check_decode_flags(unsigned flags, int rbits, int tbits, bool attention = false) {
+// decode-side flags: the packed 6-bit code layout, which exists for tbits == 3 (rbits <= 3); for the attention entry
+// points the two kernel choices; for the entry points that run the scorer / accumulator pairs, in the test build only,
+// the hook that silences the scorers
+enum class Entry { Scores, Attention, AttentionV4 };
+int check_decode_flags(unsigned flags, int rbits, int tbits, Entry entry = Entry::Scores) {
     // the score op has one slice per group; only the attention entry points cut the context
-    const unsigned known = PQ_CODES_PACKED6 | (attention ? (PQ_BALANCED_SLICES | PQ_SINGLE_WAVEFRONT | PQ_TEST_SILENT_SCORER) : 0u);
+    unsigned known = PQ_CODES_PACKED6;
+    if (entry != Entry::Scores) known |= PQ_BALANCED_SLICES;
+    // 4-bit values always run one wavefront per slice: the flag that asks for it, and the hook into the hand-over
+    // that those kernels do not have, mean nothing there
+    if (entry == Entry::Attention) known |= PQ_SINGLE_WAVEFRONT;
+#ifdef PQ_TEST_HOOKS
+    if (entry == Entry::Attention && !(flags & PQ_SINGLE_WAVEFRONT)) known |= PQ_TEST_SILENT_SCORER;
+#endif
     if (flags & ~known) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && (tbits != 3 || rbits + tbits > 6)) return PQ_ERR_BAD_BITS;
     return PQ_OK;
@@ -151,18 +161,21 @@ size_t pq_decode_attn_workspace_bytes(int B, int N, int n_splits) {
     return static_cast<size_t>(B) * N * static_cast<size_t>(n_splits) * PQ_PARTIAL_FLOATS * sizeof(float);
 }
 
-int pq_validate_decode_attn(const void* q,
-                            const uint8_t* codes, const void* rscale, const void* rmn,
-                            const void* tscale, const void* tmn, int group_capacity,
-                            int n_groups, const int32_t* n_groups_per_seq,
-                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
-                            const void* v, int64_t v_capacity,
-                            const uint8_t* mask, int64_t mask_stride,
-                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                            int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
-                            const void* out, unsigned flags) {
+}  // extern "C"
+
+namespace {
+int validate_attn(const void* q,
+                  const uint8_t* codes, const void* rscale, const void* rmn,
+                  const void* tscale, const void* tmn, int group_capacity,
+                  int n_groups, const int32_t* n_groups_per_seq,
+                  const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                  const void* v, int64_t v_capacity,
+                  const uint8_t* mask, int64_t mask_stride,
+                  float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                  int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
+                  const void* out, unsigned flags, bool v4_entry) {
     if (!q || !v || !workspace || !out) return PQ_ERR_NULL_POINTER;
-    if (int rc = check_decode_flags(flags, rbits, tbits, true)) return rc;
+    if (int rc = check_decode_flags(flags, rbits, tbits, v4_entry ? Entry::AttentionV4 : Entry::Attention)) return rc;
     if (int rc = check_heads(B, N, Nk)) return rc;
     if (static_cast<long long>(B) * Nk > 65535) return PQ_ERR_BAD_SHAPE;
     if (int rc = check_bits(rbits, tbits)) return rc;
@@ -198,6 +211,24 @@ int pq_validate_decode_attn(const void* q,
     if (k_resid && !aligned(k_resid, 16)) return PQ_ERR_MISALIGNED;
     return PQ_OK;
 }
+}  // namespace
+
+extern "C" {
+
+int pq_validate_decode_attn(const void* q,
+                            const uint8_t* codes, const void* rscale, const void* rmn,
+                            const void* tscale, const void* tmn, int group_capacity,
+                            int n_groups, const int32_t* n_groups_per_seq,
+                            const void* k_resid, int resid_capacity, int n_resid, const int32_t* n_resid_per_seq,
+                            const void* v, int64_t v_capacity,
+                            const uint8_t* mask, int64_t mask_stride,
+                            float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
+                            int n_splits, int min_groups_per_split, const void* workspace, size_t workspace_bytes,
+                            const void* out, unsigned flags) {
+    return validate_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq, k_resid,
+                         resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask, mask_stride, sm_scale, B, N, Nk,
+                         rbits, tbits, dtype, n_splits, min_groups_per_split, workspace, workspace_bytes, out, flags, false);
+}
 
 namespace {
 // The attention launch of pq_decode_attn_partials.  direct_out != nullptr (one slice per plane, default kernels): the
@@ -211,13 +242,14 @@ int run_attn_partials(const void* q,
                       const uint8_t* mask, int64_t mask_stride,
                       float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                       int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                      unsigned flags, void* stream, void* direct_out) {
+                      unsigned flags, int32_t* status, void* stream, void* direct_out) {
     // `out` is not touched by the partials: validate with a stand-in non-null, aligned pointer
     if (int rc = pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                          k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                          mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
                                          workspace, workspace_bytes, workspace, flags))
         return rc;
+    if (status && !aligned(status, 4)) return PQ_ERR_MISALIGNED;
     pq::AttnArgs a;
     a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
     a.group_capacity = group_capacity; a.n_groups = n_groups; a.n_groups_per_seq = n_groups_per_seq;
@@ -229,6 +261,7 @@ int run_attn_partials(const void* q,
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
     a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
     a.silent_scorer = (flags & PQ_TEST_SILENT_SCORER) != 0;
+    a.status = status;
     a.workspace = static_cast<float*>(workspace); a.out = direct_out;
     const int err = pq::launch_attn_partials(a, static_cast<hipStream_t>(stream));
     return err == 0 ? PQ_OK : PQ_ERR_LAUNCH;
@@ -244,11 +277,11 @@ int pq_decode_attn_partials(const void* q,
                             const uint8_t* mask, int64_t mask_stride,
                             float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                             int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                            unsigned flags, void* stream) {
+                            unsigned flags, int32_t* status, void* stream) {
     return run_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq, k_resid,
                              resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask, mask_stride, sm_scale, B, N, Nk,
-                             rbits, tbits, dtype, n_splits, min_groups_per_split, workspace, workspace_bytes, flags, stream,
-                             nullptr);
+                             rbits, tbits, dtype, n_splits, min_groups_per_split, workspace, workspace_bytes, flags, status,
+                             stream, nullptr);
 }
 
 int pq_decode_attn_merge(const void* workspace, size_t workspace_bytes, int B, int N, int n_splits, int dtype,
@@ -273,7 +306,7 @@ int pq_decode_attn(const void* q,
                    const uint8_t* mask, int64_t mask_stride,
                    float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                    int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                   void* out, unsigned flags, void* stream) {
+                   void* out, unsigned flags, int32_t* status, void* stream) {
     if (!out) return PQ_ERR_NULL_POINTER;
     if (!aligned(out, 2)) return PQ_ERR_MISALIGNED;
     // one slice per plane (a batch large enough to fill the device by itself): the default kernels write the output
@@ -282,7 +315,7 @@ int pq_decode_attn(const void* q,
     if (int rc = run_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                    k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                    mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,
-                                   workspace, workspace_bytes, flags, stream, direct ? out : nullptr))
+                                   workspace, workspace_bytes, flags, status, stream, direct ? out : nullptr))
         return rc;
     if (direct) return PQ_OK;
     return pq_decode_attn_merge(workspace, workspace_bytes, B, N, n_splits, dtype, out, stream);
@@ -296,7 +329,8 @@ int pq_decode_attn_static(const void* q,
                           const void* v, int64_t v_capacity,
                           const uint8_t* mask, int64_t mask_stride,
                           float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
-                          int n_splits, int min_groups_per_split, void* out, unsigned flags, void* stream) {
+                          int n_splits, int min_groups_per_split, void* out, unsigned flags, int32_t* status,
+                          void* stream) {
     static_assert(PQ_STATIC_MAX_PARTIALS == pq::kStaticMaxPartials, "header and library disagree");
     if (B <= 0 || N <= 0 || n_splits < 1) return PQ_ERR_BAD_SHAPE;
     if (static_cast<long long>(B) * N * n_splits > PQ_STATIC_MAX_PARTIALS) return PQ_ERR_WORKSPACE;
@@ -307,7 +341,8 @@ int pq_decode_attn_static(const void* q,
     return pq_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq, k_resid,
                           resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask, mask_stride, sm_scale, B, N, Nk,
                           rbits, tbits, dtype, n_splits, min_groups_per_split, ws,
-                          static_cast<size_t>(PQ_STATIC_MAX_PARTIALS) * PQ_PARTIAL_FLOATS * sizeof(float), out, flags, stream);
+                          static_cast<size_t>(PQ_STATIC_MAX_PARTIALS) * PQ_PARTIAL_FLOATS * sizeof(float), out, flags, status,
+                          stream);
 }
 
 // ---- fused elementwise steps of the decode layer -----------------------------------------------
@@ -501,10 +536,10 @@ int pq_validate_decode_attn_v4(const void* q,
     // everything else as in the fp16-value entry point; its V-capacity rule is met by construction here
     static const char dummy_v[16] __attribute__((aligned(16))) = {0};
     const int64_t vcap = static_cast<int64_t>(group_capacity > n_groups ? group_capacity : n_groups) * PQ_GROUP + resid_capacity + 1;
-    return pq_validate_decode_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
-                                   k_resid, resid_capacity, n_resid, n_resid_per_seq, dummy_v, vcap, mask, mask_stride,
-                                   sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
-                                   workspace_bytes, out, flags);
+    return validate_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
+                         k_resid, resid_capacity, n_resid, n_resid_per_seq, dummy_v, vcap, mask, mask_stride,
+                         sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
+                         workspace_bytes, out, flags, true);
 }
 
 int pq_decode_attn_v4(const void* q,
@@ -534,8 +569,6 @@ int pq_decode_attn_v4(const void* q,
     a.min_groups_per_split = min_groups_per_split;
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
-    a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
-    a.silent_scorer = (flags & PQ_TEST_SILENT_SCORER) != 0;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     if (any_groups) {
         a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token

@@ -61,7 +61,8 @@ struct AttnArgs {
     bool packed6 = false;        // code rows are 48 bytes of packed 6-bit codes (tbits == 3 only)
     bool balanced = false;       // slices cut on the device from the per-sequence counts (PQ_BALANCED_SLICES)
     bool single_wave = false;    // one wavefront per slice instead of a scorer / accumulator pair (PQ_SINGLE_WAVEFRONT)
-    bool silent_scorer = false;  // PQ_TEST_SILENT_SCORER
+    bool silent_scorer = false;  // PQ_TEST_SILENT_SCORER (honoured by the test build only)
+    int32_t* status = nullptr;   // optional device word the paired kernels set when a hand-over gives up
     float* workspace;
     void* out;
 };

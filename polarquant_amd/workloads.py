@@ -124,18 +124,20 @@ def algorithmic_bytes(n_kv_heads: int, n_heads: int, quant_tokens: List[int], re
 
 
 # ----------------------------------------------------------------------------- GPU-resident workloads and timing
-def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False, keep_keys_of=None):
+def build_workload(idx, dev, dtype=torch.float16, keep_keys=False, packed=False, keep_keys_of=None, variant=0):
     """configs[idx] resident in HBM: polar key cache of L/128 groups per (sequence, KV head),
     fp16 V cache, one new token whose key sits in the fp16 residual buffer.  Ragged shapes
     (configs[2]) carry per-sequence group / residual counts; their caches are sized for the longest.
     keep_keys keeps the half-precision keys of every sequence in w["keys"], keep_keys_of=n those of the
-    first n sequences only."""
+    first n sequences only.  variant > 0: an independent input set of the same shape (other random
+    data in other memory, the same per-sequence lengths), for timings that rotate input sets so that no
+    call finds its inputs in a cache."""
     from .quantize import quantize_and_pack_nbit
 
     sh = CONFIGS[idx]
     B, N, Nk, L = sh.batch, sh.n_heads, sh.n_kv_heads, sh.context
     Nb = L // 128
-    g = torch.Generator(device=dev).manual_seed(sh.seed)
+    g = torch.Generator(device=dev).manual_seed(sh.seed + 7919 * variant)
     # packed: 6-bit codes stored 48 bytes per token (needs rbits + tbits <= 6, i.e. configs[2])
     codes = torch.empty(B, Nk, Nb, 128, 48 if packed else 64, dtype=torch.uint8, device=dev)
     meta = [torch.empty(B, Nk, Nb, 1, 64, dtype=dtype, device=dev) for _ in range(4)]

@@ -23,7 +23,7 @@ int main(void) {
     /* the compute entry points refuse bad arguments before touching the device */
     if (pq_rmsnorm(NULL, NULL, p, p, NULL, 1, 128, 1e-5f, PQ_F16, NULL) != PQ_ERR_NULL_POINTER) return 10;
     if (pq_decode_attn(NULL, p, p, p, p, p, 4, 3, NULL, p, 128, 5, NULL, p, 1024, NULL, 0, 0.088f, 2, 32, 8, 4, 4, PQ_F16, 4, 0,
-                       p, 1u << 20, p, 0, NULL) != PQ_ERR_NULL_POINTER) return 11;
+                       p, 1u << 20, p, 0, NULL, NULL) != PQ_ERR_NULL_POINTER) return 11;
     if (pq_validate_decode_scores(p, p, p, p, p, p, p, 2, 28, 4, 4, 3, 3, PQ_F16, PQ_CODES_PACKED6) != PQ_OK) return 12;
     if (pq_validate_decode_scores(p, p, p, p, p, p, p, 2, 28, 4, 4, 4, 4, PQ_F16, PQ_CODES_PACKED6) != PQ_ERR_BAD_BITS) return 13;
     printf("capi ok, version %d, group %d, head_dim %d\n", pq_version(), PQ_GROUP, PQ_HEAD_DIM);

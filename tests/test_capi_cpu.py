@@ -105,7 +105,7 @@ def test_validate_quantize_groups(lib):
     assert lib.pq_validate_quantize_groups(*a) == 0
 
 
-def test_validate_decode_attn_and_plan(lib):
+def test_validate_decode_attn_and_plan(lib, hooks_lib):
     B, N, Nk, ns = 2, 32, 8, 4
     wsb = lib.pq_decode_attn_workspace_bytes(B, N, ns)
     assert wsb == B * N * ns * 132 * 4
@@ -145,8 +145,16 @@ def test_validate_decode_attn_and_plan(lib):
     a[29] = 32 | 16
     assert lib.pq_validate_decode_attn(*a) == 0
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 32) == -2
+    # PQ_TEST_SILENT_SCORER, the hook that turns a call's output into NaN: the shipping library refuses it like any
+    # unknown flag; the test build takes it, but not where there is no hand-over to silence
     a = list(ok); a[29] = 0x40000000
-    assert lib.pq_validate_decode_attn(*a) == 0                      # PQ_TEST_SILENT_SCORER (test hook of the hand-over)
+    assert lib.pq_validate_decode_attn(*a) == -2
+    hooks = hooks_lib
+    assert hooks.pq_validate_decode_attn(*a) == 0
+    a[29] = 0x40000000 | 32
+    assert hooks.pq_validate_decode_attn(*a) == -2                   # with PQ_SINGLE_WAVEFRONT
+    a[29] = 0x40000000 | 16
+    assert hooks.pq_validate_decode_attn(*a) == 0                    # with balanced slices
     a = list(ok); a[29] = 64
     assert lib.pq_validate_decode_attn(*a) == -2                     # unknown flag bit
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 16) == -2
@@ -165,7 +173,7 @@ def test_validate_decode_attn_and_plan(lib):
     assert lib.pq_decode_attn_merge(None, 0, 1, 1, 1, 0, None, None) == -1
 
 
-def test_validate_value_quantizer_and_v4_attention(lib):
+def test_validate_value_quantizer_and_v4_attention(lib, hooks_lib):
     strides = (ctypes.c_int64 * 4)(8 * 300 * 128, 300 * 128, 128, 1)
     sp = ctypes.cast(strides, ctypes.c_void_p)
     ok = [P, sp, 0, 2, 8, 300, P, P, P, 512, 100]
@@ -200,6 +208,11 @@ def test_validate_value_quantizer_and_v4_attention(lib):
     assert bad4(13, P + 8) == -5
     a = list(ok); a[1:6] = [None] * 5; a[6] = 0; a[7] = 0; a[14:17] = [None] * 3; a[17] = 0
     assert lib.pq_validate_decode_attn_v4(*a) == 0            # nothing quantized yet
+    # the 4-bit-value kernels always run one wavefront per slice: the flag that asks for that form, and the test hook
+    # into the hand-over those kernels do not have, are refused instead of silently ignored (in the test build too)
+    assert bad4(32, 16) == 0 and bad4(32, 32) == -2 and bad4(32, 0x40000000) == -2
+    a = list(ok); a[32] = 0x40000000
+    assert hooks_lib.pq_validate_decode_attn_v4(*a) == -2
     # two wavefronts per SIMD for up to 4 query heads per KV head, one beyond
     assert lib.pq_decode_attn_v4_plan(16, 32, 8, 256, 256) == 16
     assert lib.pq_decode_attn_v4_plan(64, 28, 4, 64, 256) == 4

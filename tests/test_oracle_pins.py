@@ -193,6 +193,21 @@ def test_fp32_wrap_switch_of_both_restatements(dtype):
     assert int((a[3].view(torch.int16) != d[3].view(torch.int16)).sum()) > 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_the_device_eager_lines_agree_with_the_oracle_on_cpu_tensors(dtype):
+    """oracle/device_eager.py holds the reference's lines for evaluation on GPU tensors; on CPU tensors it must be the
+    torch oracle bit for bit (the C restatement then pins both), so that only torch's own device behaviour separates
+    what it computes on a GPU from the pinned CPU evaluation."""
+    from oracle.device_eager import quantize_and_pack_nbit_eager
+    k, _ = _keys(2, 4, 1024, 5, dtype)
+    for rbits, tbits in ((4, 4), (3, 3), (2, 6)):
+        a = po.quantize_and_pack_nbit(k, rbits, tbits)
+        b = quantize_and_pack_nbit_eager(k, rbits, tbits)
+        assert torch.equal(a[0], b[0])
+        for x, y in zip(a[1:], b[1:]):
+            assert torch.equal(x.view(torch.int16), y.view(torch.int16))
+
+
 def test_rope_pair_convention_matches_hf_rotate_half():
     """x = dims [0,64), y = dims [64,128) is the HF rotate-half pairing: rotating a
     key by RoPE turns pair (d, d+64) by the angle pos * inv_freq[d] and keeps its radius."""

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 from oracle import polar_oracle as po
+from oracle.device_eager import quantize_and_pack_nbit_eager
 from polarquant_amd import workloads as wl
 from polarquant_amd.quantize import quantize_and_pack_nbit
 
@@ -145,25 +146,6 @@ def test_quantize_wrap_fp32_flag(gpu, dtype, shape, rbits, tbits, theta):
         assert all(v == 0 for v in flips.values()), (name, flips)
 
 
-def _reference_lines_on_device(key_states, rbits, tbits, G=128):
-    """models/modeling_llama_polar.py:141-155 as plain eager torch ops, meant to be called with tensors ON THE GPU:
-    torch-ROCm's own kernels (a library, not the reference) then evaluate each line the way the reference's lines
-    are evaluated when the model runs on a GPU.  Degenerate groups (0/0 -> uint8) are avoided by the callers."""
-    B, N, L, D = key_states.shape
-    D = D // 2
-    ks = key_states.view(B, N, L // G, G, 2, D)
-    phi = torch.atan2(ks[:, :, :, :, 1, :], ks[:, :, :, :, 0, :])
-    phi = torch.where(phi < 0, phi + 2 * math.pi, phi)
-    tmx, tmn = phi.max(-2, keepdim=True)[0], phi.min(-2, keepdim=True)[0]
-    tscale = (tmx - tmn) / (2 ** tbits)
-    theta = torch.clamp(torch.floor((phi - tmn) / tscale).to(torch.uint8), 0, 2 ** tbits - 1)
-    radii = torch.norm(ks, p=2, dim=-2)
-    rmx, rmn = radii.max(-2, keepdim=True)[0], radii.min(-2, keepdim=True)[0]
-    rscale = (rmx - rmn) / (2 ** rbits)
-    rho = torch.clamp(torch.floor((radii - rmn) / rscale).to(torch.uint8), 0, 2 ** rbits - 1)
-    return (rho << tbits) + theta, rscale, rmn, tscale, tmn
-
-
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("cfg,rbits,tbits", [(0, 4, 4), (2, 3, 3)])
 def test_quantize_eager_gpu_mode_against_eager_torch_on_the_device(gpu, dtype, cfg, rbits, tbits):
@@ -177,7 +159,7 @@ def test_quantize_eager_gpu_mode_against_eager_torch_on_the_device(gpu, dtype, c
     sh = wl.CONFIGS[cfg]
     g = torch.Generator().manual_seed(sh.seed)
     k = wl.make_keys(1, sh.n_kv_heads, 4096, sh.rope_theta, g, dtype).to(gpu)
-    ref = _reference_lines_on_device(k, rbits, tbits)
+    ref = quantize_and_pack_nbit_eager(k, rbits, tbits)
     got = quantize_and_pack_nbit(k, rbits, tbits, eager_gpu=True)
     torch.cuda.synchronize()
     flips = count_flips([t.cpu() for t in got], [t.cpu() for t in ref])

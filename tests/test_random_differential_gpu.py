@@ -169,9 +169,9 @@ def test_random_quantizer_case(gpu, seed):
     if mode == "group":
         # the same keys in the mode that follows eager torch on GPU tensors, against eager torch ops on the device
         # (0/0 groups, undefined in the reference, are left out: their metadata must agree, their codes need not)
-        from test_quantize_gpu import _reference_lines_on_device
+        from oracle.device_eager import quantize_and_pack_nbit_eager
         xd = x.to(gpu)
-        dref = [t.cpu() for t in _reference_lines_on_device(xd, rb, tb)]
+        dref = [t.cpu() for t in quantize_and_pack_nbit_eager(xd, rb, tb)]
         dgot = [t.cpu() for t in quantize_and_pack_nbit(xd, rb, tb, eager_gpu=True)]
         for name, a, b in zip(["rscale", "rmn", "tscale", "tmn"], dgot[1:], dref[1:]):
             a, b = a.float(), b.float()

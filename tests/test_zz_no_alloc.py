@@ -40,11 +40,11 @@ def _call(static, dev, B, N, Nk, n_groups, n_resid, n_splits, gpu, flags=0):
             1.0 / math.sqrt(128), B, N, Nk, 4, 4, _ffi.PQ_F16, n_splits, 0]
     lib = _ffi.lib()
     if static:
-        rc = lib.pq_decode_attn_static(*head, out.data_ptr(), flags, _stream_ptr(gpu))
+        rc = lib.pq_decode_attn_static(*head, out.data_ptr(), flags, None, _stream_ptr(gpu))
     else:
         nbytes = lib.pq_decode_attn_workspace_bytes(B, N, n_splits)
         ws = torch.full((nbytes // 4,), float("nan"), dtype=torch.float32, device=gpu)
-        rc = lib.pq_decode_attn(*head, ws.data_ptr(), nbytes, out.data_ptr(), flags, _stream_ptr(gpu))
+        rc = lib.pq_decode_attn(*head, ws.data_ptr(), nbytes, out.data_ptr(), flags, None, _stream_ptr(gpu))
     assert rc == 0, _ffi.STATUS_NAMES.get(rc, rc)
     torch.cuda.synchronize()
     return out.cpu()
@@ -88,5 +88,5 @@ def test_static_entry_point_rejects_sizes_beyond_its_buffer(gpu):
     rc = _ffi.lib().pq_decode_attn_static(
         q.data_ptr(), codes.data_ptr(), rs.data_ptr(), rm.data_ptr(), ts.data_ptr(), tm.data_ptr(), 2, 2, None,
         kres.data_ptr(), kres.shape[2], 1, None, v.data_ptr(), v.shape[2], None, 0, 0.088, 1, 32, 8, 4, 4, _ffi.PQ_F16,
-        513, 0, out.data_ptr(), 0, _stream_ptr(gpu))
+        513, 0, out.data_ptr(), 0, None, _stream_ptr(gpu))
     assert rc == -7          # PQ_ERR_WORKSPACE
