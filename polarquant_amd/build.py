@@ -18,7 +18,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libpolarquant_hip.so")
-SOURCES = ["pq_capi.hip", "pq_scores.hip", "pq_quantize.hip", "pq_values.hip", "pq_decode_ops.hip", "pq_linear.hip", "pq_attn.hip", "pq_attn_pair.hip"]
+# (source, defines, object tag): the two attention sources are compiled once per dtype, so that the halves of their
+# many template instantiations build side by side
+UNITS = [("pq_attn.hip", ("PQ_DTYPE=0",), ".f16"), ("pq_attn.hip", ("PQ_DTYPE=1",), ".bf16"),
+         ("pq_attn_pair.hip", ("PQ_DTYPE=0",), ".f16"), ("pq_attn_pair.hip", ("PQ_DTYPE=1",), ".bf16"),
+         ("pq_scores.hip", (), ""), ("pq_quantize.hip", (), ""), ("pq_linear.hip", (), ""), ("pq_attn_common.hip", (), ""),
+         ("pq_capi.hip", (), ""), ("pq_values.hip", (), ""), ("pq_decode_ops.hip", (), "")]
+SOURCES = sorted({u[0] for u in UNITS})
 # measurement aids (a plain streaming read, the attention kernel's loads without its arithmetic): a library of
 # their own, loaded by bench.py and its tests only
 BENCH_LIB = os.path.join(HERE, "libpolarquant_bench.so")
@@ -39,7 +45,10 @@ TIMERS_LIB = os.path.join(HERE, "libpolarquant_hip_timers.so")
 # the test build: the same library with -DPQ_TEST_HOOKS, which alone honours PQ_TEST_SILENT_SCORER (a hook that turns
 # the output into NaN on purpose).  Loaded by tests/test_pair_handover_gpu.py only, never by the package.
 HOOKS_LIB = os.path.join(HERE, "libpolarquant_hip_testhooks.so")
-HOOKS_SOURCES = ["pq_capi.hip", "pq_attn_pair.hip"]          # the sources that read the define
+# the units that read the define: the C ABI's flag check and the paired kernels (float16 only: the hook is honoured for
+# that dtype, which is what its test uses; the bfloat16 kernels of the test build are the shipping ones)
+HOOKS_UNITS = {("pq_capi.hip", ""): ("pq_capi.hip", ("PQ_TEST_HOOKS",), ".hooks"),
+               ("pq_attn_pair.hip", ".f16"): ("pq_attn_pair.hip", ("PQ_DTYPE=0", "PQ_TEST_HOOKS"), ".f16.hooks")}
 
 
 def _compile(src: str, defines=(), tag: str = "") -> str:
@@ -68,20 +77,22 @@ def build(verbose: bool = True, phase_timers: bool = False) -> str:
     whose attention kernel times its phases with the wall clock and prints them: a measuring build for
     `python -m polarquant_amd.benchmarks.phase_timing`, a few percent slower than the real one."""
     os.makedirs(OBJ, exist_ok=True)
-    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    lib, defines, tag = (TIMERS_LIB, ("PQ_ATTN_PHASE_TIMERS",), ".timers") if phase_timers else (LIB, (), "")
-    jobs = [(s_, defines, tag) for s_ in srcs]
-    if not phase_timers:
-        jobs += [(s_, ("PQ_TEST_HOOKS",), ".hooks") for s_ in HOOKS_SOURCES] + [(s_, (), "") for s_ in BENCH_SOURCES]
-    # the longest compilations first, so that they do not start last
-    jobs.sort(key=lambda j: -os.path.getsize(os.path.join(CSRC, j[0])) if "attn" not in j[0] else -1 << 30)
+    if phase_timers:
+        main = [(src, defs + ("PQ_ATTN_PHASE_TIMERS",), tag + ".timers") for src, defs, tag in UNITS]
+        jobs = list(main)
+    else:
+        main = list(UNITS)
+        hooks = [HOOKS_UNITS.get((src, tag), (src, defs, tag)) for src, defs, tag in UNITS]
+        bench = [(s_, (), "") for s_ in BENCH_SOURCES]
+        jobs = main + [u for u in hooks if u not in main] + bench
+    # the units are listed longest compilation first
     with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:
-        built = dict(zip([(j[0], j[2]) for j in jobs], ex.map(lambda j: _compile(*j), jobs)))
-    objs = [built[(s_, tag)] for s_ in srcs]
-    _link(objs, lib)
+        built = dict(zip(jobs, ex.map(lambda j: _compile(*j), jobs)))
+    lib = TIMERS_LIB if phase_timers else LIB
+    _link([built[u] for u in main], lib)
     if not phase_timers:
-        _link([built[(s_, ".hooks" if s_ in HOOKS_SOURCES else "")] for s_ in srcs], HOOKS_LIB)
-        _link([built[(s_, "")] for s_ in BENCH_SOURCES], BENCH_LIB)
+        _link([built[u] for u in hooks], HOOKS_LIB)
+        _link([built[u] for u in bench], BENCH_LIB)
         if verbose:
             print("built", HOOKS_LIB)
             print("built", BENCH_LIB)

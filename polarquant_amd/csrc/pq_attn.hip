@@ -1,7 +1,6 @@
 // Fused polar-key decode attention, the kernels with ONE wavefront per slice: quantized-key scores,
 // half-precision residual-key scores, 1/sqrt(d), mask, softmax and P.V in one pass over HBM
-// (reference decode branch: models/modeling_llama_polar.py:66-99), split over the context; and the
-// small merge kernel that follows every attention kernel.  These kernels serve the 4-bit values of the
+// (reference decode branch: models/modeling_llama_polar.py:66-99), split over the context; These kernels serve the 4-bit values of the
 // Mixed variant and PQ_SINGLE_WAVEFRONT; with half-precision values the default kernels are the
 // scorer / accumulator pairs of pq_attn_pair.hip, which share the device code of pq_attn_device.h.
 //
@@ -25,11 +24,13 @@
 // kLazyThreshold (in log2 units): probabilities stay below 2^8, and the
 // 32-register rescale of the accumulators is skipped on almost every tile.
 //
-// merge_kernel: grid B*N, 128 threads (one per output dim), or four / eight such
-// groups that share the partials when there are 32 / 128 or more: combines the n_splits
-// partials (m, l, acc[128]) of a query head and writes half words.
+// The merge kernel that follows every attention kernel is in pq_attn_common.hip.  This file is compiled once per
+// dtype (-DPQ_DTYPE=0 float16, 1 bfloat16).
 #include "pq_attn_device.h"
-#include <mutex>
+
+#ifndef PQ_DTYPE
+#error "compile with -DPQ_DTYPE=0 (float16) or 1 (bfloat16)"
+#endif
 
 #include "pq_phase_timers.h"
 
@@ -292,12 +293,12 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
 // sequence, gps = max(min_gps, ceil(groups / n_splits)); the block that holds the last group also
 // takes the residual keys.
 template <typename T, int TB, int REPP, bool V4, bool PK6>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4 && TB <= 4) ? 2 : 1, 2)))
 void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
     using L = Lut<TB, REPP>;
     // the table region doubles as the staging buffer of the residual block's scores ([REPP][64] fp32)
     constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
-    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kLutBytes];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
     PQ_ATTN_KERNEL_PACK;
@@ -335,11 +336,11 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
 }
 
 template <typename T, int TB, int REPP, bool V4, bool PK6>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4) ? 2 : 1, 2)))
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && REPP <= 4 && TB <= 4) ? 2 : 1, 2)))
 void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     using L = Lut<TB, REPP>;
     constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
-    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kLutBytes];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
     __shared__ int walk[8];
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
@@ -355,103 +356,10 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
 
 #pragma clang diagnostic pop
 
-template <typename T, int G>
-__global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __restrict__ ws, int n_part, uint16_t* __restrict__ out) {
-    // one block per query head, G groups of 128 threads: thread (grp, d) sums output dim d over
-    // the grp-th share of the partials, and the G sums are added in a fixed order through LDS.
-    // The partial headers (m, l) are fetched by one thread each, so that all loads of the block
-    // are issued at once instead of one dependent load per partial.
-    constexpr int NT = kHeadDim * G, NW = NT / kWave;
-    __shared__ float wgt[1024];
-    __shared__ float red[2][NW];
-    __shared__ float part[G][kHeadDim];
-    const int bn = blockIdx.x, tid = threadIdx.x, d = tid & (kHeadDim - 1), grp = tid / kHeadDim;
-    const float* p = ws + static_cast<size_t>(bn) * n_part * kPartialFloats;
-    float M = -INFINITY;
-    for (int s = tid; s < n_part; s += NT) M = fmaxf(M, p[static_cast<size_t>(s) * kPartialFloats]);
-    M = wave_max(M);
-    if ((tid & (kWave - 1)) == 0) red[0][tid / kWave] = M;
-    __syncthreads();
-    M = red[0][0];
-#pragma unroll
-    for (int i = 1; i < NW; i++) M = fmaxf(M, red[0][i]);
-    float num = 0.0f, den = 0.0f;
-    for (int s0 = 0; s0 < n_part; s0 += 1024) {
-        const int cnt = (n_part - s0) < 1024 ? (n_part - s0) : 1024;
-        __syncthreads();
-        for (int s = tid; s < cnt; s += NT) {
-            const float m = p[static_cast<size_t>(s0 + s) * kPartialFloats];
-            const float w = (m == -INFINITY) ? 0.0f : exp2f(m - M);
-            wgt[s] = w;
-            // an empty slice contributes nothing, whatever its sum word holds
-            den = w != 0.0f ? __builtin_fmaf(w, p[static_cast<size_t>(s0 + s) * kPartialFloats + 1], den) : den;
-        }
-        __syncthreads();
-        const float* pa = p + static_cast<size_t>(s0) * kPartialFloats + 4 + d;
-        const int per = (cnt + G - 1) / G;
-        int s = grp * per;
-        const int se = (s + per) < cnt ? (s + per) : cnt;
-        for (; s + 16 <= se; s += 16) {
-            float v[16];
-#pragma unroll
-            for (int u = 0; u < 16; u++) v[u] = pa[static_cast<size_t>(s + u) * kPartialFloats];
-#pragma unroll
-            for (int u = 0; u < 16; u++) num = wgt[s + u] != 0.0f ? __builtin_fmaf(wgt[s + u], v[u], num) : num;
-        }
-        for (; s + 8 <= se; s += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; u++) v[u] = pa[static_cast<size_t>(s + u) * kPartialFloats];
-#pragma unroll
-            for (int u = 0; u < 8; u++) num = wgt[s + u] != 0.0f ? __builtin_fmaf(wgt[s + u], v[u], num) : num;
-        }
-        for (; s < se; s++) {
-            const float v = pa[static_cast<size_t>(s) * kPartialFloats];
-            num = wgt[s] != 0.0f ? __builtin_fmaf(wgt[s], v, num) : num;
-        }
-    }
-    den = wave_sum(den);
-    __syncthreads();
-    if ((tid & (kWave - 1)) == 0) red[1][tid / kWave] = den;
-    if (G > 1) part[grp][d] = num;
-    __syncthreads();
-    if (grp != 0) return;
-    den = red[1][0];
-#pragma unroll
-    for (int i = 1; i < NW; i++) den += red[1][i];
-#pragma unroll
-    for (int i = 1; i < G; i++) num += part[i][d];
-    // nothing to attend to (den == 0) gives zeros; a NaN among the partials (a poisoned slice) must stay visible
-    out[static_cast<size_t>(bn) * kHeadDim + d] = f2lo<T>(den > 0.0f ? num / den : (den == den ? 0.0f : den));
-}
-
-// Wavefront slots of the current device for the balanced kernel: one wavefront per SIMD (4 per
-// compute unit), two for the 4-bit-value kernel with up to 4 query heads per KV head.
-static int device_compute_units() {
-    constexpr int kMaxDevices = 64;
-    static std::mutex mu;
-    static int cus[kMaxDevices] = {};
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
-    std::lock_guard<std::mutex> lock(mu);
-    if (!cus[dev]) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cus[dev] = n;
-    }
-    return cus[dev];
-}
-
 template <typename T, int TB>
-static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
+static int launch_attn_tb(const AttnArgs& a, int total, hipStream_t st) {
     const int rep = a.N / a.Nk;
-    dim3 grid(static_cast<unsigned>(a.n_splits) * static_cast<unsigned>(a.B * a.Nk)), block(kWave);
-    if (a.balanced) {
-        // as many wavefronts as the device holds at once, but never more than there are partial slots
-        const long long slots = static_cast<long long>(device_compute_units()) * ((a.v4_codes && rep_pad(rep) <= 4) ? 8 : 4);
-        const long long most = static_cast<long long>(a.n_splits) * a.B * a.Nk;
-        grid = dim3(static_cast<unsigned>(slots < most ? slots : most));
-    }
+    const dim3 grid(static_cast<unsigned>(total)), block(kWave);
     const float scale_log2 = a.sm_scale * kLog2e;
     V4Args v4{static_cast<const uint32_t*>(a.v4_codes), static_cast<const uint16_t*>(a.v4_scale),
               static_cast<const uint16_t*>(a.v4_zero), a.v4_capacity};
@@ -482,8 +390,6 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
         if (a.v4_codes) PQ_LAUNCH_V(REPP, true);                                                                     \
         else PQ_LAUNCH_V(REPP, false);                                                                               \
     } while (0)
-    // half-precision values: a scorer / accumulator pair of wavefronts per slice or segment (pq_attn_pair.hip)
-    if (!a.v4_codes && !a.single_wave) return launch_attn_pair(a, static_cast<int>(grid.x), st);
     switch (rep_pad(rep)) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;
@@ -497,65 +403,21 @@ static int launch_attn_tb(const AttnArgs& a, hipStream_t st) {
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename T>
-static int launch_attn_t(const AttnArgs& a, hipStream_t st) {
+#if PQ_DTYPE == 0
+int launch_attn_one_f16(const AttnArgs& a, int total, hipStream_t st) {
+    using T = F16;
+#else
+int launch_attn_one_bf16(const AttnArgs& a, int total, hipStream_t st) {
+    using T = BF16;
+#endif
     switch (a.tbits) {
-        case 1: return launch_attn_tb<T, 1>(a, st);
-        case 2: return launch_attn_tb<T, 2>(a, st);
-        case 3: return launch_attn_tb<T, 3>(a, st);
-        default: return launch_attn_tb<T, 4>(a, st);
+        case 1: return launch_attn_tb<T, 1>(a, total, st);
+        case 2: return launch_attn_tb<T, 2>(a, total, st);
+        case 3: return launch_attn_tb<T, 3>(a, total, st);
+        case 4: return launch_attn_tb<T, 4>(a, total, st);
+        case 5: return launch_attn_tb<T, 5>(a, total, st);
+        default: return launch_attn_tb<T, 6>(a, total, st);
     }
-}
-
-int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
-    return a.dtype == 0 ? launch_attn_t<F16>(a, st) : launch_attn_t<BF16>(a, st);
-}
-
-constexpr int kMergeWideFrom = 32, kMergeWidestFrom = 128;
-
-int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st) {
-    // many partials per head (a long context cut into many slices): four or eight groups of threads share them
-    if (n_splits >= kMergeWidestFrom) {
-        if (dtype == 0)
-            hipLaunchKernelGGL((merge_kernel<F16, 8>), dim3(B * N), dim3(kHeadDim * 8), 0, st, ws, n_splits, (uint16_t*)out);
-        else
-            hipLaunchKernelGGL((merge_kernel<BF16, 8>), dim3(B * N), dim3(kHeadDim * 8), 0, st, ws, n_splits, (uint16_t*)out);
-    } else if (n_splits >= kMergeWideFrom) {
-        if (dtype == 0)
-            hipLaunchKernelGGL((merge_kernel<F16, 4>), dim3(B * N), dim3(kHeadDim * 4), 0, st, ws, n_splits, (uint16_t*)out);
-        else
-            hipLaunchKernelGGL((merge_kernel<BF16, 4>), dim3(B * N), dim3(kHeadDim * 4), 0, st, ws, n_splits, (uint16_t*)out);
-    } else if (dtype == 0) {
-        hipLaunchKernelGGL((merge_kernel<F16, 1>), dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
-    } else {
-        hipLaunchKernelGGL((merge_kernel<BF16, 1>), dim3(B * N), dim3(kHeadDim), 0, st, ws, n_splits, (uint16_t*)out);
-    }
-    return static_cast<int>(hipGetLastError());
-}
-
-// ---- scratch of the entry point that allocates nothing (pq_decode_attn_static) -----------------
-// The split partials of that entry point live in this file-scope device array instead of a caller's
-// workspace.  Every GPU the library runs on holds its own copy at its own address until the process
-// ends; the array's name is only a host-side handle, so the device address is asked for once per
-// device (with that device current) and kept.
-static __device__ __align__(256) float scratch[static_cast<size_t>(kStaticMaxPartials) * kPartialFloats];
-
-int attn_static_scratch(float** ptr) {
-    constexpr int kMaxDevices = 64;
-    static std::mutex mu;
-    static float* per_device[kMaxDevices] = {};
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
-    std::lock_guard<std::mutex> lock(mu);
-    if (!per_device[dev]) {
-        void* p = nullptr;
-        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return static_cast<int>(e);
-        if (!p) return static_cast<int>(hipErrorInvalidSymbol);
-        per_device[dev] = static_cast<float*>(p);
-    }
-    *ptr = per_device[dev];
-    return 0;
 }
 
 }  // namespace pq

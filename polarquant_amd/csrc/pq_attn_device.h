@@ -80,7 +80,7 @@ __device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[
     }
     asm volatile("" ::: "memory");
     const int g = lane >> 4, n = lane & 15;
-    const uint32_t prow = pbuf + ((n & (REPP - 1)) * kWave + 4 * g) * 2;
+    const uint32_t prow = pbuf + ((n < REPP ? n : 0) * kWave + 4 * g) * 2;      // columns past the last head: any row, never stored
 #pragma unroll
     for (int tb = 0; tb < 4; tb++) {
         const __attribute__((address_space(3))) uint2* pp = lds_ptr<__attribute__((address_space(3))) uint2>(prow + tb * 32);
@@ -171,7 +171,7 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
     }
     asm volatile("" ::: "memory");
     const int g = lane >> 4, n = lane & 15;
-    const uint32_t prow = pbuf + ((n & (REPP - 1)) * kWave + 4 * g) * 2;
+    const uint32_t prow = pbuf + ((n < REPP ? n : 0) * kWave + 4 * g) * 2;      // columns past the last head: any row, never stored
 #pragma unroll
     for (int tb = 0; tb < 4; tb++) {
         const __attribute__((address_space(3))) uint2* pp = lds_ptr<__attribute__((address_space(3))) uint2>(prow + tb * 32);

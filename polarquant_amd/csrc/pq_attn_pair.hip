@@ -22,6 +22,10 @@
 #include "pq_attn_device.h"
 #include "pq_phase_timers.h"
 
+#ifndef PQ_DTYPE
+#error "compile with -DPQ_DTYPE=0 (float16) or 1 (bfloat16)"
+#endif
+
 namespace pq {
 
 #pragma clang diagnostic push
@@ -336,7 +340,7 @@ template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer,
                                                                               int* __restrict__ status, uint16_t* __restrict__ direct_out) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
+    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[kPairsPerBlock][REPP * kWave];
     __shared__ int flag_mem[kPairsPerBlock][4];
@@ -386,7 +390,7 @@ template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total, int silent_scorer,
                                                                                        int* __restrict__ status) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
+    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[kPairsPerBlock][REPP * kWave];
     __shared__ int flag_mem[kPairsPerBlock][4];
@@ -456,10 +460,14 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
             PQ_LAUNCH_PAIR_P(REPP, false);                                                                           \
         }                                                                                                            \
     } while (0)
-    switch (rep_pad(rep)) {
+    switch (rep) {                // every ratio has its own instantiation: no padded head costs LDS reads or FMAs
         case 1: PQ_LAUNCH_PAIR(1); break;
         case 2: PQ_LAUNCH_PAIR(2); break;
+        case 3: PQ_LAUNCH_PAIR(3); break;
         case 4: PQ_LAUNCH_PAIR(4); break;
+        case 5: PQ_LAUNCH_PAIR(5); break;
+        case 6: PQ_LAUNCH_PAIR(6); break;
+        case 7: PQ_LAUNCH_PAIR(7); break;
         default: PQ_LAUNCH_PAIR(8); break;
     }
 #undef PQ_LAUNCH_PAIR
@@ -468,21 +476,22 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
     return static_cast<int>(hipGetLastError());
 }
 
-template <typename T>
-int launch_pair_t(const AttnArgs& a, int total, hipStream_t st) {
+}  // namespace
+
+// `total`: slices (even split: n_splits * B * Nk) or segments (balanced slices: what the device holds at once), one pair each
+#if PQ_DTYPE == 0
+int launch_attn_pair_f16(const AttnArgs& a, int total, hipStream_t st) {
+    using T = F16;
+#else
+int launch_attn_pair_bf16(const AttnArgs& a, int total, hipStream_t st) {
+    using T = BF16;
+#endif
     switch (a.tbits) {
         case 1: return launch_pair_tb<T, 1>(a, total, st);
         case 2: return launch_pair_tb<T, 2>(a, total, st);
         case 3: return launch_pair_tb<T, 3>(a, total, st);
         default: return launch_pair_tb<T, 4>(a, total, st);
     }
-}
-
-}  // namespace
-
-// `total`: slices (even split: n_splits * B * Nk) or segments (balanced slices: what the device holds at once), one pair each
-int launch_attn_pair(const AttnArgs& a, int total, hipStream_t st) {
-    return a.dtype == 0 ? launch_pair_t<F16>(a, total, st) : launch_pair_t<BF16>(a, total, st);
 }
 
 }  // namespace pq

@@ -87,31 +87,39 @@ __device__ __forceinline__ float readlane_f(float v, int lane) {
     return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
 }
 
-// Geometry of the per-wave lookup table for TB angle bits and REPP (1,2,4,8)
-// padded query heads.  An entry holds min(REPP,4) floats; REPP == 8 keeps two
-// tables ("halves") of 4-float entries.  Within pair d the entry of angle bin
-// theta sits at slot theta ^ (d & (NB-1)): the XOR spreads the 64 lanes of the
-// build phase (lane == d, fixed theta) over all banks, and is undone for free in
-// the tile loop by XOR-ing four codes at a time with a compile-time constant.
+// Geometry of the per-wave lookup table for TB angle bits and REPP (1..8) query heads per KV head.
+// An entry holds the first min(REPP, 4) heads; with more than 4 heads a second table ("half") of the
+// same geometry holds the others, REPP - 4 floats per entry: a lookup reads exactly the heads that
+// exist (ds_read_b32 / b64 / b96 / b128), no padded head costs LDS bandwidth or a multiply-add.
+// Entries are 4 (one head), 8 (two) or 16 bytes apart.  Within pair d the entry of angle bin theta sits
+// at slot theta ^ (d & (NB-1)): the XOR spreads the 64 lanes of the build phase (lane == d, fixed
+// theta) over all banks, and is undone in the tile loop by XOR-ing four codes at a time with a
+// compile-time constant.
 template <int TB, int REPP>
 struct Lut {
+    static_assert(REPP >= 1 && REPP <= 8, "1..8 query heads per KV head");
     static constexpr int NB = 1 << TB;
-    static constexpr int ENTRY = REPP < 4 ? REPP : 4;
-    static constexpr int HALVES = REPP / ENTRY;
-    static constexpr int EB = ENTRY * 4;          // entry bytes
-    static constexpr int SH = ENTRY == 1 ? 2 : (ENTRY == 2 ? 3 : 4);
+    static constexpr int W0 = REPP < 4 ? REPP : 4;        // heads in the first half's entries
+    static constexpr int W1 = REPP - W0;                  // heads in the second half's entries (0: no second half)
+    static constexpr int HALVES = W1 > 0 ? 2 : 1;
+    static constexpr int EB = REPP == 1 ? 4 : (REPP == 2 ? 8 : 16);   // entry stride in bytes
+    static constexpr int SH = REPP == 1 ? 2 : (REPP == 2 ? 3 : 4);
     static constexpr int PB = NB * EB;            // bytes per pair
     static constexpr int HB = kPairs * PB;        // bytes per half
     static constexpr int BYTES = HALVES * HB;
-    static_assert(TB + SH <= 8, "theta*entry_bytes must fit a byte");
+    // theta * EB fits a byte: the four byte offsets of a code word are made by two instructions on the
+    // whole word; beyond that (TB 5, 6 with 16-byte entries) each code's offset is shifted into place
+    static constexpr bool PACKED_OFFSETS = TB + SH <= 8;
 };
 
 // LDS is addressed with 32-bit byte addresses in address space 3 so that the
 // compiler emits ds_read_b128/ds_write_b128 with the pair offset folded into
 // the instruction's immediate offset field.
 struct __attribute__((aligned(16))) Entry4 { float x, y, z, w; };
+struct __attribute__((aligned(16))) Entry3 { float x, y, z; };
 struct __attribute__((aligned(8))) Entry2 { float x, y; };
 typedef __attribute__((address_space(3))) Entry4 lds_e4;
+typedef __attribute__((address_space(3))) Entry3 lds_e3;
 typedef __attribute__((address_space(3))) Entry2 lds_e2;
 typedef __attribute__((address_space(3))) float lds_f1;
 typedef __attribute__((address_space(3))) void lds_void;
@@ -124,6 +132,38 @@ __device__ __forceinline__ P* lds_ptr(uint32_t addr) { return (P*)(addr); }
 
 __device__ __forceinline__ uint32_t lds_addr(void* p) {
     return (uint32_t)(uintptr_t)((lds_void*)p);
+}
+
+// W (1..4) consecutive floats of a table entry at LDS byte address `addr`, as one ds_read / ds_write of that width
+template <int W>
+__device__ __forceinline__ void lds_load_w(uint32_t addr, float* e) {
+    if constexpr (W == 1) {
+        e[0] = *lds_ptr<lds_f1>(addr);
+    } else if constexpr (W == 2) {
+        const lds_e2* p = lds_ptr<lds_e2>(addr);
+        e[0] = p->x; e[1] = p->y;
+    } else if constexpr (W == 3) {
+        const lds_e3* p = lds_ptr<lds_e3>(addr);
+        e[0] = p->x; e[1] = p->y; e[2] = p->z;
+    } else {
+        const lds_e4* p = lds_ptr<lds_e4>(addr);
+        e[0] = p->x; e[1] = p->y; e[2] = p->z; e[3] = p->w;
+    }
+}
+template <int W>
+__device__ __forceinline__ void lds_store_w(uint32_t addr, const float* e) {
+    if constexpr (W == 1) {
+        *lds_ptr<lds_f1>(addr) = e[0];
+    } else if constexpr (W == 2) {
+        lds_e2* p = lds_ptr<lds_e2>(addr);
+        p->x = e[0]; p->y = e[1];
+    } else if constexpr (W == 3) {
+        lds_e3* p = lds_ptr<lds_e3>(addr);
+        p->x = e[0]; p->y = e[1]; p->z = e[2];
+    } else {
+        lds_e4* p = lds_ptr<lds_e4>(addr);
+        p->x = e[0]; p->y = e[1]; p->z = e[2]; p->w = e[3];
+    }
 }
 
 // sin and cos of a bin-centre angle.  Three-constant Cody-Waite reduction by
@@ -152,7 +192,7 @@ __device__ __forceinline__ void sincos_bin(float x, float* sn, float* cs) {
 }
 
 // Build the table for one group.  lane == pair d.
-//   qx[j], qy[j]: q_j[d], q_j[d+64] (0 for padded heads)
+//   qx[j], qy[j]: q_j[d], q_j[d+64]
 //   returns c_d for this lane's pair.
 template <typename T, int TB, int REPP>
 __device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (&qx)[REPP], const float (&qy)[REPP],
@@ -177,18 +217,8 @@ __device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (
 #pragma unroll
         for (int j = 0; j < REPP; j++) e[j] = __builtin_fmaf(ax[j], c, ay[j] * s);
         const uint32_t off = base ^ (k << L::SH);
-        if constexpr (L::ENTRY == 1) {
-            *lds_ptr<lds_f1>(off) = e[0];
-        } else if constexpr (L::ENTRY == 2) {
-            lds_e2* p = lds_ptr<lds_e2>(off);
-            p->x = e[0]; p->y = e[1];
-        } else {
-#pragma unroll
-            for (int h = 0; h < L::HALVES; h++) {
-                lds_e4* p = lds_ptr<lds_e4>(off + h * L::HB);
-                p->x = e[h * 4]; p->y = e[h * 4 + 1]; p->z = e[h * 4 + 2]; p->w = e[h * 4 + 3];
-            }
-        }
+        lds_store_w<L::W0>(off, e);
+        if constexpr (L::W1 > 0) lds_store_w<L::W1>(off + L::HB, e + 4);
         const float c2 = __builtin_fmaf(c, cd, -(s * sd));
         const float s2 = __builtin_fmaf(s, cd, c * sd);
         c = c2; s = s2;
@@ -217,31 +247,25 @@ __device__ __forceinline__ void score_token(uint32_t lut, const uint32_t (&codes
         static_for<BW>([&](auto CC) {
             constexpr int cc = decltype(CC)::value, c = bi * BW + cc;
             const uint32_t w = codes[c];
-            // byte i of kc: XOR pattern of pair 4c+i, already scaled to bytes
-            constexpr uint32_t kc = ((uint32_t)(((4 * c + 0) & nbm) << L::SH)) | ((uint32_t)(((4 * c + 1) & nbm) << L::SH) << 8) |
-                                    ((uint32_t)(((4 * c + 2) & nbm) << L::SH) << 16) | ((uint32_t)(((4 * c + 3) & nbm) << L::SH) << 24);
-            uint32_t a4 = ((w & TM4) << L::SH) ^ kc;   // byte i: LDS byte offset of theta_i inside pair 4c+i
-            uint32_t r4 = (w >> TB) & RM4;             // byte i: rho_i
+            // byte i of ks: XOR pattern (slot swizzle) of pair 4c+i
+            constexpr uint32_t ks = ((uint32_t)((4 * c + 0) & nbm)) | ((uint32_t)((4 * c + 1) & nbm) << 8) |
+                                    ((uint32_t)((4 * c + 2) & nbm) << 16) | ((uint32_t)((4 * c + 3) & nbm) << 24);
+            uint32_t a4, r4 = (w >> TB) & RM4;         // r4 byte i: rho_i
+            if constexpr (L::PACKED_OFFSETS) {
+                a4 = ((w & TM4) ^ ks) << L::SH;        // byte i: LDS byte offset of theta_i inside pair 4c+i
+            } else {
+                a4 = (w & TM4) ^ ks;                   // byte i: swizzled slot of theta_i, shifted into place per code
+            }
             // keep the packed forms: byte i is then picked by v_bfe_u32 / v_cvt_f32_ubyte<i>
             asm volatile("" : "+v"(a4), "+v"(r4));
             r4s[buf][cc] = r4;
             static_for<4>([&](auto II) {
                 constexpr int i = decltype(II)::value, d = 4 * c + i;
-                const uint32_t off = (a4 >> (8 * i)) & 0xFFu;
+                uint32_t off = (a4 >> (8 * i)) & 0xFFu;
+                if constexpr (!L::PACKED_OFFSETS) off <<= L::SH;
                 const uint32_t addr = lut + off + d * L::PB;
-                if constexpr (L::ENTRY == 1) {
-                    e[buf][cc * 4 + i][0] = *lds_ptr<lds_f1>(addr);
-                } else if constexpr (L::ENTRY == 2) {
-                    const lds_e2* p = lds_ptr<lds_e2>(addr);
-                    e[buf][cc * 4 + i][0] = p->x; e[buf][cc * 4 + i][1] = p->y;
-                } else {
-                    static_for<L::HALVES>([&](auto HH) {
-                        constexpr int h = decltype(HH)::value;
-                        const lds_e4* p = lds_ptr<lds_e4>(addr + h * L::HB);
-                        e[buf][cc * 4 + i][h * 4] = p->x; e[buf][cc * 4 + i][h * 4 + 1] = p->y;
-                        e[buf][cc * 4 + i][h * 4 + 2] = p->z; e[buf][cc * 4 + i][h * 4 + 3] = p->w;
-                    });
-                }
+                lds_load_w<L::W0>(addr, &e[buf][cc * 4 + i][0]);
+                if constexpr (L::W1 > 0) lds_load_w<L::W1>(addr + L::HB, &e[buf][cc * 4 + i][4]);
             });
         });
     };

@@ -66,16 +66,30 @@ struct AttnArgs {
     float* workspace;
     void* out;
 };
+// pq_attn_common.hip: picks the kernel family and the grid, then calls one of the four launchers below
 int launch_attn_partials(const AttnArgs& a, hipStream_t st);
-// the default kernels for half-precision values (pq_attn_pair.hip); called by launch_attn_partials
-int launch_attn_pair(const AttnArgs& a, int total, hipStream_t st);
 int launch_attn_merge(const float* ws, int B, int N, int n_splits, int dtype, void* out, hipStream_t st);
+// The attention kernels are compiled once per key / value dtype (-DPQ_DTYPE=0: float16, 1: bfloat16), each into an
+// object of its own, so that the two halves of the instantiations build side by side.  `total`: slices (even split:
+// n_splits * B * Nk) or segments (balanced slices: what the device holds at once).
+//   pq_attn_pair.hip: a scorer / accumulator pair of wavefronts per slice, the default for half-precision values
+int launch_attn_pair_f16(const AttnArgs& a, int total, hipStream_t st);
+int launch_attn_pair_bf16(const AttnArgs& a, int total, hipStream_t st);
+//   pq_attn.hip: one wavefront per slice (PQ_SINGLE_WAVEFRONT, 4-bit values, more than 16 angle bins)
+int launch_attn_one_f16(const AttnArgs& a, int total, hipStream_t st);
+int launch_attn_one_bf16(const AttnArgs& a, int total, hipStream_t st);
 
 // Device address, on the current device, of the library's own buffer for split partials
 // (kStaticMaxPartials partials of 132 floats); 0 or a hipError_t.
 constexpr int kStaticMaxPartials = 16384;
 int attn_static_scratch(float** ptr);
 
+// The one-wavefront kernels are instantiated for 1, 2, 4 and 8 query heads per KV head and run other ratios with the
+// next of those (the heads that do not exist are zero queries whose results are dropped); the paired kernels and the
+// score op are instantiated for every ratio 1..8.
 inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 : 8; }
+// More than 16 angle bins (tbits 5, 6): the table is 32-128 KiB, too large for the four tables of a paired workgroup;
+// those bit widths run the one-wavefront kernels.
+constexpr int kMaxPairTbits = 4;
 
 }  // namespace pq

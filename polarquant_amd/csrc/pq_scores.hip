@@ -12,7 +12,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) v
                                                        const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
                                                        float* __restrict__ out, int N, int Nk, int Nb, int rep) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(16))) char lut_mem[L::BYTES];
+    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[L::BYTES];
     const uint32_t lut = lds_addr(lut_mem);
     const int lane = threadIdx.x;
     const int grp = blockIdx.x;
@@ -93,10 +93,14 @@ static int launch_tb(const void* q, const uint8_t* codes, const void* rscale, co
             PQ_LAUNCH_P(REPP, false);                                                                           \
         }                                                                                                       \
     } while (0)
-    switch (rep_pad(rep)) {
+    switch (rep) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;
+        case 3: PQ_LAUNCH(3); break;
         case 4: PQ_LAUNCH(4); break;
+        case 5: PQ_LAUNCH(5); break;
+        case 6: PQ_LAUNCH(6); break;
+        case 7: PQ_LAUNCH(7); break;
         default: PQ_LAUNCH(8); break;
     }
 #undef PQ_LAUNCH
@@ -111,7 +115,9 @@ static int launch_t(const void* q, const uint8_t* codes, const void* rscale, con
         case 1: return launch_tb<T, 1>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
         case 2: return launch_tb<T, 2>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
         case 3: return launch_tb<T, 3>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
-        default: return launch_tb<T, 4>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        case 4: return launch_tb<T, 4>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        case 5: return launch_tb<T, 5>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
+        default: return launch_tb<T, 6>(q, codes, rscale, rmn, tscale, tmn, out, B, N, Nk, Nb, packed6, st);
     }
 }
 

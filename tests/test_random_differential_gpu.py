@@ -15,10 +15,11 @@ pytestmark = pytest.mark.gpu
 # more seeds: PQ_RANDOM_CASES=300; another stretch of them: PQ_RANDOM_FIRST=1000
 SEEDS = range(int(os.environ.get("PQ_RANDOM_FIRST", "0")),
               int(os.environ.get("PQ_RANDOM_FIRST", "0")) + int(os.environ.get("PQ_RANDOM_CASES", "24")))
-HEADS = [(1, 1), (2, 1), (4, 4), (8, 2), (3, 1), (6, 1), (7, 1), (8, 1), (16, 2), (12, 4)]
-BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 4)]
-# dtype -> [attention cases run, cases that needed the widened band, output elements that needed it]
-WIDENED = {"float16": [0, 0, 0], "bfloat16": [0, 0, 0]}
+HEADS = [(1, 1), (2, 1), (4, 4), (8, 2), (3, 1), (6, 1), (7, 1), (8, 1), (16, 2), (12, 4), (5, 1), (10, 2), (14, 2)]
+BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 4), (3, 5), (2, 6), (1, 6)]
+# dtype -> [attention cases run, cases that needed the widened band, output elements that needed it,
+#           worst excess over the STATED bar (rtol 1e-2 / atol 1e-3) against the reference path's literal evaluation alone]
+WIDENED = {"float16": [0, 0, 0, -1.0], "bfloat16": [0, 0, 0, -1.0]}
 
 
 @pytest.mark.parametrize("seed", SEEDS)
@@ -120,6 +121,9 @@ def test_random_decode_attention_case(gpu, seed):
         # (literal, half-precision) evaluation, which is what parity is stated against
         err_lit = (out[b:b + 1].double() - literal).abs()
         needed += int(((err > atol + rtol * exact.abs()) & (err_lit > atol + rtol * literal.abs())).sum())
+        # how far the output sits from the literal reference evaluation alone, in the stated (float16) bar: > 0 means
+        # outside it.  For bfloat16 this is the measured size of the band that dtype needs, instead of a choice.
+        WIDENED[name][3] = max(WIDENED[name][3], float((err_lit - (1e-3 + 1e-2 * literal.abs())).max()))
     WIDENED[name][0] += 1
     WIDENED[name][1] += int(needed > 0)
     WIDENED[name][2] += needed
@@ -132,8 +136,9 @@ def test_random_decode_attention_case(gpu, seed):
 def test_random_widened_band_report(gpu):
     """How many of the attention cases above were inside the stated tolerance only thanks to the allowance for the
     reference path's own half-precision roundings: printed per dtype; for float16 it has to be none."""
-    for name, (cases, cases_needing, elements) in WIDENED.items():
-        print("%s: %d cases, %d needed the widened band (%d output elements)" % (name, cases, cases_needing, elements), flush=True)
+    for name, (cases, cases_needing, elements, excess) in WIDENED.items():
+        print("%s: %d cases, %d needed the widened band (%d output elements); worst excess over rtol 1e-2 / atol 1e-3 against "
+              "the literal reference evaluation alone: %.3e" % (name, cases, cases_needing, elements, excess), flush=True)
     assert WIDENED["float16"][1] == 0
 
 
