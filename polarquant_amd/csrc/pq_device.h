@@ -89,8 +89,8 @@ __device__ __forceinline__ float readlane_f(float v, int lane) {
 
 // Geometry of the per-wave lookup table for TB angle bits and REPP (1..8) query heads per KV head.
 // An entry holds the first min(REPP, 4) heads; with more than 4 heads a second table ("half") of the
-// same geometry holds the others, REPP - 4 floats per entry: a lookup reads exactly the heads that
-// exist (ds_read_b32 / b64 / b96 / b128), no padded head costs LDS bandwidth or a multiply-add.
+// same geometry holds the others, REPP - 4 floats per entry: a lookup reads the heads that exist
+// (ds_read_b32 / b64 / b128; three heads are read as four), and no padded head costs a multiply-add.
 // Entries are 4 (one head), 8 (two) or 16 bytes apart.  Within pair d the entry of angle bin theta sits
 // at slot theta ^ (d & (NB-1)): the XOR spreads the 64 lanes of the build phase (lane == d, fixed
 // theta) over all banks, and is undone in the tile loop by XOR-ing four codes at a time with a
@@ -116,12 +116,12 @@ struct Lut {
 // compiler emits ds_read_b128/ds_write_b128 with the pair offset folded into
 // the instruction's immediate offset field.
 struct __attribute__((aligned(16))) Entry4 { float x, y, z, w; };
-struct __attribute__((aligned(16))) Entry3 { float x, y, z; };
 struct __attribute__((aligned(8))) Entry2 { float x, y; };
 typedef __attribute__((address_space(3))) Entry4 lds_e4;
-typedef __attribute__((address_space(3))) Entry3 lds_e3;
 typedef __attribute__((address_space(3))) Entry2 lds_e2;
 typedef __attribute__((address_space(3))) float lds_f1;
+typedef float float4_v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) float4_v lds_f4;
 typedef __attribute__((address_space(3))) void lds_void;
 
 #pragma clang diagnostic push
@@ -134,7 +134,10 @@ __device__ __forceinline__ uint32_t lds_addr(void* p) {
     return (uint32_t)(uintptr_t)((lds_void*)p);
 }
 
-// W (1..4) consecutive floats of a table entry at LDS byte address `addr`, as one ds_read / ds_write of that width
+// W (1..4) consecutive floats of a table entry at LDS byte address `addr`, as one ds_read / ds_write of that width.
+// Three floats move as four (entries are 16 bytes apart, the fourth word belongs to nobody): a 96-bit LDS access
+// keeps the LDS busy longer than a 128-bit one (measured at 7 heads per KV head, 3-bit angles, ragged batch of 64:
+// SQ_LDS_IDX_ACTIVE 22.1 M with ds_read_b96 against 18.7 M with two ds_read_b128 for the same lookups).
 template <int W>
 __device__ __forceinline__ void lds_load_w(uint32_t addr, float* e) {
     if constexpr (W == 1) {
@@ -143,8 +146,8 @@ __device__ __forceinline__ void lds_load_w(uint32_t addr, float* e) {
         const lds_e2* p = lds_ptr<lds_e2>(addr);
         e[0] = p->x; e[1] = p->y;
     } else if constexpr (W == 3) {
-        const lds_e3* p = lds_ptr<lds_e3>(addr);
-        e[0] = p->x; e[1] = p->y; e[2] = p->z;
+        const float4_v v = *lds_ptr<const lds_f4>(addr);           // one 128-bit access; the fourth word is not used
+        e[0] = v.x; e[1] = v.y; e[2] = v.z;
     } else {
         const lds_e4* p = lds_ptr<lds_e4>(addr);
         e[0] = p->x; e[1] = p->y; e[2] = p->z; e[3] = p->w;
@@ -158,8 +161,8 @@ __device__ __forceinline__ void lds_store_w(uint32_t addr, const float* e) {
         lds_e2* p = lds_ptr<lds_e2>(addr);
         p->x = e[0]; p->y = e[1];
     } else if constexpr (W == 3) {
-        lds_e3* p = lds_ptr<lds_e3>(addr);
-        p->x = e[0]; p->y = e[1]; p->z = e[2];
+        lds_e4* p = lds_ptr<lds_e4>(addr);
+        p->x = e[0]; p->y = e[1]; p->z = e[2]; p->w = 0.0f;
     } else {
         lds_e4* p = lds_ptr<lds_e4>(addr);
         p->x = e[0]; p->y = e[1]; p->z = e[2]; p->w = e[3];

@@ -7,7 +7,7 @@
 namespace pq {
 
 template <typename T, int TB, int REPP, bool PK6>
-__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2, 4))) void scores_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
+__global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(Lut<TB, REPP>::BYTES > 40960 ? 1 : 2, 4))) void scores_kernel(const uint16_t* __restrict__ q, const uint8_t* __restrict__ codes,
                                                        const uint16_t* __restrict__ rscale, const uint16_t* __restrict__ rmn,
                                                        const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
                                                        float* __restrict__ out, int N, int Nk, int Nb, int rep) {
