@@ -106,7 +106,7 @@ typedef enum { PQ_F16 = 0, PQ_BF16 = 1 } pq_dtype;
                                         the failing pair worked on are NaN */
 
 /* Test hook of pq_decode_attn / _partials / _static (scorer / accumulator kernels only; refused together with
- * PQ_SINGLE_WAVEFRONT and by the 4-bit-value entry point, whose kernels have no hand-over): the scorers publish nothing,
+ * PQ_SINGLE_WAVEFRONT, whose kernels have no hand-over, and by the 4-bit-value entry point): the scorers publish nothing,
  * and the bounded waits of the hand-over give up after 1000 polls instead of 2^22.  Every kernel still ends normally;
  * every output of the call is NaN and the status word is set.  For the test that a hand-over which fails can neither
  * hang the GPU nor pass for a result.  ONLY the test build of the library (compiled with -DPQ_TEST_HOOKS:
@@ -358,6 +358,9 @@ int pq_decode_attn_static(const void *q,
  * [B,Nk,resid_capacity,128] holds the half-precision values of the residual
  * window only, row r belonging to residual key r (:238).  Keys and values
  * share the window's fill (n_resid) and are flushed together (:207,:243).
+ * flags, status: as for pq_decode_attn.  The kernels for 4-bit values run one wavefront per slice whatever
+ * the flags say; PQ_SINGLE_WAVEFRONT and `status` matter only while no group has been quantized yet, when the
+ * call is served by the half-precision-value kernels over the residual window.
  * ------------------------------------------------------------------------- */
 int pq_quantize_values(const void *v, const int64_t *v_strides, int dtype, int B, int Nk, int T,
                        int32_t *codes, void *scale, void *zero,
@@ -377,7 +380,7 @@ int pq_decode_attn_v4(const void *q,
                       const uint8_t *mask, int64_t mask_stride,
                       float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                       int n_splits, int min_groups_per_split, void *workspace, size_t workspace_bytes,
-                      void *out, unsigned flags, void *stream);
+                      void *out, unsigned flags, int32_t *status, void *stream);
 
 /* RoPE over whole sequences, the prompt pass's `apply_rotary_pos_emb(query_states, key_states, cos, sin)`
  * (models/modeling_llama_polar.py:56-59) in one launch, bit-identical to the eager

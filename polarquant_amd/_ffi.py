@@ -61,7 +61,7 @@ SIGNATURES = {
     "pq_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                    c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                    c_void_p, c_int64, c_float]
-                          + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p]),
+                          + [c_int] * 8 + [c_void_p, c_size_t, c_void_p, c_uint, c_void_p, c_void_p]),
     "pq_validate_decode_attn_v4": (c_int, [c_void_p] * 6 + [c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p,
                                                             c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                                             c_void_p, c_int64, c_float]

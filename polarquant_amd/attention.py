@@ -191,9 +191,11 @@ def polar_decode_attention_v4(
     n_groups_per_seq: Optional[torch.Tensor] = None, n_resid_per_seq: Optional[torch.Tensor] = None,
     n_splits: Optional[int] = None, out: Optional[torch.Tensor] = None, min_groups_per_split: int = 0,
     workspace: Optional[torch.Tensor] = None, balanced: bool = False, total_groups: Optional[int] = None,
+    single_wavefront: bool = False, status: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Decode attention of the reference's Mixed variant (polar keys + 4-bit values,
-    models/modeling_llama_polar.py:185-241) -> [B,N,1,128] in the query dtype."""
+    models/modeling_llama_polar.py:185-241) -> [B,N,1,128] in the query dtype.
+    `single_wavefront`, `status`: as for polar_decode_attention."""
     if not query_states.is_cuda:
         raise RuntimeError("polarquant_amd: decode attention needs tensors on the GPU (no CPU fallback)")
     dev = query_states.device
@@ -226,12 +228,19 @@ def polar_decode_attention_v4(
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(hd)
     max_groups = g_cap if n_groups_per_seq is not None else n_groups
+    if single_wavefront:
+        flags |= _ffi.PQ_SINGLE_WAVEFRONT
     if balanced:
         flags |= _ffi.PQ_BALANCED_SLICES
         if n_splits is None:
             n_splits = balanced_slots(B, Nk, max_groups, total_groups, (8 if N // Nk <= 4 else 4) * _num_cus(dev), r_cap)
     if n_splits is None:
         n_splits = _ffi.lib().pq_decode_attn_v4_plan(B, N, Nk, max(max_groups, 1), _num_cus(dev))
+    sptr = None
+    if status is not None:
+        if status.dtype != torch.int32 or status.device != dev or status.numel() != 1:
+            raise ValueError("polarquant_amd: status must be one int32 on %s" % dev)
+        sptr = status.data_ptr()
     ws = _pick_workspace(workspace, B, N, n_splits, dev)
     if out is None:
         out = torch.empty((B, N, 1, hd), dtype=query_states.dtype, device=dev)
@@ -241,6 +250,6 @@ def polar_decode_attention_v4(
         rc = _ffi.lib().pq_decode_attn_v4(
             q.data_ptr(), *cptr, g_cap, n_groups, gps, key_resid.data_ptr(), r_cap, n_resid, rps,
             value_resid.data_ptr(), *vptr, v4_cap, mptr, mstride, float(sm_scale), B, N, Nk, rbits, tbits, dt,
-            n_splits, min_groups_per_split, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, _stream_ptr(dev))
+            n_splits, min_groups_per_split, ws.data_ptr(), ws.numel() * 4, out.data_ptr(), flags, sptr, _stream_ptr(dev))
     _ffi.check(rc, "pq_decode_attn_v4")
     return out

@@ -1,6 +1,8 @@
 """Build recipe of the HIP library: hipcc for gfx950, in-tree.
 
-    python -m polarquant_amd.build            # (re)build polarquant_amd/libpolarquant_hip.so and libpolarquant_bench.so
+    python -m polarquant_amd.build                    # (re)build polarquant_amd/libpolarquant_hip.so, its test build and libpolarquant_bench.so
+    python -m polarquant_amd.build --phase-timers     # the measuring build (benchmarks/phase_timing.py)
+    python -m polarquant_amd.build --probe no_values  # a probe build (benchmarks/probe_bench.py)
 
 hipcc cross-compiles without a GPU.  Flags that matter:
   -ffp-contract=off            the quantizer reproduces eager half-precision torch
@@ -72,6 +74,27 @@ def _link(objs, lib: str) -> None:
     os.replace(tmp, lib)
 
 
+# probe builds: the library with one unit compiled for a timing-only experiment (results wrong on purpose); loaded by
+# polarquant_amd/benchmarks/probe_bench.py only
+PROBE_LIB = os.path.join(HERE, "libpolarquant_hip_probe.so")
+PROBES = {"no_values": {("pq_attn.hip", ".f16"): ("pq_attn.hip", ("PQ_DTYPE=0", "PQ_PROBE_NO_VALUES"), ".f16.no_values")}}
+
+
+def build_probe(name: str, verbose: bool = True) -> str:
+    """libpolarquant_hip_probe.so for probe `name`: the shipping objects (built if missing) with the probe's units
+    recompiled."""
+    os.makedirs(OBJ, exist_ok=True)
+    swap = PROBES[name]
+    units = [swap.get((src, tag), (src, defs, tag)) for src, defs, tag in UNITS]
+    todo = [u for u in units if u in swap.values() or not os.path.exists(os.path.join(OBJ, os.path.splitext(u[0])[0] + u[2] + ".o"))]
+    with ThreadPoolExecutor(max_workers=min(8, max(len(todo), 1))) as ex:
+        list(ex.map(lambda j: _compile(*j), todo))
+    _link([os.path.join(OBJ, os.path.splitext(u[0])[0] + u[2] + ".o") for u in units], PROBE_LIB)
+    if verbose:
+        print("built", PROBE_LIB, "(probe %s)" % name)
+    return PROBE_LIB
+
+
 def build(verbose: bool = True, phase_timers: bool = False) -> str:
     """The library the package loads; or, with phase_timers, a second library (same ABI, not loaded by default)
     whose attention kernel times its phases with the wall clock and prints them: a measuring build for
@@ -102,4 +125,7 @@ def build(verbose: bool = True, phase_timers: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    build(phase_timers="--phase-timers" in sys.argv[1:])
+    if "--probe" in sys.argv[1:]:
+        build_probe(sys.argv[sys.argv.index("--probe") + 1])
+    else:
+        build(phase_timers="--phase-timers" in sys.argv[1:])

@@ -176,7 +176,9 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
             const uint32_t voff_q = static_cast<uint32_t>(lane >> 4) * 64 + static_cast<uint32_t>(lane & 15) * 4;
             uint16_t vsz[2][2] = {{0, 0}, {0, 0}};             // (scale, zero-point) words of this lane's token, by tile parity
             auto load_values = [&](int buf, uint32_t tile_tok, bool in_range) {
-                if constexpr (V4) {
+                if constexpr (V4 && kProbeNoValues) {
+                    return;                                    // probe build: the 4-bit-value kernel without its value path
+                } else if constexpr (V4) {
                     load_v4_tile(vv[buf].r, rq, voff_q, in_range ? tile_tok * 64u : 0xFFFF0000u);
                     const int so = in_range ? static_cast<int>(tile_tok * 2u) : static_cast<int>(0x7FFFFF00);
                     vsz[buf][0] = __builtin_amdgcn_raw_buffer_load_b16(rvs, lane * 2, so, 0);
@@ -251,7 +253,9 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
                     const bool keep = has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, static_cast<int>(tok0), 0) != 0) : true;
 #pragma unroll
                     for (int j = 0; j < REPP; j++) s[j] = keep ? s[j] * scale_log2 : -INFINITY;
-                    if constexpr (V4) {
+                    if constexpr (V4 && kProbeNoValues) {
+                        softmax_sums_only<REPP>(st, s, kLazyThresholdV4);
+                    } else if constexpr (V4) {
                         softmax_pv_tile_v4<REPP>(st, s, vv[half].r, lo2f<T>(vsz[half][0]), lo2f<T>(vsz[half][1]), pbuf, lane);
                     } else {
                         softmax_pv_tile<T, REPP>(st, s, vv[half].r, pbuf, lane);

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(kHeadDim * G) void merge_kernel(const float* __rest
         __syncthreads();
         for (int s = tid; s < cnt; s += NT) {
             const float m = p[static_cast<size_t>(s0 + s) * kPartialFloats];
-            const float w = (m == -INFINITY) ? 0.0f : exp2f(m - M);
+            const float w = (m == -INFINITY) ? 0.0f : exp2_raw(m - M);
             wgt[s] = w;
             // an empty slice contributes nothing, whatever its sum word holds
             den = w != 0.0f ? __builtin_fmaf(w, p[static_cast<size_t>(s0 + s) * kPartialFloats + 1], den) : den;
@@ -99,7 +99,9 @@ static int device_compute_units() {
 
 int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
     const int rep = a.N / a.Nk;
-    // half-precision values and at most 16 angle bins: a scorer / accumulator pair of wavefronts per slice or segment
+    // half-precision values and at most 16 angle bins: a scorer / accumulator pair of wavefronts per slice or segment.
+    // (4-bit values stay with one wavefront per slice, two per SIMD: a paired form of that kernel at four wavefronts per
+    // SIMD was measured no faster -- the vector ALU's total work bounds it, however it is spread over wavefronts.)
     const bool pairs = !a.v4_codes && !a.single_wave && a.tbits <= kMaxPairTbits;
     long long total = static_cast<long long>(a.n_splits) * a.B * a.Nk;
     if (a.balanced) {

@@ -24,6 +24,11 @@ template <> __device__ __forceinline__ floatx4 mfma16<BF16>(uint2 a, uint2 b, fl
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0, 0, 0);
 }
 
+// 2^x as the bare v_exp_f32: exact to 1 ulp over the normal range and 0 below 2^-126, where the library's exp2f spends
+// five more instructions to return a denormal.  Every use here is a softmax weight relative to a running maximum: a
+// weight below 2^-126 is nothing against the maximum's weight of at least 2^-8.
+__device__ __forceinline__ float exp2_raw(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
@@ -61,7 +66,7 @@ __device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[
 #pragma unroll
         for (int j = 0; j < REPP; j++) {
             const float mn = fmaxf(st.m[j], wave_max(t[j]));
-            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2f(st.m[j] - mn);
+            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2_raw(st.m[j] - mn);
             st.m[j] = mn;
             st.l[j] *= alpha[j];
         }
@@ -74,7 +79,7 @@ __device__ __forceinline__ void softmax_pv_tile(AttnState<REPP>& st, float (&t)[
 #pragma unroll
     for (int j = 0; j < REPP; j++) {
         const float ms = (st.m[j] == -INFINITY) ? 0.0f : st.m[j];
-        const float p = exp2f(t[j] - ms);
+        const float p = exp2_raw(t[j] - ms);
         st.l[j] += p;
         *lds_ptr<__attribute__((address_space(3))) uint16_t>(pbuf + (j * kWave + lane) * 2) = f2lo<T>(p);
     }
@@ -141,7 +146,7 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
 #pragma unroll
         for (int j = 0; j < REPP; j++) {
             const float mn = fmaxf(st.m[j], wave_max(t[j]));
-            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2f(st.m[j] - mn);
+            alpha[j] = (mn == -INFINITY) ? 1.0f : exp2_raw(st.m[j] - mn);
             st.m[j] = mn;
             st.l[j] *= alpha[j];
             st.zp[j] *= alpha[j];
@@ -159,11 +164,13 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
     // its rounding error (2^-11) would leave an error of that size times ~3 when one token dominates.
     // A constant row has scale 0 and all codes 0: any scale serves, take 1.
     const float scp = sc == 0.0f ? 1.0f : sc;
-    const float zq = zp / scp;
+    // (a reciprocal to 1 ulp instead of the ten-instruction IEEE division: what matters is that both terms see the same
+    // rounded weight, not the last bit of zero / scale)
+    const float zq = zp * __builtin_amdgcn_rcpf(scp);
 #pragma unroll
     for (int j = 0; j < REPP; j++) {
         const float ms = (st.m[j] == -INFINITY) ? 0.0f : st.m[j];
-        const float p = exp2f(t[j] - ms);
+        const float p = exp2_raw(t[j] - ms);
         st.l[j] += p;
         const uint16_t wh = f2lo<F16>(p * scp);
         st.zp[j] = __builtin_fmaf(lo2f<F16>(wh), zq, st.zp[j]);
@@ -194,6 +201,25 @@ __device__ __forceinline__ void softmax_pv_tile_v4(AttnState<REPP>& st, float (&
     }
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+}
+
+// Probe builds only: the softmax bookkeeping of a tile (running maximum, probabilities, their sum) without any
+// product with the values.
+template <int REPP>
+__device__ __forceinline__ void softmax_sums_only(AttnState<REPP>& st, float (&t)[REPP], float lazy) {
+    bool raise = false;
+#pragma unroll
+    for (int j = 0; j < REPP; j++) raise |= t[j] > st.m[j] + lazy;
+    if (__any(raise)) {
+#pragma unroll
+        for (int j = 0; j < REPP; j++) {
+            const float mn = fmaxf(st.m[j], wave_max(t[j]));
+            st.l[j] *= (mn == -INFINITY) ? 1.0f : exp2_raw(st.m[j] - mn);
+            st.m[j] = mn;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < REPP; j++) st.l[j] += exp2_raw(t[j] - ((st.m[j] == -INFINITY) ? 0.0f : st.m[j]));
 }
 
 // After the last 4-bit tile: accumulators back to real units, plus the zero-point term (the same

@@ -24,9 +24,8 @@ int check_decode_flags(unsigned flags, int rbits, int tbits, Entry entry = Entry
     // the score op has one slice per group; only the attention entry points cut the context
     unsigned known = PQ_CODES_PACKED6;
     if (entry != Entry::Scores) known |= PQ_BALANCED_SLICES;
-    // 4-bit values always run one wavefront per slice: the flag that asks for it, and the hook into the hand-over
-    // that those kernels do not have, mean nothing there
-    if (entry == Entry::Attention) known |= PQ_SINGLE_WAVEFRONT;
+    if (entry != Entry::Scores) known |= PQ_SINGLE_WAVEFRONT;
+    // (the test hook exists for the entry points with half-precision values only)
 #ifdef PQ_TEST_HOOKS
     if (entry == Entry::Attention && !(flags & PQ_SINGLE_WAVEFRONT)) known |= PQ_TEST_SILENT_SCORER;
 #endif
@@ -559,13 +558,14 @@ int pq_decode_attn_v4(const void* q,
                       const uint8_t* mask, int64_t mask_stride,
                       float sm_scale, int B, int N, int Nk, int rbits, int tbits, int dtype,
                       int n_splits, int min_groups_per_split, void* workspace, size_t workspace_bytes,
-                      void* out, unsigned flags, void* stream) {
+                      void* out, unsigned flags, int32_t* status, void* stream) {
     if (int rc = pq_validate_decode_attn_v4(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups,
                                             n_groups_per_seq, k_resid, resid_capacity, n_resid, n_resid_per_seq,
                                             v_resid, v_codes, v_scale, v_zero, v4_capacity, mask, mask_stride, sm_scale,
                                             B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,
                                             workspace_bytes, out, flags))
         return rc;
+    if (status && !aligned(status, 4)) return PQ_ERR_MISALIGNED;
     const bool any_groups = n_groups_per_seq ? group_capacity > 0 : n_groups > 0;
     pq::AttnArgs a;
     a.q = q; a.codes = codes; a.rscale = rscale; a.rmn = rmn; a.tscale = tscale; a.tmn = tmn;
@@ -576,6 +576,8 @@ int pq_decode_attn_v4(const void* q,
     a.min_groups_per_split = min_groups_per_split;
     a.packed6 = (flags & PQ_CODES_PACKED6) != 0;
     a.balanced = (flags & PQ_BALANCED_SLICES) != 0;
+    a.single_wave = (flags & PQ_SINGLE_WAVEFRONT) != 0;
+    a.status = status;
     a.workspace = static_cast<float*>(workspace); a.out = nullptr;
     if (any_groups) {
         a.v = v_resid; a.v_capacity = resid_capacity;      // residual rows only, row 0 = first residual token

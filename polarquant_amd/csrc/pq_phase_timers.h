@@ -3,6 +3,17 @@
 // polarquant_amd/benchmarks/phase_timing.py).  In the shipping build every macro below expands to nothing.
 #pragma once
 
+// ---- probe builds (timing only: their results are wrong on purpose) ----
+// -DPQ_PROBE_NO_VALUES (`python -m polarquant_amd.build --probe no_values` -> libpolarquant_hip_probe.so, timed by
+// polarquant_amd/benchmarks/probe_bench.py): the 4-bit-value kernels without their value path -- no value loads, no
+// nibble unpacking, no matrix products, no zero-point term; codes, tables, scores, mask and the softmax sums remain.
+// What is left is the floor the score side alone sets for that kernel.
+#ifdef PQ_PROBE_NO_VALUES
+constexpr bool kProbeNoValues = true;
+#else
+constexpr bool kProbeNoValues = false;
+#endif
+
 // ---- one wavefront per slice (pq_attn.hip) ----
 // Measuring build only (-DPQ_ATTN_PHASE_TIMERS, `python -m polarquant_amd.build --phase-timers`): wall-clock
 // (100 MHz) time of each phase of the group loop, summed per wavefront and printed by a few of them.

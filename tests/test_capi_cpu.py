@@ -217,9 +217,10 @@ def test_validate_value_quantizer_and_v4_attention(lib, hooks_lib):
     assert bad4(13, P + 8) == -5
     a = list(ok); a[1:6] = [None] * 5; a[6] = 0; a[7] = 0; a[14:17] = [None] * 3; a[17] = 0
     assert lib.pq_validate_decode_attn_v4(*a) == 0            # nothing quantized yet
-    # the 4-bit-value kernels always run one wavefront per slice: the flag that asks for that form, and the test hook
-    # into the hand-over those kernels do not have, are refused instead of silently ignored (in the test build too)
-    assert bad4(32, 16) == 0 and bad4(32, 32) == -2 and bad4(32, 0x40000000) == -2
+    # balanced slices and the choice of the kernel form as for half-precision values; the test hook into the hand-over
+    # exists for the half-precision-value entry points only and is refused here instead of silently ignored (in the test
+    # build too)
+    assert bad4(32, 16) == 0 and bad4(32, 32) == 0 and bad4(32, 0x40000000) == -2
     a = list(ok); a[32] = 0x40000000
     assert hooks_lib.pq_validate_decode_attn_v4(*a) == -2
     # two wavefronts per SIMD for up to 4 query heads per KV head, one beyond

@@ -97,7 +97,7 @@ def test_random_decode_attention_case(gpu, seed):
     cq = [dev(codes)] + [dev(m) for m in meta] if have_groups else [None] * 5
     if values4:
         vq_d = [dev(vcodes)] + [dev(m) for m in vmeta] if have_groups else [None] * 3
-        out = polar_decode_attention_v4(dev(q), *cq, dev(kres), dev(vres), *vq_d, ng, nr, **kw)
+        out = polar_decode_attention_v4(dev(q), *cq, dev(kres), dev(vres), *vq_d, ng, nr, single_wavefront=seed % 4 == 3, **kw)
     else:
         # one case in four takes the one-wavefront-per-slice kernels instead of the scorer / accumulator pairs
         out = polar_decode_attention(dev(q), *cq, dev(kres), dev(vfull), ng, nr, single_wavefront=seed % 4 == 3, **kw)

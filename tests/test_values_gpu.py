@@ -8,11 +8,27 @@ import torch
 
 from oracle import polar_oracle as po
 from polarquant_amd import workloads as wl
-from polarquant_amd.attention import polar_decode_attention_v4
+from polarquant_amd.attention import polar_decode_attention_v4 as _polar_decode_attention_v4
 from polarquant_amd.values import quantize_values
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-2, 1e-3
+
+# Every test of this file runs twice: with the default flags and with PQ_SINGLE_WAVEFRONT, which for this entry point
+# changes the kernels only while nothing has been quantized yet (the residual window alone goes through the
+# half-precision-value kernels: scorer / accumulator pairs, or one wavefront per slice).
+_FORM = {"single": False}
+
+
+@pytest.fixture(autouse=True, params=[False, True], ids=["pairs", "single"])
+def _kernel_form(request):
+    _FORM["single"] = request.param
+    yield
+    _FORM["single"] = False
+
+
+def polar_decode_attention_v4(*args, **kwargs):
+    return _polar_decode_attention_v4(*args, single_wavefront=_FORM["single"], **kwargs)
 
 
 def _same_bits(a, b):
