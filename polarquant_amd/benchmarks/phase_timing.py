@@ -6,7 +6,7 @@ Needs the measuring build of the library (`python -m polarquant_amd.build --phas
 kernel brackets its phases with the 100 MHz wall clock and lets every 97th wavefront print its sums.  The
 instrumentation costs a few percent, so totals are a little above the real kernel's; the split is what matters.
 
-    python -m polarquant_amd.benchmarks.phase_timing [--config 1] [--values4]
+    python -m polarquant_amd.benchmarks.phase_timing [--config 1 | --shape B,N,Nk,L] [--values4] [--pairs] [--pieces]
 
 Phases of one 128-token group: table = build of the per-group angle table in LDS; value_issue = issue of the
 next tile's value loads (16 buffer loads; the time is spent in the issue itself when the compute unit's miss
@@ -34,6 +34,8 @@ PHASES = ("table", "value_issue", "code_wait", "code_issue", "score", "softmax_p
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--config", type=int, default=1)
+    ap.add_argument("--shape", type=str, default=None, help="B,N,Nk,L: a uniform batch of this shape (4/4 bits, float16, random keys "
+                    "quantized on the GPU, one residual key) instead of a benchmark configuration")
     ap.add_argument("--values4", action="store_true")
     ap.add_argument("--even", action="store_true", help="ragged batches: even slices per sequence instead of balanced slices")
     ap.add_argument("--pairs", action="store_true", help="the default kernels instead (a scorer / accumulator pair of wavefronts per slice): "
@@ -47,9 +49,20 @@ def main():
     from ..attention import polar_decode_attention, polar_decode_attention_v4
     from ..values import quantize_values
     dev = torch.device("cuda:0")
-    w = wl.build_workload(args.config, dev)
-    sh = w["shape"]
-    kw = dict(rbits=sh.rbits, tbits=sh.tbits)
+    if args.shape:
+        from ..quantize import quantize_and_pack_nbit
+        B, N, Nk, L = (int(x) for x in args.shape.split(","))
+        g = torch.Generator(device=dev).manual_seed(5)
+        quant = quantize_and_pack_nbit(torch.randn(B, Nk, L, 128, generator=g, device=dev).half(), 4, 4)
+        w = dict(q=torch.randn(B, N, 1, 128, generator=g, device=dev).half(), codes=quant[0], meta=list(quant[1:]),
+                 kres=torch.randn(B, Nk, 128, 128, generator=g, device=dev).half(),
+                 v=torch.randn(B, Nk, L + 1, 128, generator=g, device=dev).half(), n_groups=L // 128, n_resid=1)
+        kw = dict(rbits=4, tbits=4)
+        args.config = args.shape
+    else:
+        w = wl.build_workload(args.config, dev)
+        sh = w["shape"]
+        kw = dict(rbits=sh.rbits, tbits=sh.tbits)
     if w.get("groups_per_seq") is not None:
         kw.update(n_groups_per_seq=w["groups_per_seq"], n_resid_per_seq=w["resid_per_seq"], total_groups=int(w["groups_per_seq"].sum()),
                   balanced=not args.even)
@@ -81,18 +94,27 @@ def main():
     if args.pairs:
         roles = {0: [], 1: []}
         for line in text.splitlines():
-            m = re.match(r"pq_pair block (\d+) wave (\d+) role (\d+) tiles (\d+) life (\d+) waited (\d+)", line)
+            m = re.match(r"pq_pair block (\d+) wave (\d+) role (\d+) tiles (\d+) entry (\d+) first (\d+) last (\d+) exit (\d+) waited (\d+)", line)
             if m and int(m.group(4)) > 0:
-                roles[int(m.group(3))].append((int(m.group(4)), int(m.group(5)) * 0.01, int(m.group(6)) * 0.01))
+                roles[int(m.group(3))].append(tuple(int(x) for x in m.groups()[3:]))       # tiles, entry, first, last, exit, waited
         if not roles[0] or not roles[1]:
             sys.exit("phase_timing: no pair reported (is this the measuring build?)")
-        out = {"config": args.config, "kernels": "scorer / accumulator pairs"}
+        origin = min(v[1] for r in roles.values() for v in r)
+        end = max(v[4] for r in roles.values() for v in r)
+        out = {"config": args.config, "kernels": "scorer / accumulator pairs",
+               "first_entry_to_last_exit_us": round((end - origin) * 0.01, 2)}
+        mean = lambda xs: sum(xs) / len(xs)
         for r, name in ((0, "scorer"), (1, "accumulator")):
             v = roles[r]
-            out[name] = {"wavefronts_reporting": len(v), "tiles": round(sum(t for t, _, _ in v) / len(v), 1),
-                         "life_us": round(sum(l for _, l, _ in v) / len(v), 2),
-                         "waiting_for_the_partner_us": round(sum(x for _, _, x in v) / len(v), 2),
-                         "waiting_share": round(sum(x for _, _, x in v) / sum(l for _, l, _ in v), 3)}
+            many = [x for x in v if x[0] > 1]
+            out[name] = {"wavefronts_reporting": len(v), "tiles": round(mean([x[0] for x in v]), 1),
+                         "life_us": round(mean([x[4] - x[1] for x in v]) * 0.01, 2),
+                         "entry_after_the_first_entry_us": round(mean([x[1] - origin for x in v]) * 0.01, 2),
+                         "entry_to_first_tile_handed_over_us": round(mean([x[2] - x[1] for x in v]) * 0.01, 2),
+                         "us_per_tile_between_first_and_last_hand_over": round(mean([(x[3] - x[2]) / (x[0] - 1) for x in many]) * 0.01, 3) if many else None,
+                         "last_hand_over_to_exit_us": round(mean([x[4] - x[3] for x in v]) * 0.01, 2),
+                         "waiting_for_the_partner_us": round(mean([x[5] for x in v]) * 0.01, 2),
+                         "waiting_share": round(sum(x[5] for x in v) / sum(x[4] - x[1] for x in v), 3)}
         print(json.dumps(out))
         return
     rows = []

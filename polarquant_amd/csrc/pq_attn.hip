@@ -346,7 +346,7 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
     __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kLutBytes];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
-    __shared__ int walk[8];
+    __shared__ int walk[kWalkInts];
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
     PQ_ATTN_KERNEL_PACK;
     const int lane = threadIdx.x;

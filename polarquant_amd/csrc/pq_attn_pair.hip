@@ -114,7 +114,7 @@ __device__ __forceinline__ void pair_roles(int* simd_of, int* flags, int wave, i
 // has handed over since the kernel began.  -> false if the partner stopped answering.
 template <typename T, int TB, int REPP, bool PK6>
 __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& pm, int lane, int b, int kvh, const SeqCounts& sc,
-                                            int t0, int t1, int r0, int r1, int& k, long long& pw_total_) {
+                                            int t0, int t1, int r0, int r1, int& k, PairTimes& pw_times_) {
     const int rep = p.rep;
     const int bh = b * p.Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
@@ -129,6 +129,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
         k++;
         if (lane == 0 && !pm.silent) *lds_ptr<lds_vi>(pm.flags) = k;
         asm volatile("" ::: "memory");
+        PQ_PAIR_T_TILE();
     };
     if (t0 < t1) {
         const int g0 = t0 >> 1, g1 = (t1 + 1) >> 1;
@@ -245,7 +246,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
 // Accumulator: the same tiles in the same order; writes the partial of the piece to `slot`.
 template <typename T, int REPP>
 __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const PairMem& pm, int lane, int b, int kvh, const SeqCounts& sc,
-                                                 int t0, int t1, int r0, int r1, int slot, int& k, long long& pw_total_,
+                                                 int t0, int t1, int r0, int r1, int slot, int& k, PairTimes& pw_times_,
                                                  uint16_t* direct_out = nullptr) {
     const int N = p.N, rep = p.rep;
     const int bh = b * p.Nk + kvh;
@@ -283,6 +284,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         k++;
         if (lane == 0) *lds_ptr<lds_vi>(pm.flags + 4) = k;
         asm volatile("" ::: "memory");
+        PQ_PAIR_T_TILE();
 #pragma unroll
         for (int j = 0; j < REPP; j++) {
             // the reference multiplies q . K^T of the residual keys in the model dtype before promoting (:79)
@@ -373,15 +375,12 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
     const int r1 = split == last_split ? (sc.nres + kWave - 1) / kWave : 0;
     int k = 0;
-    long long waited = 0;
+    PairTimes waited;
     PQ_PAIR_T_DECL;
     const bool ok = role == 0 ? pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited)
                               : pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
     if (!ok) report_timeout(status, lane);
-#ifdef PQ_ATTN_PHASE_TIMERS
-    pw_total_ = waited;
-#endif
-    PQ_PAIR_T_REPORT(role, k);
+    PQ_PAIR_T_REPORT(role, k, waited);
 }
 
 
@@ -395,7 +394,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[kPairsPerBlock][REPP * kWave];
     __shared__ int flag_mem[kPairsPerBlock][4];
     __shared__ int simd_of[2 * kPairsPerBlock];
-    __shared__ int walk_mem[2 * kPairsPerBlock][8];
+    __shared__ int walk_mem[2 * kPairsPerBlock][kWalkInts];
     PQ_ATTN_KERNEL_PACK;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int pair, role;
@@ -405,7 +404,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
     if (w >= n_pairs_total) return;
     int k = 0;
     bool ok = true;
-    long long waited = 0;
+    PairTimes waited;
     PQ_PAIR_T_DECL;
     walk_segment<false>(p, v4, n_pairs_total, w, lane, lds_addr(walk_mem[wave]),
                         [&](int cb, int ckvh, const SeqCounts& sc, int t0, int t1, int r0, int r1, int slot, bool ends_plane) {
@@ -422,10 +421,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
                             }
                         });
     if (!ok) report_timeout(status, lane);
-#ifdef PQ_ATTN_PHASE_TIMERS
-    pw_total_ = waited;
-#endif
-    PQ_PAIR_T_REPORT(role, k);
+    PQ_PAIR_T_REPORT(role, k, waited);
 }
 
 #pragma clang diagnostic pop

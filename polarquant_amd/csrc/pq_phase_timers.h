@@ -59,18 +59,25 @@ constexpr bool kProbeNoValues = false;
 
 // ---- scorer / accumulator pairs (pq_attn_pair.hip) ----
 // Measuring build only (-DPQ_ATTN_PHASE_TIMERS): every wavefront adds up the wall-clock time (100 MHz) it spends in
-// pair_wait, and the wavefronts of every 97th workgroup print it with their role when their kernel ends.
+// pair_wait and notes the clock at its entry, at its first and last hand-over and at its exit; the wavefronts of every
+// 97th workgroup print them with their role when their kernel ends.  From these the reader takes a pair's start-up
+// (entry -> first tile handed over), its pace in the steady state and its tail (last hand-over -> exit).
+struct PairTimes { long long waited = 0, first = 0, last = 0; };
 #ifdef PQ_ATTN_PHASE_TIMERS
-#define PQ_PAIR_T_DECL long long pw_total_ = 0; const long long pw_entry_ = wall_clock64()
-#define PQ_PAIR_T_WAIT(call) [&]() { const long long t0_ = wall_clock64(); const bool r_ = (call); pw_total_ += wall_clock64() - t0_; return r_; }()
-#define PQ_PAIR_T_REPORT(role, tiles)                                                                                \
+#define PQ_PAIR_T_DECL const long long pw_entry_ = wall_clock64()
+#define PQ_PAIR_T_WAIT(call) [&]() { const long long t0_ = wall_clock64(); const bool r_ = (call); pw_times_.waited += wall_clock64() - t0_; return r_; }()
+#define PQ_PAIR_T_TILE() do { pw_times_.last = wall_clock64(); if (pw_times_.first == 0) pw_times_.first = pw_times_.last; } while (0)
+#define PQ_PAIR_T_REPORT(role, tiles, times)                                                                         \
     do {                                                                                                             \
+        const long long pw_exit_ = wall_clock64();                                                                   \
         if ((threadIdx.x & 63) == 0 && blockIdx.x % 97 == 0)                                                         \
-            printf("pq_pair block %d wave %d role %d tiles %d life %lld waited %lld\n", static_cast<int>(blockIdx.x),  \
-                   static_cast<int>(threadIdx.x >> 6), role, tiles, wall_clock64() - pw_entry_, pw_total_);          \
+            printf("pq_pair block %d wave %d role %d tiles %d entry %lld first %lld last %lld exit %lld waited %lld\n", \
+                   static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x >> 6), role, tiles, pw_entry_,         \
+                   (times).first, (times).last, pw_exit_, (times).waited);                                           \
     } while (0)
 #else
 #define PQ_PAIR_T_DECL
 #define PQ_PAIR_T_WAIT(call) (call)
-#define PQ_PAIR_T_REPORT(role, tiles)
+#define PQ_PAIR_T_TILE()
+#define PQ_PAIR_T_REPORT(role, tiles, times)
 #endif
