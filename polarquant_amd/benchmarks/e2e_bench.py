@@ -51,9 +51,11 @@ def _check_against_eager(model, ids, first_logits, graph_tokens, graph_logits):
     mask = torch.ones_like(ids)
     out = model(input_ids=ids, attention_mask=mask, past_key_values=None, num_logits_to_keep=1)
     cache = out.past_key_values
+    cos = lambda a, b: float(torch.nn.functional.cosine_similarity(a.float().flatten(1), b.float().flatten(1), dim=1).min())
     agree = int((out.logits.argmax(-1) == first_logits.argmax(-1)).sum())
     total = first_logits.shape[0]
     diff = float((out.logits.float() - first_logits.float()).abs().max())
+    worst_cos = cos(out.logits, first_logits)
     finite = bool(torch.isfinite(first_logits.float()).all())
     for tok, lg in zip(graph_tokens, graph_logits):
         mask = torch.cat([mask, torch.ones_like(tok)], dim=-1)
@@ -62,10 +64,12 @@ def _check_against_eager(model, ids, first_logits, graph_tokens, graph_logits):
         agree += int((out.logits.argmax(-1) == lg.argmax(-1)).sum())
         total += lg.shape[0]
         diff = max(diff, float((out.logits.float() - lg.float()).abs().max()))
+        worst_cos = min(worst_cos, cos(out.logits, lg))
         finite = finite and bool(torch.isfinite(lg.float()).all())
     scale = float(first_logits.float().abs().max())
     return {"greedy_tokens_agreeing_with_the_eager_model": "%d of %d" % (agree, total), "steps_compared": len(graph_tokens) + 1,
-            "max_abs_logit_diff": round(diff, 5), "max_abs_logit": round(scale, 4), "logits_finite": finite,
+            "max_abs_logit_diff": round(diff, 5), "max_abs_logit": round(scale, 4),
+            "min_cosine_of_a_sequence's_logit_vectors": round(worst_cos, 6), "logits_finite": finite,
             "how": "eager model (module by module, Python-driven) fed the graph decoder's own tokens; all %d layers" % len(model.model.layers)}
 
 
@@ -73,6 +77,7 @@ def run(batch=8, prompt=16384, new=256, layers=32, graph=False, values4=False, f
         fp16_kv=None, check_tokens=0):
     """One timed prefill and the timed greedy loop -> dict of figures (see the module docstring)."""
     dev = torch.device("cuda:0")
+    torch.cuda.reset_peak_memory_stats()
     cfg = PolarConfig.llama3_8b(num_hidden_layers=layers, cache_capacity=prompt + new + 128,
                                 eos_token_id=[128256 + 10], vbits=4 if values4 else 16)
     model = build_model(cfg, dev)
@@ -114,6 +119,7 @@ def run(batch=8, prompt=16384, new=256, layers=32, graph=False, values4=False, f
             t_decode = time.perf_counter() - t0
             steps = new - 2
             cache = dec.cache()
+            peak = torch.cuda.max_memory_allocated()        # before the check below builds the eager model's own cache
             if check_tokens and not fp16_kv:
                 n = min(check_tokens, len(kept_logits))
                 sanity = _check_against_eager(model, ids, first_logits, kept_tok[:n], kept_logits[:n])
@@ -135,6 +141,7 @@ def run(batch=8, prompt=16384, new=256, layers=32, graph=False, values4=False, f
             torch.cuda.synchronize()
             t_decode = time.perf_counter() - t0
             steps = new - 1
+            peak = torch.cuda.max_memory_allocated()
     kv = model.kv_cache_bytes_per_token()
     fp16_bytes = cfg.num_hidden_layers * cfg.num_key_value_heads * 2 * 128 * 2
     if fp16_kv:
@@ -144,7 +151,7 @@ def run(batch=8, prompt=16384, new=256, layers=32, graph=False, values4=False, f
             "layers": layers, "graph": True, "attention": fp16_kv, "prefill_s": round(t_prefill, 3), "decode_s": round(t_decode, 3),
             "decode_ms_per_step": round(1e3 * t_decode / steps, 3), "decode_tokens_per_s": round(batch * steps / t_decode, 1),
             "kv_cache_bytes_per_token": fp16_bytes, "kv_seq_len": cache[0][-1],
-            "peak_memory_GiB": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+            "peak_memory_GiB": round(peak / 2 ** 30, 2),
         }
     res = {
         "workload": "configs[4]: greedy decode, random-init Llama-3-8B architecture, bf16, batch %d, prompt %d, %d new tokens"
@@ -154,7 +161,7 @@ def run(batch=8, prompt=16384, new=256, layers=32, graph=False, values4=False, f
         "decode_tokens_per_s": round(batch * steps / t_decode, 1),
         "kv_cache_bytes_per_token": kv, "fp16_kv_cache_bytes_per_token": fp16_bytes,
         "kv_seq_len": cache[0][-1], "quantized_groups": cache[0][1].shape[2],
-        "peak_memory_GiB": round(torch.cuda.max_memory_allocated() / 2 ** 30, 2),
+        "peak_memory_GiB": round(peak / 2 ** 30, 2),
     }
     if sanity is not None:
         res["sanity"] = sanity

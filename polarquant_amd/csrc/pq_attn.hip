@@ -302,7 +302,7 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
     using L = Lut<TB, REPP>;
     // the table region doubles as the staging buffer of the residual block's scores ([REPP][64] fp32)
     constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
-    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);
     PQ_ATTN_KERNEL_PACK;
@@ -344,7 +344,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu((V4 && RE
 void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
     using L = Lut<TB, REPP>;
     constexpr int kLutBytes = L::BYTES > REPP * kWave * 4 ? L::BYTES : REPP * kWave * 4;
-    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kLutBytes];
+    __shared__ __attribute__((aligned(16))) char lut_mem[kLutBytes];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[REPP * kWave];
     __shared__ int walk[kWalkInts];
     const uint32_t lut = lds_addr(lut_mem), pbuf = lds_addr(p_mem);

@@ -59,8 +59,15 @@ __device__ __forceinline__ PairMem pair_mem(uint32_t lut, uint32_t sbuf, uint32_
 }
 
 // A hand-over gave up: tell the host, if it passed a status word.  One lane, an ordinary vector store of a constant
-// (every wavefront that fails writes the same value, so no atomic is needed).
-__device__ __forceinline__ void report_timeout(int* status, int lane) {
+// (every wavefront that fails writes the same value, so no atomic is needed).  The pointer waits in LDS (stash_status,
+// before the workgroup's barrier) instead of in two scalar registers for the whole kernel: the scorer's group loop holds
+// 64 wave-uniform radius offsets in scalar registers and has none to spare.
+typedef __attribute__((address_space(3))) unsigned long long lds_u64;
+__device__ __forceinline__ void stash_status(unsigned long long* slot, int* status) {
+    if (threadIdx.x == 0) *slot = reinterpret_cast<unsigned long long>(status);
+}
+__device__ __forceinline__ void report_timeout(uint32_t slot, int lane) {
+    int* status = reinterpret_cast<int*>(*lds_ptr<lds_u64>(slot));
     if (status != nullptr && lane == 0) *status = kStatusHandoverTimeout;
 }
 
@@ -78,6 +85,7 @@ typedef __attribute__((address_space(3))) volatile int lds_vi;
 
 __device__ __forceinline__ bool pair_wait(uint32_t addr, int want, int spin_limit) {
     bool seen = false;
+#pragma clang loop unroll(disable)
     for (int i = 0; i < spin_limit; i++) {
         if (*lds_ptr<lds_vi>(addr) >= want) { seen = true; break; }
         __builtin_amdgcn_s_sleep(1);
@@ -119,9 +127,12 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
     const int bh = b * p.Nk + kvh;
     const int nb = sc.nb, nres = sc.nres;
     const uint16_t* qb = p.q + (static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * rep) * kHeadDim;
-    bool ok = true;
+    // polls a wait may still make: after one wait has given up it is 0, and every later wait falls through at once.  (One
+    // scalar register; a separate "all hand-overs succeeded so far" flag would be a second and third, which the group
+    // loop, with its 64 wave-uniform radius offsets, does not have.)
+    int spin = pm.spin_limit;
     auto publish_begin = [&]() {            // the buffer of tile k is free once tile k - 2 has been consumed
-        if (k >= 2) ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1, pm.spin_limit));
+        if (k >= 2 && !PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1, spin))) spin = 0;
         return pm.sbuf + (k & 1) * (REPP * kWave * 4);
     };
     auto publish_end = [&]() {
@@ -240,7 +251,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
             publish_end();
         }
     }
-    return ok;
+    return spin != 0;
 }
 
 // Accumulator: the same tiles in the same order; writes the partial of the piece to `slot`.
@@ -262,7 +273,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
     for (int j = 0; j < REPP; j++) { st.m[j] = -INFINITY; st.l[j] = 0.0f; st.zp[j] = 0.0f; }
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    bool ok = true;
+    int spin = pm.spin_limit;            // 0 once a wait has given up (see pair_scorer)
     // tile i of the piece: quantized tile t0 + i, or residual tile r0 + (i - nq); -> absolute row of its first token
     const int nq = t1 > t0 ? t1 - t0 : 0, nr = r1 > r0 ? r1 - r0 : 0, nt = nq + nr;
     auto row_of = [&](int i) { return i < nq ? (t0 + i) * kWave : nb * kGroup + (r0 + i - nq) * kWave; };
@@ -275,7 +286,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         const bool resid = i >= nq;
         const bool valid = resid ? (r0 + i - nq) * kWave + lane < nres : true;
         const bool keep = valid && (has_mask ? (__builtin_amdgcn_raw_buffer_load_b8(rm, lane, row, 0) != 0) : true);
-        ok = ok && PQ_PAIR_T_WAIT(pair_wait(pm.flags, k + 1, pm.spin_limit));
+        if (!PQ_PAIR_T_WAIT(pair_wait(pm.flags, k + 1, spin))) spin = 0;
         const uint32_t src = pm.sbuf + (k & 1) * (REPP * kWave * 4);
         float s[REPP];
 #pragma unroll
@@ -297,6 +308,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         step(std::integral_constant<int, 0>{}, i);
         if (i + 1 < nt) step(std::integral_constant<int, 1>{}, i + 1);
     }
+    const bool ok = spin != 0;
     float lsum[REPP];
 #pragma unroll
     for (int j = 0; j < REPP; j++) lsum[j] = wave_sum(st.l[j]);
@@ -342,14 +354,16 @@ template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer,
                                                                               int* __restrict__ status, uint16_t* __restrict__ direct_out) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kPairsPerBlock][L::BYTES];
+    __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[kPairsPerBlock][REPP * kWave];
     __shared__ int flag_mem[kPairsPerBlock][4];
     __shared__ int simd_of[2 * kPairsPerBlock];
+    __shared__ unsigned long long status_slot;
     PQ_ATTN_KERNEL_PACK;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int pair, role;
+    stash_status(&status_slot, status);
     pair_roles(simd_of, &flag_mem[0][0], wave, lane, pair, role);
     const PairMem pm = pair_mem(lds_addr(lut_mem[pair]), lds_addr(s_mem[pair]), lds_addr(p_mem[pair]), lds_addr(flag_mem[pair]), silent_scorer);
 
@@ -379,7 +393,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     PQ_PAIR_T_DECL;
     const bool ok = role == 0 ? pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited)
                               : pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
-    if (!ok) report_timeout(status, lane);
+    if (!ok) report_timeout(lds_addr(&status_slot), lane);
     PQ_PAIR_T_REPORT(role, k, waited);
 }
 
@@ -389,15 +403,17 @@ template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced_kernel(PQ_ATTN_KERNEL_PARAMS, int n_pairs_total, int silent_scorer,
                                                                                        int* __restrict__ status) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[kPairsPerBlock][L::BYTES];
+    __shared__ __attribute__((aligned(16))) char lut_mem[kPairsPerBlock][L::BYTES];
     __shared__ __attribute__((aligned(16))) float s_mem[kPairsPerBlock][2 * REPP * kWave];
     __shared__ __attribute__((aligned(16))) uint16_t p_mem[kPairsPerBlock][REPP * kWave];
     __shared__ int flag_mem[kPairsPerBlock][4];
     __shared__ int simd_of[2 * kPairsPerBlock];
     __shared__ int walk_mem[2 * kPairsPerBlock][kWalkInts];
+    __shared__ unsigned long long status_slot;
     PQ_ATTN_KERNEL_PACK;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     int pair, role;
+    stash_status(&status_slot, status);
     pair_roles(simd_of, &flag_mem[0][0], wave, lane, pair, role);
     const PairMem pm = pair_mem(lds_addr(lut_mem[pair]), lds_addr(s_mem[pair]), lds_addr(p_mem[pair]), lds_addr(flag_mem[pair]), silent_scorer);
     const int w = blockIdx.x * kPairsPerBlock + pair;
@@ -420,7 +436,7 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_balanced
                                 else poison_slot(p, lane, cb, ckvh, slot);
                             }
                         });
-    if (!ok) report_timeout(status, lane);
+    if (!ok) report_timeout(lds_addr(&status_slot), lane);
     PQ_PAIR_T_REPORT(role, k, waited);
 }
 

@@ -213,13 +213,16 @@ __device__ __forceinline__ float build_lut(uint32_t lut, int lane, const float (
     float ax[REPP], ay[REPP];
 #pragma unroll
     for (int j = 0; j < REPP; j++) { ax[j] = qx[j] * a; ay[j] = qy[j] * a; }
-    const uint32_t base = lut + lane * L::PB + ((lane & (L::NB - 1)) << L::SH);
+    // slot of bin k inside this lane's pair: k ^ (d & (NB-1)).  Computed on the slot number, then scaled and added to the
+    // pair's base: nothing here depends on how the table is aligned in LDS.
+    const uint32_t pair_base = lut + lane * L::PB;
+    const uint32_t swz = lane & (L::NB - 1);
 #pragma unroll
     for (int k = 0; k < L::NB; k++) {
         float e[REPP];
 #pragma unroll
         for (int j = 0; j < REPP; j++) e[j] = __builtin_fmaf(ax[j], c, ay[j] * s);
-        const uint32_t off = base ^ (k << L::SH);
+        const uint32_t off = pair_base + ((swz ^ k) << L::SH);
         lds_store_w<L::W0>(off, e);
         if constexpr (L::W1 > 0) lds_store_w<L::W1>(off + L::HB, e + 4);
         const float c2 = __builtin_fmaf(c, cd, -(s * sd));

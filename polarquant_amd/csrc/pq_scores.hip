@@ -12,7 +12,7 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(Lut<TB, R
                                                        const uint16_t* __restrict__ tscale, const uint16_t* __restrict__ tmn,
                                                        float* __restrict__ out, int N, int Nk, int Nb, int rep) {
     using L = Lut<TB, REPP>;
-    __shared__ __attribute__((aligned(L::PB < 16 ? 16 : L::PB))) char lut_mem[L::BYTES];
+    __shared__ __attribute__((aligned(16))) char lut_mem[L::BYTES];
     const uint32_t lut = lds_addr(lut_mem);
     const int lane = threadIdx.x;
     const int grp = blockIdx.x;
