@@ -28,9 +28,9 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # HBM bytes per launch of the dominant kernel at this workload, from two
 # `rocprofv3 --pmc` runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters
 # read for a copy kernel of known size; see profiles/attn_pair_kernel_cfg1_pmc.md.
-MEASURED_TRAFFIC_BYTES = int(675253 * 2.0 * 1024 + 2112.53 * 1024)
-TRAFFIC_SOURCE = ("constant, not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of 2026-11-25 with the attention "
-                  "kernel as of the commit 'Paired-wavefront kernels in their own source file' (profiles/attn_pair_kernel_cfg1_pmc.md)")
+MEASURED_TRAFFIC_BYTES = int(675343 * 2.0 * 1024 + 2112.58 * 1024)
+TRAFFIC_SOURCE = ("constant, not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of 2026-11-26 with the attention "
+                  "kernel as of the commit 'Table build independent of the table's LDS alignment' (profiles/attn_pair_kernel_cfg1_pmc.md)")
 
 
 def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):

@@ -20,7 +20,9 @@ the checks live in tests/test_oracle_pins.py):
                            GPU evaluation, the device library's atan2f, cannot be
                            restated on the CPU and is pinned on the GPU against
                            eager torch ops on device tensors
-                           (tests/test_quantize_gpu.py).
+                           (oracle/device_eager.py holds those ops, itself pinned
+                           on CPU tensors against this function bit for bit;
+                           tests/test_quantize_gpu.py runs them on the GPU).
   dequantize_keys          pinned: closed form on the known-answer group,
                            error bounds |phi-phi^|<=tscale/2, |r-r^|<=rscale/2.
   decode_scores            pinned: textbook q.K^T (torch.matmul) on the

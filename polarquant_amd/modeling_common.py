@@ -282,6 +282,9 @@ class PolarGroupAttention(nn.Module):
         self.hidden_size = config.hidden_size
         self.num_heads = config.num_attention_heads
         self.head_dim = _cfg(config, "head_dim", None) or self.hidden_size // self.num_heads
+        if self.head_dim != 128:
+            raise ValueError("polar attention kernels are built for head_dim 128 (64 pairs (d, d+64) per key); "
+                             "this configuration has head_dim %d" % self.head_dim)
         self.num_key_value_heads = _cfg(config, "num_key_value_heads", self.num_heads)
         self.num_key_value_groups = self.num_heads // self.num_key_value_heads
         self.is_causal = True

@@ -156,3 +156,15 @@ def test_padding_mask_conversion_is_not_fooled_by_a_recycled_address():
     # a uint8 mask passes through untouched
     m8 = torch.ones(shape, dtype=torch.uint8)
     assert _mask_u8(m8) is m8 and _mask_u8(None) is None
+
+
+def test_the_attention_class_refuses_a_head_dim_the_kernels_are_not_built_for():
+    """head_dim is fixed at 128 in the C ABI (PQ_HEAD_DIM); the drop-in classes say so when they are constructed
+    instead of failing inside a launch."""
+    from polarquant_amd.modeling_common import PolarConfig, PolarGroupAttention
+    cfg = PolarConfig(hidden_size=256, num_attention_heads=4, num_key_value_heads=2, num_hidden_layers=1,
+                      intermediate_size=128, vocab_size=64, head_dim=64)
+    with pytest.raises(ValueError, match="head_dim 128"):
+        PolarGroupAttention(cfg, 0)
+    PolarGroupAttention(PolarConfig(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, num_hidden_layers=1,
+                                    intermediate_size=128, vocab_size=64), 0)
