@@ -102,7 +102,7 @@ int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
     // half-precision values and at most 16 angle bins: a scorer / accumulator pair of wavefronts per slice or segment.
     // (4-bit values stay with one wavefront per slice, two per SIMD: a paired form of that kernel at four wavefronts per
     // SIMD was measured no faster -- the vector ALU's total work bounds it, however it is spread over wavefronts.)
-    const bool pairs = !a.v4_codes && !a.single_wave && a.tbits <= kMaxPairTbits;
+    const bool pairs = attn_runs_pairs(a.v4_codes, a.single_wave, a.tbits);
     long long total = static_cast<long long>(a.n_splits) * a.B * a.Nk;
     if (a.balanced) {
         // as many wavefronts (or pairs) as the device holds at once, but never more than there are partial slots

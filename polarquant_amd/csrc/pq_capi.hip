@@ -317,7 +317,9 @@ int pq_decode_attn(const void* q,
     if (!aligned(out, 2)) return PQ_ERR_MISALIGNED;
     // one slice per plane (a batch large enough to fill the device by itself): the default kernels write the output
     // themselves and the merge launch is saved
-    const bool direct = n_splits == 1 && !(flags & (PQ_SINGLE_WAVEFRONT | PQ_BALANCED_SLICES)) && aligned(out, 16);
+    // (only the paired kernels do that: angle widths that run the one-wavefront kernels keep the merge)
+    const bool direct = n_splits == 1 && !(flags & PQ_BALANCED_SLICES) && aligned(out, 16) &&
+                        pq::attn_runs_pairs(false, (flags & PQ_SINGLE_WAVEFRONT) != 0, tbits);
     if (int rc = run_attn_partials(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                                    k_resid, resid_capacity, n_resid, n_resid_per_seq, v, v_capacity, mask,
                                    mask_stride, sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split,

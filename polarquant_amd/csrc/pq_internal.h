@@ -91,5 +91,11 @@ inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 
 // More than 16 angle bins (tbits 5, 6): the table is 32-128 KiB, too large for the four tables of a paired workgroup;
 // those bit widths run the one-wavefront kernels.
 constexpr int kMaxPairTbits = 4;
+// Which family a call runs: the scorer / accumulator pairs (the only kernels that can write the finished output
+// themselves when a plane has a single slice) or the one-wavefront kernels.  One predicate for the launcher and for
+// the entry point that decides whether a merge launch follows.
+inline bool attn_runs_pairs(bool v4_codes, bool single_wave, int tbits) {
+    return !v4_codes && !single_wave && tbits <= kMaxPairTbits;
+}
 
 }  // namespace pq

@@ -151,6 +151,17 @@ def test_attn_split_invariance(gpu, n_splits):
     assert _close(out, ref64)[0] == 0
 
 
+@pytest.mark.parametrize("N,Nk,rbits,tbits", [(7, 1, 1, 6), (8, 2, 3, 5), (4, 4, 2, 6)])
+def test_attn_one_slice_per_plane_with_wide_angle_tables(gpu, N, Nk, rbits, tbits):
+    """n_splits == 1 lets the paired kernels write the output themselves; angle widths above 4 bits run the
+    one-wavefront kernels, which write a partial, so the merge has to follow (a call that skipped it returned
+    whatever the output buffer held)."""
+    print("case", N, Nk, rbits, tbits, flush=True)
+    out, ref, ref64 = _case(gpu, 1, N, Nk, 3, 1, rbits, tbits, torch.float16, seed=81, n_splits=1)
+    nbad, emax = _close(out, ref64)
+    assert nbad == 0, emax
+
+
 @pytest.mark.parametrize("n_splits,dtype", [(33, torch.float16), (70, torch.bfloat16), (130, torch.float16), (1030, torch.float16)])
 def test_attn_many_splits(gpu, n_splits, dtype):
     """32 or more / 128 or more partials per head take the merge kernel's 4- and 8-group forms; more
