@@ -94,9 +94,9 @@ def main():
     if args.pairs:
         roles = {0: [], 1: []}
         for line in text.splitlines():
-            m = re.match(r"pq_pair block (\d+) wave (\d+) role (\d+) tiles (\d+) entry (\d+) first (\d+) last (\d+) exit (\d+) waited (\d+)", line)
+            m = re.match(r"pq_pair block (\d+) wave (\d+) role (\d+) tiles (\d+) entry (\d+) first (\d+) last (\d+) exit (\d+) waited (\d+) marks (\d+) (\d+) (\d+)", line)
             if m and int(m.group(4)) > 0:
-                roles[int(m.group(3))].append(tuple(int(x) for x in m.groups()[3:]))       # tiles, entry, first, last, exit, waited
+                roles[int(m.group(3))].append(tuple(int(x) for x in m.groups()[3:]))       # tiles, entry, first, last, exit, waited, marks 0..2
         if not roles[0] or not roles[1]:
             sys.exit("phase_timing: no pair reported (is this the measuring build?)")
         origin = min(v[1] for r in roles.values() for v in r)
@@ -114,7 +114,11 @@ def main():
                          "us_per_tile_between_first_and_last_hand_over": round(mean([(x[3] - x[2]) / (x[0] - 1) for x in many]) * 0.01, 3) if many else None,
                          "last_hand_over_to_exit_us": round(mean([x[4] - x[3] for x in v]) * 0.01, 2),
                          "waiting_for_the_partner_us": round(mean([x[5] for x in v]) * 0.01, 2),
-                         "waiting_share": round(sum(x[5] for x in v) / sum(x[4] - x[1] for x in v), 3)}
+                         "waiting_share": round(sum(x[5] for x in v) / sum(x[4] - x[1] for x in v), 3),
+                         "entry_to_role_known_us": round(mean([x[6] - x[1] for x in v]) * 0.01, 2)}
+            if r == 0:
+                out[name]["entry_to_first_loads_arrived_us"] = round(mean([x[7] - x[1] for x in v if x[7]]) * 0.01, 2)
+                out[name]["entry_to_first_table_built_us"] = round(mean([x[8] - x[1] for x in v if x[8]]) * 0.01, 2)
         print(json.dumps(out))
         return
     rows = []

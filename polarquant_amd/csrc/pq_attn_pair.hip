@@ -131,6 +131,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
     // scalar register; a separate "all hand-overs succeeded so far" flag would be a second and third, which the group
     // loop, with its 64 wave-uniform radius offsets, does not have.)
     int spin = pm.spin_limit;
+    PQ_PAIR_T_MARK(0, false);
     auto publish_begin = [&]() {            // the buffer of tile k is free once tile k - 2 has been consumed
         if (k >= 2 && !PQ_PAIR_T_WAIT(pair_wait(pm.flags + 4, k - 1, spin))) spin = 0;
         return pm.sbuf + (k & 1) * (REPP * kWave * 4);
@@ -171,10 +172,12 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
         }
         for (int grp = g0; grp < g1; grp++) {
             asm volatile("" ::: "memory");
+            PQ_PAIR_T_MARK(1, true);
             const float cdv = build_lut<T, TB, REPP>(pm.lut, lane, qx, qy, mrs, mrm, mts, mtm);
             float cds[kPairs];
             broadcast_cd(cdv, cds);
             asm volatile("" ::: "memory");
+            PQ_PAIR_T_MARK(2, false);
             if (grp + 1 < g1) {
                 const int o = (grp + 1) * kPairs;
                 mrs = prs[o]; mrm = prm[o]; mts = pts[o]; mtm = ptm[o];
@@ -274,6 +277,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     int spin = pm.spin_limit;            // 0 once a wait has given up (see pair_scorer)
+    PQ_PAIR_T_MARK(0, false);
     // tile i of the piece: quantized tile t0 + i, or residual tile r0 + (i - nq); -> absolute row of its first token
     const int nq = t1 > t0 ? t1 - t0 : 0, nr = r1 > r0 ? r1 - r0 : 0, nt = nq + nr;
     auto row_of = [&](int i) { return i < nq ? (t0 + i) * kWave : nb * kGroup + (r0 + i - nq) * kWave; };

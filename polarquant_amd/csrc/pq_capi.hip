@@ -25,9 +25,10 @@ int check_decode_flags(unsigned flags, int rbits, int tbits, Entry entry = Entry
     unsigned known = PQ_CODES_PACKED6;
     if (entry != Entry::Scores) known |= PQ_BALANCED_SLICES;
     if (entry != Entry::Scores) known |= PQ_SINGLE_WAVEFRONT;
-    // (the test hook exists for the entry points with half-precision values only)
+    // (the test hook exists where a call runs the scorer / accumulator pairs: half-precision values, up to 4 angle bits)
 #ifdef PQ_TEST_HOOKS
-    if (entry == Entry::Attention && !(flags & PQ_SINGLE_WAVEFRONT)) known |= PQ_TEST_SILENT_SCORER;
+    if (entry == Entry::Attention && pq::attn_runs_pairs(false, (flags & PQ_SINGLE_WAVEFRONT) != 0, tbits))
+        known |= PQ_TEST_SILENT_SCORER;
 #endif
     if (flags & ~known) return PQ_ERR_BAD_SHAPE;
     if ((flags & PQ_CODES_PACKED6) && (tbits != 3 || rbits + tbits > 6)) return PQ_ERR_BAD_BITS;

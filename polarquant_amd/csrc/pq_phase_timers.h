@@ -62,22 +62,34 @@ constexpr bool kProbeNoValues = false;
 // pair_wait and notes the clock at its entry, at its first and last hand-over and at its exit; the wavefronts of every
 // 97th workgroup print them with their role when their kernel ends.  From these the reader takes a pair's start-up
 // (entry -> first tile handed over), its pace in the steady state and its tail (last hand-over -> exit).
-struct PairTimes { long long waited = 0, first = 0, last = 0; };
+struct PairTimes { long long waited = 0, first = 0, last = 0, mark[3] = {0, 0, 0}; };
 #ifdef PQ_ATTN_PHASE_TIMERS
 #define PQ_PAIR_T_DECL const long long pw_entry_ = wall_clock64()
 #define PQ_PAIR_T_WAIT(call) [&]() { const long long t0_ = wall_clock64(); const bool r_ = (call); pw_times_.waited += wall_clock64() - t0_; return r_; }()
 #define PQ_PAIR_T_TILE() do { pw_times_.last = wall_clock64(); if (pw_times_.first == 0) pw_times_.first = pw_times_.last; } while (0)
+// the clock the first time a wavefront passes a point of its start-up (scorer: 0 = role known, 1 = first loads have
+// arrived, which the measuring build waits for at this point, 2 = first table built; accumulator: 0 = role known)
+#define PQ_PAIR_T_MARK(i, drain)                                                                                     \
+    do {                                                                                                             \
+        if (pw_times_.mark[i] == 0) {                                                                                \
+            if (drain) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                              \
+            pw_times_.mark[i] = wall_clock64();                                                                      \
+        }                                                                                                            \
+    } while (0)
 #define PQ_PAIR_T_REPORT(role, tiles, times)                                                                         \
     do {                                                                                                             \
         const long long pw_exit_ = wall_clock64();                                                                   \
         if ((threadIdx.x & 63) == 0 && blockIdx.x % 97 == 0)                                                         \
-            printf("pq_pair block %d wave %d role %d tiles %d entry %lld first %lld last %lld exit %lld waited %lld\n", \
+            printf("pq_pair block %d wave %d role %d tiles %d entry %lld first %lld last %lld exit %lld waited %lld " \
+                   "marks %lld %lld %lld\n",                                                                         \
                    static_cast<int>(blockIdx.x), static_cast<int>(threadIdx.x >> 6), role, tiles, pw_entry_,         \
-                   (times).first, (times).last, pw_exit_, (times).waited);                                           \
+                   (times).first, (times).last, pw_exit_, (times).waited, (times).mark[0], (times).mark[1],          \
+                   (times).mark[2]);                                                                                 \
     } while (0)
 #else
 #define PQ_PAIR_T_DECL
 #define PQ_PAIR_T_WAIT(call) (call)
 #define PQ_PAIR_T_TILE()
+#define PQ_PAIR_T_MARK(i, drain)
 #define PQ_PAIR_T_REPORT(role, tiles, times)
 #endif

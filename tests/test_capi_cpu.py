@@ -164,6 +164,8 @@ def test_validate_decode_attn_and_plan(lib, hooks_lib):
     assert hooks.pq_validate_decode_attn(*a) == -2                   # with PQ_SINGLE_WAVEFRONT
     a[29] = 0x40000000 | 16
     assert hooks.pq_validate_decode_attn(*a) == 0                    # with balanced slices
+    a[29], a[21], a[22] = 0x40000000, 3, 5
+    assert hooks.pq_validate_decode_attn(*a) == -2                   # 5 angle bits run the one-wavefront kernels
     a = list(ok); a[29] = 64
     assert lib.pq_validate_decode_attn(*a) == -2                     # unknown flag bit
     assert lib.pq_validate_decode_scores(P, P, P, P, P, P, P, 2, 32, 8, 4, 4, 4, 0, 16) == -2
