@@ -36,8 +36,13 @@ def test_random_decode_attention_case(gpu, seed):
     resid = [rnd.randint(1, 128) for _ in range(B)] if ragged else [rnd.randint(1, 128)] * B
     use_mask = rnd.random() < 0.4
     n_splits = rnd.choice([None, 1, 2, 3, 5])
+    # further draws from a generator of their own, so that the cases above stay what they were for every seed:
+    # 3/3-bit codes stored as packed 6-bit rows; slices cut on the device also where a split count is given
+    rnd2 = random.Random(77000 + seed)
+    packed = (rb, tb) == (3, 3) and rnd2.random() < 0.5
+    balanced = True if (ragged and n_splits is not None and n_splits >= 2 and rnd2.random() < 0.5) else None
     print("case", dict(seed=seed, N=N, Nk=Nk, bits=(rb, tb), B=B, dtype=str(dtype), values4=values4, groups=groups,
-                       resid=resid, mask=use_mask, n_splits=n_splits), flush=True)
+                       resid=resid, mask=use_mask, n_splits=n_splits, packed=packed, balanced=balanced), flush=True)
     g = torch.Generator().manual_seed(seed)
     q = wl.make_half((B, N, 1, 128), g, dtype)
     codes = torch.zeros(B, Nk, cap, 128, 64, dtype=torch.uint8)
@@ -94,7 +99,12 @@ def test_random_decode_attention_case(gpu, seed):
     else:
         ng, nr = groups[0], resid[0]
     have_groups = any(groups) or ragged
-    cq = [dev(codes)] + [dev(m) for m in meta] if have_groups else [None] * 5
+    cq = [dev(po.pack_codes6(codes) if packed else codes)] + [dev(m) for m in meta] if have_groups else [None] * 5
+    # every call gets a status word: no hand-over between a scorer and its accumulator may ever give up
+    status = torch.zeros(1, dtype=torch.int32, device=gpu)
+    kw.update(status=status)
+    if balanced:
+        kw.update(balanced=True)
     if values4:
         vq_d = [dev(vcodes)] + [dev(m) for m in vmeta] if have_groups else [None] * 3
         out = polar_decode_attention_v4(dev(q), *cq, dev(kres), dev(vres), *vq_d, ng, nr, single_wavefront=seed % 4 == 3, **kw)
@@ -102,6 +112,7 @@ def test_random_decode_attention_case(gpu, seed):
         # one case in four takes the one-wavefront-per-slice kernels instead of the scorer / accumulator pairs
         out = polar_decode_attention(dev(q), *cq, dev(kres), dev(vfull), ng, nr, single_wavefront=seed % 4 == 3, **kw)
     out = out.cpu()
+    assert int(status) == 0
     assert torch.isfinite(out.float()).all()
     # the band is centred on the fp64 value and widened, element by element, by the distance of the
     # reference path's own half-precision evaluation from it (scores of the residual window and
