@@ -1,6 +1,9 @@
 """pq_linear_small_m (the decode step's projections at <= 16 rows) against fp32 torch matmuls of the
 same half-precision operands.  Tolerance: the result is one rounding of an fp32 sum whose order differs
 from the reference's, so at most one unit in the last place of the dtype, plus a little accumulation noise."""
+import os
+import random
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -60,6 +63,43 @@ def test_gated_linear_follows_the_eager_roundings(gpu, dtype, M, N, K):
     ref = (act.double() * up.double())
     # a last-place difference in gate or up (summation order) moves the product by about one more unit
     _check(y, ref, dtype, ulps=3.0)
+
+
+# more seeds: PQ_RANDOM_LINEAR_CASES=2000; another stretch of them: PQ_RANDOM_LINEAR_FIRST=1000
+_SEEDS = range(int(os.environ.get("PQ_RANDOM_LINEAR_FIRST", "0")),
+               int(os.environ.get("PQ_RANDOM_LINEAR_FIRST", "0")) + int(os.environ.get("PQ_RANDOM_LINEAR_CASES", "16")))
+
+
+@pytest.mark.parametrize("seed", _SEEDS)
+def test_random_linear_case(gpu, seed):
+    """Random rows (1..16), outputs (any multiple of 16), inner size (any multiple of 32: every K-split and stage
+    remainder), bias or gate, dtype, dense or strided x."""
+    rnd = random.Random(9000 + seed)
+    dtype = torch.bfloat16 if seed % 3 == 2 else torch.float16
+    M = rnd.randint(1, 16)
+    N = 16 * rnd.randint(1, 96)
+    K = 32 * rnd.randint(1, rnd.choice([8, 64, 300]))
+    gated = rnd.random() < 0.3
+    bias = not gated and rnd.random() < 0.5
+    strided = rnd.random() < 0.3
+    print("case", dict(seed=seed, dtype=str(dtype), M=M, N=N, K=K, gated=gated, bias=bias, strided=strided), flush=True)
+    g = torch.Generator().manual_seed(seed)
+    wide = torch.randn(M, K + 64, generator=g).to(dtype)
+    x = wide[:, 32:32 + K] if strided else wide[:, :K].contiguous()
+    sc = 1.0 / (K ** 0.5)
+    w = (torch.randn(N, K, generator=g) * sc).to(dtype)
+    if gated:
+        wu = (torch.randn(N, K, generator=g) * sc).to(dtype)
+        y = linear_small_m(wide.to(gpu)[:, 32:32 + K] if strided else x.to(gpu), w.to(gpu), up_weight=wu.to(gpu))
+        gate = F.linear(x.double(), w.double()).to(dtype)
+        up = F.linear(x.double(), wu.double()).to(dtype)
+        act = (gate.double() * torch.sigmoid(gate.double())).to(dtype)
+        _check(y, act.double() * up.double(), dtype, ulps=3.0)
+    else:
+        b = torch.randn(N, generator=g).to(dtype) if bias else None
+        y = linear_small_m(wide.to(gpu)[:, 32:32 + K] if strided else x.to(gpu), w.to(gpu), None if b is None else b.to(gpu))
+        _check(y, F.linear(x.double(), w.double(), None if b is None else b.double()), dtype)
+    assert y.shape == (M, N) and y.dtype == dtype
 
 
 def test_linear_rejects_what_the_kernel_does_not_cover(gpu):
