@@ -257,9 +257,9 @@ int pq_selftest_quantizer_math(int dtype, uint64_t *counters, void *stream);
  *            its first few slices (the others return at once).  n_splits * max(this,
  *            ceil(groups / n_splits)) always covers the sequence.
  *   workspace  device fp32 buffer of pq_decode_attn_workspace_bytes(...) bytes
- *   out      [B,N,128] half words.  With n_splits == 1 and a 16-byte aligned `out` the default kernels write it
- *            themselves (bit for bit what pq_decode_attn_merge makes of the one partial) and no merge is launched;
- *            the workspace then stays untouched
+ *   out      [B,N,128] half words.  With n_splits == 1 and a 16-byte aligned `out` the default kernels (tbits <= 4,
+ *            no PQ_SINGLE_WAVEFRONT, no PQ_BALANCED_SLICES) write it themselves (bit for bit what pq_decode_attn_merge
+ *            makes of the one partial) and no merge is launched; the workspace then stays untouched
  *   flags    0, or PQ_CODES_PACKED6 (code plane stride is then group_capacity*128*48) and / or
  *            PQ_BALANCED_SLICES (slices cut on the device from the per-sequence counts, see above) and / or
  *            PQ_SINGLE_WAVEFRONT (one wavefront per slice instead of a scorer / accumulator pair)
