@@ -377,6 +377,7 @@ __device__ __forceinline__ int wave_sum_i(int v) {
     return v;
 }
 
+
 // Balanced slices: the work of the whole batch is laid out as one line of units, plane after plane
 // (plane = (sequence, KV head), sequence-major).  A plane is kStartUnits units that stand for its
 // start-up, then one unit per tile of 64 tokens: two per quantized group, then one per 64 residual

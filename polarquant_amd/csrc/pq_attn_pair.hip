@@ -352,6 +352,43 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
     return ok;
 }
 
+// Even slices of one plane, in 64-token tiles: slice `split` of `n_splits` takes quantized tiles [t0, t1) and, if it is
+// the slice that ends the plane, the residual tiles [0, r1).  Normally a slice is a whole number of groups,
+// max(min_gps, ceil(groups / n_splits)), and the last one carries the residual keys on top of its share.  That share
+// is a full one when the groups divide evenly, and a full residual window then makes the last slice of every plane the
+// slowest of the launch (two more tiles that move 32 KB each where a quantized tile moves 20 KB: 19 tile times against
+// 16 at 8 groups per slice: 69.9 us against 62.1 us at batch 8 x 16384 tokens).  So the residual keys are given a
+// weight in tiles (3 per 128 keys, to the nearest tile) and, where that lowers the longest slice, the plane is cut into
+// equal runs of [quantized tiles | residual weight] instead; such slices begin and end in the middle of groups, which the
+// tile loops allow.  With one residual key (and whenever the even cut is already the better one) the slices are exactly
+// the whole-group ones.  Only the paired kernels cut this way: in the one-wavefront kernels (4-bit values, wide angle
+// tables) the same arithmetic ahead of the first loads cost more than the cut returned.
+struct EvenSlice { int t0, t1, r1; bool nothing; };
+__device__ __forceinline__ EvenSlice even_slice(const SeqCounts& sc, int n_splits, int min_gps, int split) {
+    const int T = 2 * sc.nb, R = (sc.nres + kWave - 1) / kWave;
+    EvenSlice e;
+    if (T == 0) {                                  // nothing quantized yet: slice 0 has the residual keys, if any
+        e.t0 = e.t1 = 0; e.r1 = split == 0 ? R : 0; e.nothing = split > 0;
+        return e;
+    }
+    const int RW = (3 * sc.nres + kGroup / 2) / kGroup;     // to the nearest tile: 0 below 22 keys, 3 from 107
+    int ups = 2 * ((sc.nb + n_splits - 1) / n_splits);
+    ups = ups < 2 * min_gps ? 2 * min_gps : ups;
+    const int last = (T - 1) / ups;
+    const int tail = T - last * ups + RW;          // what the last whole-group slice carries
+    const int worst = (last > 0 && ups > tail) ? ups : tail;
+    int alt = (T + RW + n_splits - 1) / n_splits;
+    alt = alt < 2 * min_gps ? 2 * min_gps : alt;
+    const bool weighted = alt < worst;
+    const int per = weighted ? alt : ups;
+    const int lo = split * per, hi = lo + per;
+    e.t0 = lo < T ? lo : T;
+    e.t1 = hi < T ? hi : T;
+    e.r1 = split == (weighted ? (T + RW - 1) / alt : last) ? R : 0;
+    e.nothing = split > 0 && e.t0 >= e.t1 && e.r1 == 0;
+    return e;
+}
+
 // Even slices, one slice per pair: pair index = 4 * blockIdx.x + (pair within the block), laid out as attn_kernel's
 // block index (plane fastest).
 template <typename T, int TB, int REPP, bool PK6>
@@ -378,9 +415,8 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     const int b = bh / Nk, kvh = bh - b * Nk;
     const V4Args v4none = v4;
     const SeqCounts sc = seq_counts<false>(p, v4none, b);
-    int gps = (sc.nb + n_splits - 1) / n_splits;
-    gps = gps < min_gps ? min_gps : gps;
-    if (split > 0 && split * gps >= sc.nb) {
+    const EvenSlice es = even_slice(sc, n_splits, min_gps, split);
+    if (es.nothing) {
         if (role == 1 && lane < rep) {
             float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats;
             pw[0] = -INFINITY;
@@ -388,15 +424,11 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
         }
         return;
     }
-    const int g0 = split * gps;
-    const int g1 = (g0 + gps) < sc.nb ? (g0 + gps) : sc.nb;
-    const int last_split = sc.nb > 0 ? (sc.nb - 1) / gps : 0;
-    const int r1 = split == last_split ? (sc.nres + kWave - 1) / kWave : 0;
     int k = 0;
     PairTimes waited;
     PQ_PAIR_T_DECL;
-    const bool ok = role == 0 ? pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, k, waited)
-                              : pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, 2 * g0, 2 * g1, 0, r1, split, k, waited, direct_out);
+    const bool ok = role == 0 ? pair_scorer<T, TB, REPP, PK6>(p, pm, lane, b, kvh, sc, es.t0, es.t1, 0, es.r1, k, waited)
+                              : pair_accumulator<T, REPP>(p, pm, lane, b, kvh, sc, es.t0, es.t1, 0, es.r1, split, k, waited, direct_out);
     if (!ok) report_timeout(lds_addr(&status_slot), lane);
     PQ_PAIR_T_REPORT(role, k, waited);
 }

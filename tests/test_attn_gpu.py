@@ -172,6 +172,27 @@ def test_attn_many_splits(gpu, n_splits, dtype):
     assert _close(out, ref64, rtol, atol)[0] == 0
 
 
+@pytest.mark.parametrize("n_groups,n_splits", [(1, 2), (2, 3), (3, 2), (8, 4), (8, 8), (16, 16), (5, 7)])
+def test_attn_slices_that_count_the_residual_keys(gpu, n_groups, n_splits):
+    """A long residual window makes the plane's last slice the longest, so the even cut then weighs the residual
+    keys and slices begin and end inside groups.  Every residual length around the weights' steps, against the
+    oracle, with a workspace full of NaN so that a slot nobody wrote would show."""
+    from polarquant_amd import attention
+    for n_resid in (1, 42, 43, 64, 65, 85, 86, 127, 128):
+        print("case", n_groups, n_splits, n_resid, flush=True)
+        ws = attention.new_workspace(2, 8, n_splits, gpu)
+        ws.fill_(float("nan"))
+        out, ref, ref64 = _case(gpu, 2, 8, 2, n_groups, n_resid, 4, 4, torch.float16, seed=100 * n_groups + n_resid,
+                                n_splits=n_splits, workspace=ws)
+        # a short context whose window holds a good part of the softmax mass: the stated tolerance against the fp64
+        # value or the reference path's own evaluation, else widened by what the reference's rounding of the window's
+        # scores can move (as in the random differential test)
+        o, r, r64 = out.double(), ref.double(), ref64.double()
+        e64, el = (o - r64).abs(), (o - r).abs()
+        bad = (e64 > ATOL + RTOL * r64.abs()) & (el > ATOL + RTOL * r.abs()) & (e64 > ATOL + RTOL * r64.abs() + _LAST["band"])
+        assert int(bad.sum()) == 0, (n_resid, float(e64.max()))
+
+
 @pytest.mark.parametrize("poison", [float("nan"), float("inf"), -1.0])
 def test_attn_ignores_what_the_workspace_held(gpu, poison):
     """The workspace is never cleared, and slices past a sequence's last group write only an empty

@@ -144,6 +144,17 @@ def test_attention_v4_split_counts_agree(gpu, n_splits):
     assert nbad == 0, (nbad, emax)
 
 
+@pytest.mark.parametrize("n_groups,n_splits", [(1, 2), (3, 2), (8, 8), (5, 7)])
+@pytest.mark.parametrize("n_resid", [64, 65, 128])
+def test_attention_v4_long_residual_windows_and_split_counts(gpu, n_groups, n_splits, n_resid):
+    """A full or nearly full residual window on the slice that ends the plane, at several split counts."""
+    out, ref, ref64 = _case(gpu, 2, 8, 2, n_groups, n_resid, 4, 4, torch.float16, seed=17 * n_groups + n_resid, n_splits=n_splits)
+    # a short context: each element against the fp64 value or the reference path's own evaluation
+    o, r, r64 = out.double(), ref.double(), ref64.double()
+    bad = ((o - r64).abs() > ATOL + RTOL * r64.abs()) & ((o - r).abs() > ATOL + RTOL * r.abs())
+    assert int(bad.sum()) == 0, float((o - r64).abs().max())
+
+
 def test_attention_v4_bf16(gpu):
     out, ref, ref64 = _case(gpu, 2, 8, 2, 16, 3, 4, 4, torch.bfloat16, seed=4)
     nbad, emax = _close(out, ref64, 2e-2, 4e-3)      # bf16 has 8 mantissa bits
