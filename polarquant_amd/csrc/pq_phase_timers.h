@@ -37,12 +37,13 @@ constexpr bool kProbeNoValues = false;
 #define PQ_T_EXIT()                                                                                                  \
     do {                                                                                                             \
         const long long pt_exit_ = wall_clock64();                                                                   \
-        if (threadIdx.x == 0 && blockIdx.x % 97 == 0) {                                                              \
+        const int pt_block_ = static_cast<int>((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x);      \
+        if (threadIdx.x == 0 && pt_block_ % 97 == 0) {                                                               \
             printf("pq_phase block %d groups %d total %lld table %lld value_issue %lld code_wait %lld code_issue %lld score %lld softmax_pv %lld\n", \
-                   static_cast<int>(blockIdx.x), pt_groups_, pt_loop1_ - pt_loop0_, pt_sum_[0], pt_sum_[1], pt_sum_[2], \
+                   pt_block_, pt_groups_, pt_loop1_ - pt_loop0_, pt_sum_[0], pt_sum_[1], pt_sum_[2], \
                    pt_sum_[3], pt_sum_[4], pt_sum_[5]);                                                              \
             printf("pq_piece block %d groups %d entry %lld exit %lld before_loop %lld first_group %lld loop %lld after_loop %lld\n", \
-                   static_cast<int>(blockIdx.x), pt_groups_, pt_entry_, pt_exit_, pt_loop0_ - pt_entry_, pt_first_,   \
+                   pt_block_, pt_groups_, pt_entry_, pt_exit_, pt_loop0_ - pt_entry_, pt_first_,   \
                    pt_loop1_ - pt_loop0_, pt_exit_ - pt_loop1_);                                                     \
         }                                                                                                            \
     } while (0)
