@@ -365,12 +365,6 @@ __device__ __forceinline__ void mark_empty_slots(const AttnParams& p, int lane, 
     p.v = v; p.v_capacity = v_capacity; p.mask = mask; p.mask_stride = mask_stride; p.scale_log2 = scale_log2;      \
     p.B = B; p.N = N; p.Nk = Nk; p.rep = rep; p.n_splits = n_splits; p.min_gps = min_gps; p.ws = ws
 
-// Units a plane's start-up counts for when the slices are cut on the device (query, first table, first loads, the
-// partial's write).  Measured at configs[2]: one wavefront per slice, 0 / 1 / 2 / 3 units: 92.8 / 89.6 / 87.9 / 88.6 us;
-// a pair per slice, whose tiles are faster and whose start-up is not, 1 / 2 / 3 / 4 / 5 units: 81.0 / 79.5 / 77.9 / 77.3 /
-// 77.3 us.
-constexpr int kStartUnits = 3;
-
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -401,8 +395,11 @@ __device__ __forceinline__ int wave_sum_i(int v) {
 // code or value load; measured at 64 ragged sequences: 13 us from entry to the first tile against 7.7 us with even slices).
 constexpr int kWalkInts = 8 + 2 * kWave;
 template <bool V4, typename F>
-__device__ __forceinline__ void walk_segment(const AttnParams& p, const V4Args& v4, long long W, long long w, int lane,
+__device__ __forceinline__ void walk_segment(const AttnParams& p, const V4Args& v4, unsigned W, unsigned w, int lane,
                                              uint32_t walk, F&& piece) {
+    // All positions on the line are 32-bit: the host refuses a call whose capacities could hold 2^31 units (far beyond
+    // what fits in device memory).  64-bit quotients here were a thousand instructions in front of every wavefront's
+    // first load.
     const int B = p.B, Nk = p.Nk;
     typedef __attribute__((address_space(3))) int lds_i1;
     // the counts of sequences 0..63 as the caller gave them, one per lane, into this wavefront's LDS
@@ -428,22 +425,23 @@ __device__ __forceinline__ void walk_segment(const AttnParams& p, const V4Args& 
     // length of the line
     int mine = 0;
     for (int base = 0; base < B; base += kWave) mine += (base + lane < B) ? units_of(base + lane) : 0;
-    const long long per_head = wave_sum_i(mine);          // units of one KV head's planes, all sequences
-    const long long total = per_head * Nk;
-    long long seg = (total + W - 1) / W;
-    seg = seg < 2 * p.min_gps ? 2 * p.min_gps : seg;
+    const unsigned per_head = static_cast<unsigned>(wave_sum_i(mine));          // units of one KV head's planes, all sequences
+    const unsigned total = per_head * static_cast<unsigned>(Nk);
+    unsigned seg = (total + W - 1u) / W;
+    seg = seg < 2u * static_cast<unsigned>(p.min_gps) ? 2u * static_cast<unsigned>(p.min_gps) : seg;
     // the most units a plane can have (the residual window is 128 keys in the reference, but the interface takes
     // any resid_capacity)
-    const long long cap_units = 2 * static_cast<long long>(p.group_capacity) + (p.resid_capacity + kWave - 1) / kWave + kStartUnits;
-    const long long fit = (cap_units + p.n_splits - 2) / (p.n_splits - 1);      // n_splits >= 2 (checked on the host)
+    const unsigned cap_units = 2u * static_cast<unsigned>(p.group_capacity) + static_cast<unsigned>((p.resid_capacity + kWave - 1) / kWave + kStartUnits);
+    const unsigned fit = (cap_units + static_cast<unsigned>(p.n_splits) - 2u) / static_cast<unsigned>(p.n_splits - 1);      // n_splits >= 2 (checked on the host)
     seg = seg < fit ? fit : seg;
-    const long long start = w * seg;
-    if (start >= total) return;
-    const long long end = (start + seg) < total ? (start + seg) : total;
+    // (w * seg can pass 2^32 only for wavefronts far behind the end of the line)
+    if (static_cast<unsigned long long>(w) * seg >= total) return;
+    const unsigned start = w * seg;
+    const unsigned end = (total - start) > seg ? (start + seg) : total;
 
     // the sequence that holds unit `start`: units before sequence bb are Nk * (sum of u over earlier sequences)
     int b = 0;
-    long long before = 0;                                  // units of one head's planes before sequence b
+    unsigned before = 0;                                   // units of one head's planes before sequence b
     for (int base = 0; base < B; base += kWave) {
         const int u = (base + lane < B) ? units_of(base + lane) : 0;
         int incl = u;
@@ -452,26 +450,25 @@ __device__ __forceinline__ void walk_segment(const AttnParams& p, const V4Args& 
             const int t = __shfl_up(incl, o);
             incl += (lane >= o) ? t : 0;
         }
-        const long long chunk = __shfl(incl, kWave - 1);
-        if (start < (before + chunk) * Nk) {
-            const unsigned long long past = __ballot((before + incl) * Nk > start);
+        const unsigned chunk = static_cast<unsigned>(__shfl(incl, kWave - 1));
+        if (start < (before + chunk) * static_cast<unsigned>(Nk)) {
+            const unsigned long long past = __ballot((before + static_cast<unsigned>(incl)) * static_cast<unsigned>(Nk) > start);
             const int l0 = __builtin_ctzll(past);
             b = base + l0;
-            before += __shfl(incl - u, l0);
+            before += static_cast<unsigned>(__shfl(incl - u, l0));
             break;
         }
         before += chunk;
     }
     {
-        const int u0 = units_of(b);
-        const long long seq_start = before * Nk;            // line position of plane (b, 0)
-        const int kvh0 = static_cast<int>((start - seq_start) / u0);
-        const long long plane_start = seq_start + static_cast<long long>(kvh0) * u0;
-        const long long span = end - start;
+        const unsigned u0 = static_cast<unsigned>(units_of(b));
+        const unsigned seq_start = before * static_cast<unsigned>(Nk);            // line position of plane (b, 0)
+        const unsigned kvh0 = (start - seq_start) / u0;
+        const unsigned plane_start = seq_start + kvh0 * u0;
         if (lane == 0) {
             lds_i1* wk = lds_ptr<lds_i1>(walk);
-            wk[0] = b; wk[1] = kvh0; wk[2] = static_cast<int>(start - plane_start); wk[3] = u0;
-            wk[4] = static_cast<int>(span < 0x7fffffffLL ? span : 0x7fffffffLL);          // units left in the segment
+            wk[0] = b; wk[1] = static_cast<int>(kvh0); wk[2] = static_cast<int>(start - plane_start); wk[3] = static_cast<int>(u0);
+            wk[4] = static_cast<int>(end - start);                                         // units left in the segment
             wk[5] = static_cast<int>(w - plane_start / seg);                               // slot of the first piece
         }
     }

@@ -207,6 +207,9 @@ int validate_attn(const void* q,
     if (n_splits < 1 || n_splits > 65534 || min_groups_per_split < 0) return PQ_ERR_WORKSPACE;
     // balanced slices: a plane shorter than a segment can still lie across one cut, i.e. two partials
     if ((flags & PQ_BALANCED_SLICES) && n_splits < 2) return PQ_ERR_WORKSPACE;
+    // ... and the kernels count the batch's units (64-token tiles plus the start-up units of every plane) in 32 bits
+    if ((flags & PQ_BALANCED_SLICES) &&
+        (2LL * group_capacity + (resid_capacity + 63) / 64 + pq::kStartUnits) * B * Nk > 0x7fffffffLL) return PQ_ERR_BAD_SHAPE;
     if (workspace_bytes < pq_decode_attn_workspace_bytes(B, N, n_splits)) return PQ_ERR_WORKSPACE;
     // q rows are read as 16-byte pieces (operands of the residual keys' matrix product)
     if (!aligned(q, 16) || !aligned(v, 16) || !aligned(out, 2) || !aligned(workspace, 16)) return PQ_ERR_MISALIGNED;

@@ -91,6 +91,12 @@ inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 
 // More than 16 angle bins (tbits 5, 6): the table is 32-128 KiB, too large for the four tables of a paired workgroup;
 // those bit widths run the one-wavefront kernels.
 constexpr int kMaxPairTbits = 4;
+// Units a plane's start-up counts for when the slices are cut on the device (query, first table, first loads, the
+// partial's write).  Measured at configs[2]: one wavefront per slice, 0 / 1 / 2 / 3 units: 92.8 / 89.6 / 87.9 / 88.6 us;
+// a pair per slice, whose tiles are faster and whose start-up is not, 1 / 2 / 3 / 4 / 5 units: 81.0 / 79.5 / 77.9 / 77.3 /
+// 77.3 us.
+constexpr int kStartUnits = 3;
+
 // Which family a call runs: the scorer / accumulator pairs (the only kernels that can write the finished output
 // themselves when a plane has a single slice) or the one-wavefront kernels.  One predicate for the launcher and for
 // the entry point that decides whether a merge launch follows.

@@ -164,6 +164,11 @@ def test_validate_decode_attn_and_plan(lib, hooks_lib):
     assert hooks.pq_validate_decode_attn(*a) == -2                   # with PQ_SINGLE_WAVEFRONT
     a[29] = 0x40000000 | 16
     assert hooks.pq_validate_decode_attn(*a) == 0                    # with balanced slices
+    # balanced slices count the batch's units in 32 bits: capacities that could hold 2^31 of them are refused
+    a = list(ok); a[29] = 16; a[6] = 1 << 17; a[18], a[19], a[20] = 4095, 16, 16; a[27] = lib.pq_decode_attn_workspace_bytes(4095, 16, 4)
+    assert lib.pq_validate_decode_attn(*a) == -2
+    a[29] = 0
+    assert lib.pq_validate_decode_attn(*a) == 0                      # even slices have no such line
     a[29], a[21], a[22] = 0x40000000, 3, 5
     assert hooks.pq_validate_decode_attn(*a) == -2                   # 5 angle bits run the one-wavefront kernels
     a = list(ok); a[29] = 64
