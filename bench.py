@@ -30,7 +30,9 @@ METRIC = "polar decode-attn µs/step + HBM GB/s (% of peak); Llama-3-8B shape b1
 # read for a copy kernel of known size; see profiles/attn_pair_kernel_cfg1_pmc.md.
 MEASURED_TRAFFIC_BYTES = int(675343 * 2.0 * 1024 + 2112.58 * 1024)
 TRAFFIC_SOURCE = ("constant, not read in this run: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of 2026-11-26 with the attention "
-                  "kernel as of the commit 'Table build independent of the table's LDS alignment' (profiles/attn_pair_kernel_cfg1_pmc.md)")
+                  "kernel as of the commit 'Table build independent of the table's LDS alignment', re-measured unchanged "
+                  "(675 341 / 2 112.55 counts) after the commit 'Device-side cut of balanced slices in 32-bit arithmetic' "
+                  "(profiles/attn_pair_kernel_cfg1_pmc.md)")
 
 
 def build_cfg1(dev, dtype=torch.float16, keep_keys_of=None):
