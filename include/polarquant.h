@@ -33,11 +33,11 @@ extern "C" {
 #define PQ_PAIRS 64
 #define PQ_GROUP 128
 #define PQ_MAX_REP 8          /* query heads per KV head (GQA ratio) supported by the kernels */
-#define PQ_MAX_TBITS 6        /* angle bits: the reference takes any split with rbits + tbits <= 8
-                                 (models/kernel4group.py:83-109); here 1..6, i.e. every split but 1/7, whose
-                                 128-bin angle table (128 KiB per four query heads) does not fit the LDS budget.
-                                 Up to 4 angle bits run the tuned kernels; 5 and 6 run the one-wavefront kernels
-                                 with a 32-128 KiB table (correct, not tuned). */
+#define PQ_MAX_TBITS 7        /* angle bits: every split the reference takes (rbits + tbits <= 8,
+                                 models/kernel4group.py:83-109).  Up to 4 angle bits run the tuned kernels; 5 to 7
+                                 run the one-wavefront kernels with a 32-128 KiB table (correct, not tuned); with 7
+                                 (128 bins: 128 KiB for four query heads, all the LDS a workgroup can have) a KV
+                                 head's query heads are worked through four at a time, in two launches. */
 #define PQ_PARTIAL_FLOATS 132 /* floats per split-K partial: m, l, 2 pad, acc[128] */
 #define PQ_MAX_PLANE_TOKENS 16776960 /* 2^24 - 256: most value rows (v_capacity, v4_capacity) or residual
                                         keys (resid_capacity) of one (batch, KV head) plane */
@@ -46,7 +46,7 @@ typedef enum {
     PQ_OK = 0,
     PQ_ERR_NULL_POINTER = -1,
     PQ_ERR_BAD_SHAPE = -2,      /* non-positive size, N % Nk != 0, rep > PQ_MAX_REP ... */
-    PQ_ERR_BAD_BITS = -3,       /* rbits/tbits outside [1,..], rbits + tbits > 8, tbits > PQ_MAX_TBITS */
+    PQ_ERR_BAD_BITS = -3,       /* rbits/tbits outside [1,..], rbits + tbits > 8 */
     PQ_ERR_BAD_DTYPE = -4,
     PQ_ERR_MISALIGNED = -5,     /* a pointer or stride breaks the alignment a kernel needs */
     PQ_ERR_BAD_STRIDE = -6,

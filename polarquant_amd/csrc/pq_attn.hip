@@ -59,7 +59,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
     const float scale_log2 = p.scale_log2;
     float* ws = p.ws;
 
-    const uint16_t* qb = p.q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep) * kHeadDim;
+    const uint16_t* qb = p.q + (static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * p.rep_stride) * kHeadDim;
     const __amdgpu_buffer_rsrc_t rv = make_rsrc(p.v + static_cast<size_t>(bh) * v_capacity * kHeadDim,
                                                 static_cast<uint32_t>((V4 ? nres : n_tokens) * (kHeadDim * 2)));
     const uint32_t voff_v = static_cast<uint32_t>(lane >> 4) * (4 * kHeadDim * 2) + static_cast<uint32_t>(lane & 15) * 16;
@@ -281,7 +281,7 @@ __device__ __forceinline__ void attn_piece(const AttnParams& p, const V4Args& v4
         float mm = st.m[0], ll = lsum[0];
 #pragma unroll
         for (int j = 1; j < REPP; j++) { mm = (n == j) ? st.m[j] : mm; ll = (n == j) ? lsum[j] : ll; }
-        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + n) * n_splits + slot) * kPartialFloats;
+        float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * p.rep_stride + n) * n_splits + slot) * kPartialFloats;
         if (g == 0) { pw[0] = mm; pw[1] = ll; }
         float* pa = pw + 4 + 32 * g;
 #pragma unroll
@@ -324,7 +324,7 @@ void attn_kernel(PQ_ATTN_KERNEL_PARAMS) {
     // slices past the end of a short sequence have nothing to do: mark their partials empty and leave
     if (split > 0 && split * gps >= sc.nb) {
         if (lane < rep) {
-            float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep + lane) * n_splits + split) * kPartialFloats;
+            float* pw = ws + ((static_cast<size_t>(b) * N + static_cast<size_t>(kvh) * rep_stride + lane) * n_splits + split) * kPartialFloats;
             pw[0] = -INFINITY;
             pw[1] = 0.0f;
         }
@@ -361,7 +361,9 @@ void attn_balanced_kernel(PQ_ATTN_KERNEL_PARAMS) {
 
 template <typename T, int TB>
 static int launch_attn_tb(const AttnArgs& a, int total, hipStream_t st) {
-    const int rep = a.N / a.Nk;
+    // a.rep_count: this launch's share of the query heads of every KV head (0: all of them); q and the workspace then
+    // point at the share's first head
+    const int rep_stride = a.N / a.Nk, rep = a.rep_count ? a.rep_count : rep_stride;
     const dim3 grid(static_cast<unsigned>(total)), block(kWave);
     const float scale_log2 = a.sm_scale * kLog2e;
     V4Args v4{static_cast<const uint32_t*>(a.v4_codes), static_cast<const uint16_t*>(a.v4_scale),
@@ -372,7 +374,7 @@ static int launch_attn_tb(const AttnArgs& a, int total, hipStream_t st) {
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
-                       a.n_splits, a.min_groups_per_split, a.workspace, v4)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4, rep_stride)
 #define PQ_LAUNCH_VP(REPP, V4, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_K(attn_balanced_kernel, REPP, V4, PK6);                                            \
@@ -393,11 +395,15 @@ static int launch_attn_tb(const AttnArgs& a, int total, hipStream_t st) {
         if (a.v4_codes) PQ_LAUNCH_V(REPP, true);                                                                     \
         else PQ_LAUNCH_V(REPP, false);                                                                               \
     } while (0)
+    // (128 angle bins: a table holds four heads at most, and the caller sends the heads in two launches)
     switch (rep_pad(rep)) {
         case 1: PQ_LAUNCH(1); break;
         case 2: PQ_LAUNCH(2); break;
         case 4: PQ_LAUNCH(4); break;
-        default: PQ_LAUNCH(8); break;
+        default:
+            if constexpr (TB <= 6) PQ_LAUNCH(8);
+            else return static_cast<int>(hipErrorInvalidValue);
+            break;
     }
 #undef PQ_LAUNCH
 #undef PQ_LAUNCH_V
@@ -419,7 +425,8 @@ int launch_attn_one_bf16(const AttnArgs& a, int total, hipStream_t st) {
         case 3: return launch_attn_tb<T, 3>(a, total, st);
         case 4: return launch_attn_tb<T, 4>(a, total, st);
         case 5: return launch_attn_tb<T, 5>(a, total, st);
-        default: return launch_attn_tb<T, 6>(a, total, st);
+        case 6: return launch_attn_tb<T, 6>(a, total, st);
+        default: return launch_attn_tb<T, 7>(a, total, st);
     }
 }
 

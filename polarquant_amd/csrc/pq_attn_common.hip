@@ -110,7 +110,19 @@ int launch_attn_partials(const AttnArgs& a, hipStream_t st) {
         total = slots < total ? slots : total;
     }
     if (pairs) return a.dtype == 0 ? launch_attn_pair_f16(a, static_cast<int>(total), st) : launch_attn_pair_bf16(a, static_cast<int>(total), st);
-    return a.dtype == 0 ? launch_attn_one_f16(a, static_cast<int>(total), st) : launch_attn_one_bf16(a, static_cast<int>(total), st);
+    auto one = [&](const AttnArgs& x) {
+        return x.dtype == 0 ? launch_attn_one_f16(x, static_cast<int>(total), st) : launch_attn_one_bf16(x, static_cast<int>(total), st);
+    };
+    if (a.tbits <= 6 || rep <= kMaxHeadsWidestTable) return one(a);
+    // 128 angle bins: the table of four query heads is 128 KiB, all the LDS a workgroup can have.  More heads per KV
+    // head go in two launches, heads [0, 4) and [4, rep) of every KV head, each writing its own heads' partials.
+    AttnArgs lo = a, hi = a;
+    lo.rep_count = kMaxHeadsWidestTable;
+    hi.rep_count = rep - kMaxHeadsWidestTable;
+    hi.q = static_cast<const uint16_t*>(a.q) + static_cast<size_t>(kMaxHeadsWidestTable) * kHeadDim;
+    hi.workspace = a.workspace + static_cast<size_t>(kMaxHeadsWidestTable) * a.n_splits * kPartialFloats;
+    if (int rc = one(lo)) return rc;
+    return one(hi);
 }
 
 constexpr int kMergeWideFrom = 32, kMergeWidestFrom = 128;

@@ -307,6 +307,9 @@ struct AttnParams {
     int64_t mask_stride;
     float scale_log2;
     int B, N, Nk, rep, n_splits, min_gps;
+    // query heads from one KV head to the next in q and in the partials: rep, except when a call's heads are worked
+    // through in two launches (128 angle bins: a table holds at most four heads)
+    int rep_stride;
     float* ws;
 };
 
@@ -343,7 +346,7 @@ __device__ __forceinline__ void mark_empty_slots(const AttnParams& p, int lane, 
     const int count = (p.n_splits - first) * p.rep;
     for (int i = lane; i < count; i += kWave) {
         const int j = i / (p.n_splits - first), s = first + i % (p.n_splits - first);
-        float* pw = p.ws + ((static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * p.rep + j) * p.n_splits + s) * kPartialFloats;
+        float* pw = p.ws + ((static_cast<size_t>(b) * p.N + static_cast<size_t>(kvh) * p.rep_stride + j) * p.n_splits + s) * kPartialFloats;
         pw[0] = -INFINITY;
         pw[1] = 0.0f;
     }
@@ -356,14 +359,15 @@ __device__ __forceinline__ void mark_empty_slots(const AttnParams& p, int lane, 
         const uint16_t* __restrict__ k_resid, int resid_capacity, int n_resid,                                       \
         const int32_t* __restrict__ n_resid_per_seq, const uint16_t* __restrict__ v, int64_t v_capacity,             \
         const uint8_t* __restrict__ mask, int64_t mask_stride, float scale_log2, int B, int N, int Nk, int rep,      \
-        int n_splits, int min_gps, float* __restrict__ ws, V4Args v4
+        int n_splits, int min_gps, float* __restrict__ ws, V4Args v4, int rep_stride
 #define PQ_ATTN_KERNEL_PACK                                                                                          \
     AttnParams p;                                                                                                    \
     p.q = q; p.codes = codes; p.rscale = rscale; p.rmn = rmn; p.tscale = tscale; p.tmn = tmn;                        \
     p.group_capacity = group_capacity; p.n_groups = n_groups; p.n_groups_per_seq = n_groups_per_seq;                 \
     p.k_resid = k_resid; p.resid_capacity = resid_capacity; p.n_resid = n_resid; p.n_resid_per_seq = n_resid_per_seq; \
     p.v = v; p.v_capacity = v_capacity; p.mask = mask; p.mask_stride = mask_stride; p.scale_log2 = scale_log2;      \
-    p.B = B; p.N = N; p.Nk = Nk; p.rep = rep; p.n_splits = n_splits; p.min_gps = min_gps; p.ws = ws
+    p.B = B; p.N = N; p.Nk = Nk; p.rep = rep; p.n_splits = n_splits; p.min_gps = min_gps; p.ws = ws;         \
+    p.rep_stride = rep_stride
 
 __device__ __forceinline__ int wave_sum_i(int v) {
 #pragma unroll

@@ -492,7 +492,7 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
                        (const uint16_t*)a.tmn, a.group_capacity, a.n_groups, a.n_groups_per_seq,                     \
                        (const uint16_t*)a.k_resid, a.resid_capacity, a.n_resid, a.n_resid_per_seq,                   \
                        (const uint16_t*)a.v, a.v_capacity, a.mask, a.mask_stride, scale_log2, a.B, a.N, a.Nk, rep,   \
-                       a.n_splits, a.min_groups_per_split, a.workspace, v4, total, a.silent_scorer ? 1 : 0, a.status, ##__VA_ARGS__)
+                       a.n_splits, a.min_groups_per_split, a.workspace, v4, rep, total, a.silent_scorer ? 1 : 0, a.status, ##__VA_ARGS__)
 #define PQ_LAUNCH_PAIR_P(REPP, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_PAIR_K(attn_pair_balanced_kernel, REPP, PK6);                                      \

@@ -10,8 +10,8 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 
 int check_bits(int rbits, int tbits) {
     if (rbits < 1 || tbits < 1 || rbits + tbits > 8) return PQ_ERR_BAD_BITS;
-    // 7 angle bits (128 bins) would need a table of 64 pairs x 128 bins x 16 bytes = 128 KiB per four query heads, which
-    // leaves no room in a compute unit's 160 KiB of LDS for a second wavefront's table or for eight heads; refused
+    // (7 angle bits: one byte per code leaves one radius bit; the decode kernels then work through a KV head's query
+    // heads four at a time, see kMaxHeadsWidestTable)
     if (tbits > PQ_MAX_TBITS) return PQ_ERR_BAD_BITS;
     return PQ_OK;
 }
@@ -52,8 +52,7 @@ const char* pq_status_string(int status) {
         case PQ_OK: return "ok";
         case PQ_ERR_NULL_POINTER: return "null pointer argument";
         case PQ_ERR_BAD_SHAPE: return "bad shape (non-positive size, N % Nk != 0, or N/Nk > 8)";
-        case PQ_ERR_BAD_BITS: return "bad bit widths (need rbits >= 1, 1 <= tbits <= 6, rbits + tbits <= 8; the reference's 1/7 split is "
-                                     "refused: its 128-bin angle table does not fit the kernels' LDS budget; packed 6-bit rows need tbits == 3)";
+        case PQ_ERR_BAD_BITS: return "bad bit widths (need rbits >= 1, tbits >= 1, rbits + tbits <= 8; packed 6-bit rows need tbits == 3)";
         case PQ_ERR_BAD_DTYPE: return "bad dtype (0 = float16, 1 = bfloat16)";
         case PQ_ERR_MISALIGNED: return "pointer or stride not aligned as the kernel requires";
         case PQ_ERR_BAD_STRIDE: return "bad stride or capacity";

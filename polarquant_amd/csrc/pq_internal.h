@@ -58,6 +58,7 @@ struct AttnArgs {
     int64_t mask_stride;
     float sm_scale;
     int B, N, Nk, tbits, dtype, n_splits, min_groups_per_split;
+    int rep_count = 0;           // query heads per KV head this launch works on (0: all N / Nk), see launch_attn_partials
     bool packed6 = false;        // code rows are 48 bytes of packed 6-bit codes (tbits == 3 only)
     bool balanced = false;       // slices cut on the device from the per-sequence counts (PQ_BALANCED_SLICES)
     bool single_wave = false;    // one wavefront per slice instead of a scorer / accumulator pair (PQ_SINGLE_WAVEFRONT)
@@ -91,6 +92,9 @@ inline int rep_pad(int rep) { return rep <= 1 ? 1 : rep <= 2 ? 2 : rep <= 4 ? 4 
 // More than 16 angle bins (tbits 5, 6): the table is 32-128 KiB, too large for the four tables of a paired workgroup;
 // those bit widths run the one-wavefront kernels.
 constexpr int kMaxPairTbits = 4;
+// 128 angle bins (tbits 7): 64 pairs x 128 bins x 16 bytes = 128 KiB for up to four query heads, which is all the LDS
+// a workgroup can have; KV heads with more query heads are worked through four heads at a time.
+constexpr int kMaxHeadsWidestTable = 4;
 // Units a plane's start-up counts for when the slices are cut on the device (query, first table, first loads, the
 // partial's write).  Measured at configs[2]: one wavefront per slice, 0 / 1 / 2 / 3 units: 92.8 / 89.6 / 87.9 / 88.6 us;
 // a pair per slice, whose tiles are faster and whose start-up is not, 1 / 2 / 3 / 4 / 5 units: 81.0 / 79.5 / 77.9 / 77.3 /

@@ -109,7 +109,9 @@ def _case(gpu, B, N, Nk, n_groups, n_resid, rbits, tbits, dtype, theta=5e5, mask
                                               # every head ratio has its own kernel: 3, 5, 6, 7 (and 7 with 16 bins)
                                               (12, 4, 4, 4), (10, 2, 4, 4), (12, 2, 4, 4), (7, 1, 4, 4), (14, 2, 2, 2),
                                               # more than 16 angle bins (the one-wavefront kernels in either form)
-                                              (32, 8, 3, 5), (8, 1, 2, 6), (16, 4, 2, 6), (6, 2, 1, 6), (4, 4, 3, 5)])
+                                              (32, 8, 3, 5), (8, 1, 2, 6), (16, 4, 2, 6), (6, 2, 1, 6), (4, 4, 3, 5),
+                                              # 128 angle bins: a table holds four heads, more heads per KV head go in two launches
+                                              (8, 2, 1, 7), (3, 1, 1, 7), (8, 1, 1, 7), (14, 2, 1, 7), (10, 2, 1, 7)])
 def test_attn_matches_oracle(gpu, dtype, N, Nk, rbits, tbits):
     print("case", dtype, N, Nk, rbits, tbits, flush=True)
     out, ref, ref64 = _case(gpu, 2, N, Nk, 6, 37, rbits, tbits, dtype, seed=1)

@@ -58,10 +58,10 @@ def test_validate_decode_scores(lib):
     assert bad(7, 0) == -2 and bad(9, 5) == -2 and bad(10, 0) == -2   # B<=0, N % Nk, Nb<=0
     assert bad(8, 72) == -2                                          # rep 9 > 8
     assert bad(11, 5) == -3 and bad(12, 5) == -3 and bad(12, 0) == -3  # r+t>8 (twice), tbits<1
-    # every split the reference takes (rbits + tbits <= 8) but 1/7, whose 128-bin table does not fit the LDS budget
-    for rb, tb, want in ((3, 5, 0), (2, 6, 0), (1, 6, 0), (4, 1, 0), (7, 1, 0), (1, 7, -3), (2, 7, -3), (0, 4, -3)):
+    # every split the reference takes (rbits + tbits <= 8), 1/7 included
+    for rb, tb, want in ((3, 5, 0), (2, 6, 0), (1, 6, 0), (4, 1, 0), (7, 1, 0), (1, 7, 0), (2, 7, -3), (1, 8, -3), (0, 4, -3)):
         assert lib.pq_validate_decode_scores(*ok[:11], rb, tb, 0, 0) == want, (rb, tb)
-    assert b"1 <= tbits <= 6" in lib.pq_status_string(-3)
+    assert b"rbits + tbits <= 8" in lib.pq_status_string(-3)
     assert bad(13, 2) == -4                                          # dtype
     assert bad(1, P + 4) == -5 and bad(6, P + 2) == -5               # misaligned codes / out
     # the launching entry point runs the same checks before touching the device
@@ -84,12 +84,14 @@ def test_validate_quantize_groups(lib):
     assert bad(0, None) == -1 and bad(1, None) == -1 and bad(9, None) == -1
     assert bad(3, 0) == -2 and bad(5, 0) == -2
     assert bad(6, 5) == -3 and bad(7, 0) == -3
-    # bit widths the decode entry points cannot read are refused by the quantizer too (tbits 7)
+    # the quantizer takes every split the decode entry points read
     a = list(ok); a[6], a[7] = 2, 5
     assert lib.pq_validate_quantize_groups(*a) == 0
     a[6], a[7] = 2, 6
     assert lib.pq_validate_quantize_groups(*a) == 0
     a[6], a[7] = 1, 7
+    assert lib.pq_validate_quantize_groups(*a) == 0
+    a[6], a[7] = 2, 7
     assert lib.pq_validate_quantize_groups(*a) == -3
     assert bad(2, 7) == -4
     assert bad(8, 1) == 0 and bad(8, 2) == 0 and bad(8, 3) == 0   # PQ_WRAP_FP32, PQ_ANGLE_UNIFORM
@@ -121,7 +123,7 @@ def test_validate_decode_attn_and_plan(lib, hooks_lib):
     assert lib.pq_validate_decode_attn(*a) == 0                      # packed 6-bit codes with 3/3 bits
     a[21] = 4
     assert lib.pq_validate_decode_attn(*a) == -3
-    for rb, tb, want in ((3, 5, 0), (2, 6, 0), (1, 7, -3)):
+    for rb, tb, want in ((3, 5, 0), (2, 6, 0), (1, 7, 0), (2, 7, -3)):
         a = list(ok); a[21], a[22] = rb, tb
         assert lib.pq_validate_decode_attn(*a) == want, (rb, tb)
 

@@ -35,7 +35,7 @@ def count_flips(got, ref):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (2, 4), (5, 3), (4, 2)])
+@pytest.mark.parametrize("rbits,tbits", [(4, 4), (3, 3), (2, 4), (5, 3), (4, 2), (2, 6), (1, 7)])
 def test_quantize_bit_exact(gpu, dtype, rbits, tbits):
     print("case", dtype, rbits, tbits, flush=True)
     g = torch.Generator().manual_seed(21)

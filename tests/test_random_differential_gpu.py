@@ -39,6 +39,8 @@ def test_random_decode_attention_case(gpu, seed):
     # further draws from a generator of their own, so that the cases above stay what they were for every seed:
     # 3/3-bit codes stored as packed 6-bit rows; slices cut on the device also where a split count is given
     rnd2 = random.Random(77000 + seed)
+    if rnd2.random() < 0.06:
+        rb, tb = 1, 7                       # 128 angle bins (more than four heads per KV head: two launches)
     packed = (rb, tb) == (3, 3) and rnd2.random() < 0.5
     balanced = True if (ragged and n_splits is not None and n_splits >= 2 and rnd2.random() < 0.5) else None
     print("case", dict(seed=seed, N=N, Nk=Nk, bits=(rb, tb), B=B, dtype=str(dtype), values4=values4, groups=groups,
@@ -173,6 +175,8 @@ def test_random_quantizer_case(gpu, seed):
     rnd = random.Random(5000 + seed)
     dtype = torch.bfloat16 if seed % 3 == 2 else torch.float16
     rb, tb = rnd.choice(BITS)
+    if random.Random(78000 + seed).random() < 0.06:
+        rb, tb = 1, 7
     mode = rnd.choice(["group", "group", "uniform"])
     scale = 10.0 ** rnd.uniform(-6, 4 if dtype == torch.bfloat16 else 3.5)
     kind = rnd.choice(["normal", "cauchy", "sparse", "flat"])
@@ -222,6 +226,8 @@ def test_random_scores_case(gpu, seed):
     rnd = random.Random(9000 + seed)
     N, Nk = rnd.choice(HEADS)
     rb, tb = rnd.choice(BITS)
+    if random.Random(79000 + seed).random() < 0.06:
+        rb, tb = 1, 7
     B, Nb = rnd.randint(1, 3), rnd.randint(1, 6)
     dtype = torch.bfloat16 if seed % 4 == 3 else torch.float16
     synthetic = rnd.random() < 0.4

@@ -30,7 +30,9 @@ def _run(gpu, q, quant, rbits, tbits):
 @pytest.mark.parametrize("heads,kv,rbits,tbits", [(32, 32, 4, 4), (32, 8, 4, 4), (28, 4, 3, 3), (16, 8, 4, 4),
                                                   (8, 1, 5, 3), (6, 2, 2, 2), (5, 1, 4, 4), (12, 2, 4, 4), (3, 1, 4, 1),
                                                   # more than 16 angle bins: the wide table (32-128 KiB)
-                                                  (8, 1, 2, 6), (32, 8, 3, 5), (6, 2, 2, 5), (7, 1, 1, 6), (2, 2, 2, 6)])
+                                                  (8, 1, 2, 6), (32, 8, 3, 5), (6, 2, 2, 5), (7, 1, 1, 6), (2, 2, 2, 6),
+                                                  # 128 angle bins: four heads per table, more heads in two launches
+                                                  (4, 1, 1, 7), (3, 1, 1, 7), (8, 1, 1, 7), (14, 2, 1, 7), (10, 2, 1, 7), (2, 2, 1, 7)])
 def test_scores_match_oracle(gpu, dtype, heads, kv, rbits, tbits):
     print("case", dtype, heads, kv, rbits, tbits, flush=True)
     g = torch.Generator().manual_seed(7)
