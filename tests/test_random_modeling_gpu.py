@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 # more seeds: PQ_RANDOM_MODEL_CASES=200; another stretch of them: PQ_RANDOM_MODEL_FIRST=1000
 SEEDS = range(int(os.environ.get("PQ_RANDOM_MODEL_FIRST", "0")),
               int(os.environ.get("PQ_RANDOM_MODEL_FIRST", "0")) + int(os.environ.get("PQ_RANDOM_MODEL_CASES", "8")))
-BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 5), (2, 6)]
+BITS = [(4, 4), (3, 3), (4, 2), (5, 3), (2, 4), (3, 5), (2, 6), (1, 7)]
 
 
 def _rope(theta, start, n, dtype, dev):
