@@ -9,7 +9,10 @@
 // puts exactly two on every SIMD; which two is read from the hardware id register, and the two
 // that share a SIMD form a pair (lower wavefront index = scorer).  If the ids do not come out in
 // pairs the wavefronts are paired as (w, w + 4): the results are the same, only the overlap is lost.
-// The two hand tiles over through two counters in LDS (tiles published / tiles consumed); a wait
+// The two hand tiles over through two counters in LDS (tiles published / tiles consumed).  A counter is stored only
+// after `s_waitcnt lgkmcnt(0)`: the wavefront's own LDS writes of the tile (or its reads of it, for the "consumed"
+// counter) have completed by then, so whoever sees the counter sees the tile, and the order in which the LDS serves
+// requests of different wavefronts is not relied on (the wait costs 0.3 us per launch).  A wait
 // gives up after kSpinLimit polls (about half a second), after which both wavefronts run out
 // without waiting again, the accumulator writes NaN into the partial of this piece and of every
 // later piece of its segment, and both set the caller's status word (if one was passed) with a plain
@@ -137,7 +140,7 @@ __device__ __forceinline__ bool pair_scorer(const AttnParams& p, const PairMem& 
         return pm.sbuf + (k & 1) * (REPP * kWave * 4);
     };
     auto publish_end = [&]() {
-        asm volatile("" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         k++;
         if (lane == 0 && !pm.silent) *lds_ptr<lds_vi>(pm.flags) = k;
         asm volatile("" ::: "memory");
@@ -295,7 +298,7 @@ __device__ __forceinline__ bool pair_accumulator(const AttnParams& p, const Pair
         float s[REPP];
 #pragma unroll
         for (int j = 0; j < REPP; j++) s[j] = *lds_ptr<lds_f1>(src + (j * kWave + lane) * 4);
-        asm volatile("" ::: "memory");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         k++;
         if (lane == 0) *lds_ptr<lds_vi>(pm.flags + 4) = k;
         asm volatile("" ::: "memory");
