@@ -546,7 +546,9 @@ int pq_validate_decode_attn_v4(const void* q,
     if ((v_codes && !aligned(v_codes, 4)) || (v_resid && !aligned(v_resid, 16))) return PQ_ERR_MISALIGNED;
     // everything else as in the fp16-value entry point; its V-capacity rule is met by construction here
     static const char dummy_v[16] __attribute__((aligned(16))) = {0};
-    const int64_t vcap = static_cast<int64_t>(group_capacity > n_groups ? group_capacity : n_groups) * PQ_GROUP + resid_capacity + 1;
+    // (a stand-in, not memory: no more than the limit, so that the largest code and value stores pass as they should)
+    int64_t vcap = static_cast<int64_t>(group_capacity > n_groups ? group_capacity : n_groups) * PQ_GROUP + resid_capacity + 1;
+    vcap = vcap > PQ_MAX_PLANE_TOKENS ? PQ_MAX_PLANE_TOKENS : vcap;
     return validate_attn(q, codes, rscale, rmn, tscale, tmn, group_capacity, n_groups, n_groups_per_seq,
                          k_resid, resid_capacity, n_resid, n_resid_per_seq, dummy_v, vcap, mask, mask_stride,
                          sm_scale, B, N, Nk, rbits, tbits, dtype, n_splits, min_groups_per_split, workspace,

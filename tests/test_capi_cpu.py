@@ -230,6 +230,11 @@ def test_validate_value_quantizer_and_v4_attention(lib, hooks_lib):
     # exists for the half-precision-value entry points only and is refused here instead of silently ignored (in the test
     # build too)
     assert bad4(32, 16) == 0 and bad4(32, 32) == 0 and bad4(32, 0x40000000) == -2
+    # the largest stores: 2^24 - 256 rows of packed values, as many whole groups of codes as fit under that
+    a = list(ok); a[6], a[17] = ((1 << 24) - 256) // 128, (1 << 24) - 256
+    assert lib.pq_validate_decode_attn_v4(*a) == 0
+    a[17] += 1
+    assert lib.pq_validate_decode_attn_v4(*a) == -2
     a = list(ok); a[32] = 0x40000000
     assert hooks_lib.pq_validate_decode_attn_v4(*a) == -2
     # two wavefronts per SIMD for up to 4 query heads per KV head, one beyond

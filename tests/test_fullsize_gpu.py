@@ -242,3 +242,125 @@ def test_cfg4_attention_layer_at_full_width(gpu):
         assert torch.equal(solo_cache[1][0, :, :L // 128], again[1][5, :, :L // 128])
         close = (solo[0].float() - batched[5].float()).abs().max().item()
         assert close <= 2e-2 * max(1.0, batched[5].float().abs().max().item()), close
+
+
+@pytest.mark.parametrize("form", ["pairs", "one_wavefront", "device_cut", "three_slices"])
+def test_largest_plane(gpu, form):
+    """One (sequence, KV head) plane at the size limit: 2^24 - 256 value rows (4.29 GB of values, 1.07 GB of codes), the
+    largest offsets the kernels form.  The context is one block of 7 quantized groups repeated 18 724 times, so every block
+    carries the same softmax mass; value dimensions 0..14 hold the binary digits of a token's block number, whose
+    attention-weighted mean is then the fraction of blocks with that digit set (a closed form), and the other dimensions
+    repeat the block's values, whose result is the oracle's for a single block.  A value row fetched from a wrong offset, a
+    slice skipped or read twice, or a group's metadata taken from another group (7 is odd: no power-of-two stride maps a
+    block onto itself) moves one or the other."""
+    from polarquant_amd import workloads as wl
+    print("case", form, flush=True)
+    G_BLK, N_BLK = 7, 18724
+    n_groups = G_BLK * N_BLK                                  # 131 068 groups = 16 776 704 tokens
+    rows, group_cap = (1 << 24) - 256, ((1 << 24) - 256) // 128
+    g = torch.Generator().manual_seed(77)
+    kb = wl.make_keys(1, 1, G_BLK * 128, 5e5, g, torch.float16)
+    quant = po.quantize_and_pack_nbit(kb, 4, 4)
+    vb = wl.make_half((1, 1, G_BLK * 128, 128), g, torch.float16)
+    vb[..., :16] = 0
+    q = wl.make_half((1, 4, 1, 128), g, torch.float16)
+    ref_block = po.decode_attention_exact(q, None, *quant, vb, None, 4, 4)          # dimensions 16.. of the expected output
+    codes = torch.zeros(1, 1, group_cap, 128, 64, dtype=torch.uint8, device=gpu)
+    codes[:, :, :n_groups] = quant[0].to(gpu).repeat(1, 1, N_BLK, 1, 1)
+    meta = []
+    for m in quant[1:]:
+        t = torch.zeros(1, 1, group_cap, 1, 64, dtype=torch.float16, device=gpu)
+        t[:, :, :n_groups] = m.to(gpu).repeat(1, 1, N_BLK, 1, 1)
+        meta.append(t)
+    v = torch.zeros(1, 1, rows, 128, dtype=torch.float16, device=gpu)
+    T = n_groups * 128
+    v[0, 0, :T, 16:] = vb[0, 0, :, 16:].to(gpu).repeat(N_BLK, 1)
+    blk = torch.arange(T, device=gpu) // (G_BLK * 128)
+    for d in range(15):
+        v[0, 0, :T, d] = ((blk >> d) & 1).to(torch.float16)
+    v[0, 0, T:] = float("nan")                               # rows behind the context must not be read as values
+    del blk
+    want = ref_block.clone().double()
+    idx = torch.arange(N_BLK)
+    for d in range(15):
+        want[..., d] = float(((idx >> d) & 1).double().mean())
+    want[..., 15] = 0.0
+    kres = torch.zeros(1, 1, 128, 128, dtype=torch.float16, device=gpu)
+    kw = dict(rbits=4, tbits=4)
+    if form == "one_wavefront":
+        kw.update(single_wavefront=True)
+    elif form == "device_cut":
+        kw.update(n_groups_per_seq=torch.tensor([n_groups], dtype=torch.int32, device=gpu),
+                  n_resid_per_seq=torch.tensor([0], dtype=torch.int32, device=gpu))
+    elif form == "three_slices":
+        kw.update(n_splits=3)
+    ng = 0 if form == "device_cut" else n_groups
+    out = polar_decode_attention(q.to(gpu), codes, *meta, kres, v, ng, 0, **kw).cpu()
+    assert torch.isfinite(out.float()).all()
+    ok, emax = _ok(out, want)
+    assert ok, emax
+
+
+@pytest.mark.parametrize("form", ["even", "device_cut"])
+def test_largest_plane_with_4bit_values(gpu, form):
+    """The same construction for the 4-bit-value kernels at their largest value store (2^24 - 256 rows of packed codes):
+    every row has scale 1/15 and zero-point 0, digit dimensions hold code 0 or 15, the others the block's own codes."""
+    from polarquant_amd import workloads as wl
+    from polarquant_amd.attention import polar_decode_attention_v4
+    print("case", form, flush=True)
+    G_BLK, N_BLK = 7, 18724
+    n_groups = G_BLK * N_BLK
+    rows, group_cap = (1 << 24) - 256, ((1 << 24) - 256) // 128
+    g = torch.Generator().manual_seed(78)
+    kb = wl.make_keys(1, 1, G_BLK * 128, 5e5, g, torch.float16)
+    quant = po.quantize_and_pack_nbit(kb, 4, 4)
+    q = wl.make_half((1, 4, 1, 128), g, torch.float16)
+    TB = G_BLK * 128
+    cb = torch.randint(0, 16, (TB, 128), generator=g, dtype=torch.int64)
+    cb[:, :16] = 0
+    pack = lambda c: (c.reshape(-1, 16, 8) << (4 * torch.arange(8))).sum(-1).to(torch.int32)      # dim 8w + i -> bits [4i, 4i + 4) of word w
+    scale_b = torch.full((1, 1, TB, 1), 1.0 / 15.0).half()
+    zero_b = torch.zeros(1, 1, TB, 1).half()
+    empty = torch.zeros(1, 1, 0, 128, dtype=torch.float16)
+    ref_block = po.decode_attention_mixed_exact(q, None, *quant, empty, pack(cb).reshape(1, 1, TB, 16), scale_b, zero_b, None, 4, 4)
+    codes = torch.zeros(1, 1, group_cap, 128, 64, dtype=torch.uint8, device=gpu)
+    codes[:, :, :n_groups] = quant[0].to(gpu).repeat(1, 1, N_BLK, 1, 1)
+    meta = []
+    for m in quant[1:]:
+        t = torch.zeros(1, 1, group_cap, 1, 64, dtype=torch.float16, device=gpu)
+        t[:, :, :n_groups] = m.to(gpu).repeat(1, 1, N_BLK, 1, 1)
+        meta.append(t)
+    T = n_groups * 128
+    # digits of the block number: dims 0..14 are codes 0 / 15 in words 0 and 1 (8 dims per word)
+    blk = torch.arange(T, device=gpu) // TB
+    vc = torch.full((1, 1, rows, 16), -1, dtype=torch.int32, device=gpu)
+    vc[0, 0, :T] = pack(cb).to(gpu).repeat(N_BLK, 1)
+    for w in range(2):
+        word = torch.zeros(T, dtype=torch.int64, device=gpu)
+        for i in range(8):
+            d = 8 * w + i
+            if d < 15:
+                word |= (((blk >> d) & 1) * 15) << (4 * i)
+        vc[0, 0, :T, w] = word.to(torch.int32)
+    del blk, word
+    vs = torch.full((1, 1, rows, 1), float("nan"), dtype=torch.float16, device=gpu)
+    vz = torch.full((1, 1, rows, 1), float("nan"), dtype=torch.float16, device=gpu)
+    vs[0, 0, :T] = 1.0 / 15.0
+    vz[0, 0, :T] = 0.0
+    want = ref_block.clone().double()
+    idx = torch.arange(N_BLK)
+    one = float(torch.tensor(1.0 / 15.0).half()) * 15.0
+    for d in range(15):
+        want[..., d] = float(((idx >> d) & 1).double().mean()) * one
+    want[..., 15] = 0.0
+    kres = torch.zeros(1, 1, 128, 128, dtype=torch.float16, device=gpu)
+    vres = torch.zeros(1, 1, 128, 128, dtype=torch.float16, device=gpu)
+    kw = dict(rbits=4, tbits=4)
+    if form == "device_cut":
+        kw.update(n_groups_per_seq=torch.tensor([n_groups], dtype=torch.int32, device=gpu),
+                  n_resid_per_seq=torch.tensor([0], dtype=torch.int32, device=gpu), balanced=True)
+    ng = 0 if form == "device_cut" else n_groups
+    out = polar_decode_attention_v4(q.to(gpu), codes, *meta, kres, vres, vc, vs, vz, ng, 0, **kw).cpu()
+    assert torch.isfinite(out.float()).all()
+    ok, emax = _ok(out, want)
+    assert ok, emax
