@@ -364,3 +364,36 @@ def test_largest_plane_with_4bit_values(gpu, form):
     assert torch.isfinite(out.float()).all()
     ok, emax = _ok(out, want)
     assert ok, emax
+
+
+def test_most_planes(gpu):
+    """The largest batch the entry points take: 65 520 (sequence, KV head) planes (the limit is 65 535).  Eight different
+    sequences repeated 1 023 times and a few more: the quantizer, the score op and the attention must give every replica
+    the bits of its original, and the originals must agree with the oracle."""
+    from polarquant_amd import workloads as wl
+    from polarquant_amd.kernel4group import attention_decode_forward_triton_impl
+    B0, Nk, reps = 8, 8, 1023
+    B = B0 * reps + 6                                   # 8 190 sequences x 8 KV heads = 65 520 planes
+    g = torch.Generator().manual_seed(91)
+    k0 = wl.make_keys(B0, Nk, 128 + 5, 5e5, g, torch.float16)
+    v0 = wl.make_half((B0, Nk, 128 + 5, 128), g, torch.float16)
+    q0 = wl.make_half((B0, Nk, 1, 128), g, torch.float16)
+    tile = lambda t: t.to(gpu).repeat(reps + 1, *([1] * (t.dim() - 1)))[:B].contiguous()
+    k, v, q = tile(k0), tile(v0), tile(q0)
+    quant = quantize_and_pack_nbit(k[:, :, :128], 4, 4)
+    ref_quant = po.quantize_and_pack_nbit(k0[:, :, :128].contiguous(), 4, 4)
+    for got, ref in zip(quant, ref_quant):
+        assert torch.equal(got[:B0].cpu().view(torch.uint8 if got.dtype == torch.uint8 else torch.int16),
+                           ref.view(torch.uint8 if ref.dtype == torch.uint8 else torch.int16))
+        assert torch.equal(got[B0:2 * B0], got[:B0]) and torch.equal(got[B - B0 - 6:B - 6], got[:B0]) and torch.equal(got[B - 6:], got[:6])
+    scores = attention_decode_forward_triton_impl(q, *quant, rbits=4, tbits=4)
+    ref_scores = po.decode_scores(q0, *ref_quant, 4, 4)
+    assert float((scores[:B0].cpu().double() - ref_scores.double()).abs().max()) <= 2e-5 * float(ref_scores.abs().max())
+    assert torch.equal(scores[B - B0 - 6:B - 6], scores[:B0]) and torch.equal(scores[B - 6:], scores[:6])
+    kres = torch.zeros(B, Nk, 128, 128, dtype=torch.float16, device=gpu)
+    kres[:, :, :5] = k[:, :, 128:]
+    out = polar_decode_attention(q, *quant, kres, v, 1, 5, rbits=4, tbits=4)
+    ref = po.decode_attention_exact(q0, k0[:, :, 128:], *ref_quant, v0, None, 4, 4)
+    ok, emax = _ok(out[:B0].cpu(), ref)
+    assert ok, emax
+    assert torch.equal(out[B0:2 * B0], out[:B0]) and torch.equal(out[B - B0 - 6:B - 6], out[:B0]) and torch.equal(out[B - 6:], out[:6])
