@@ -77,7 +77,8 @@ def _link(objs, lib: str) -> None:
 # probe builds: the library with one unit compiled for a timing-only experiment (results wrong on purpose); loaded by
 # polarquant_amd/benchmarks/probe_bench.py only
 PROBE_LIB = os.path.join(HERE, "libpolarquant_hip_probe.so")
-PROBES = {"no_values": {("pq_attn.hip", ".f16"): ("pq_attn.hip", ("PQ_DTYPE=0", "PQ_PROBE_NO_VALUES"), ".f16.no_values")}}
+PROBES = {"no_values": {("pq_attn.hip", ".f16"): ("pq_attn.hip", ("PQ_DTYPE=0", "PQ_PROBE_NO_VALUES"), ".f16.no_values")},
+          "direct_bins": {("pq_quantize.hip", ""): ("pq_quantize.hip", ("PQ_PROBE_DIRECT_BINS",), ".direct_bins")}}
 
 
 def build_probe(name: str, verbose: bool = True) -> str:

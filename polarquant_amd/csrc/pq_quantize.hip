@@ -366,6 +366,10 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(
     }
 }
 
+#ifdef PQ_PROBE_DIRECT_BINS
+#include "pq_quantize_probe.h"
+#endif
+
 // Exhaustive check of angle_radius against angle_radius_exact: block == bit pattern of y,
 // thread t covers x patterns t, t+256, ...; NaN operands are skipped.
 template <typename T, bool LIBM>
@@ -463,6 +467,18 @@ int launch_quantize(const void* k, const int64_t* strides, int dtype, int B, int
         if (packed6) PQ_LAUNCH_QP(T, U, true);                                                                       \
         else PQ_LAUNCH_QP(T, U, false);                                                                              \
     } while (0)
+#ifdef PQ_PROBE_DIRECT_BINS
+    // the probe build: every launch in the reference's angle mode with byte-per-code rows runs the probe kernel
+    if (!uniform && !packed6) {
+        if (dtype == 0)
+            hipLaunchKernelGGL(quantize_direct_bins_probe_kernel<F16>, grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],
+                               strides[2], Nk, rbits, tbits, am.two_pi, codes, (uint16_t*)rscale, (uint16_t*)rmn, (uint16_t*)tscale, (uint16_t*)tmn, cap, off);
+        else
+            hipLaunchKernelGGL(quantize_direct_bins_probe_kernel<BF16>, grid, block, 0, st, (const uint16_t*)k, strides[0], strides[1],
+                               strides[2], Nk, rbits, tbits, am.two_pi, codes, (uint16_t*)rscale, (uint16_t*)rmn, (uint16_t*)tscale, (uint16_t*)tmn, cap, off);
+        return static_cast<int>(hipGetLastError());
+    }
+#endif
     if (dtype == 0) { if (uniform) PQ_LAUNCH_Q(F16, true); else PQ_LAUNCH_Q(F16, false); }
     else            { if (uniform) PQ_LAUNCH_Q(BF16, true); else PQ_LAUNCH_Q(BF16, false); }
 #undef PQ_LAUNCH_Q
