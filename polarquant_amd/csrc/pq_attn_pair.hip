@@ -392,8 +392,10 @@ __device__ __forceinline__ EvenSlice even_slice(const SeqCounts& sc, int n_split
     return e;
 }
 
-// Even slices, one slice per pair: pair index = 4 * blockIdx.x + (pair within the block), laid out as attn_kernel's
-// block index (plane fastest).
+// Even slices, one slice per pair.  Grid (ceil(planes / 4), slices): a workgroup's four pairs take the same slice of four
+// consecutive (sequence, KV head) planes, and workgroups are handed out x first, so the plane index runs fastest as in
+// attn_kernel.  (One index taken apart by two more integer divisions cost 0.3-0.4 us ahead of the first loads; `n_slices_total`
+// is what the balanced kernel takes in this place and is not used here.)
 template <typename T, int TB, int REPP, bool PK6>
 __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(PQ_ATTN_KERNEL_PARAMS, int n_slices_total, int silent_scorer,
                                                                               int* __restrict__ status, uint16_t* __restrict__ direct_out) {
@@ -411,10 +413,9 @@ __global__ __launch_bounds__(kPairsPerBlock * 2 * kWave) void attn_pair_kernel(P
     pair_roles(simd_of, &flag_mem[0][0], wave, lane, pair, role);
     const PairMem pm = pair_mem(lds_addr(lut_mem[pair]), lds_addr(s_mem[pair]), lds_addr(p_mem[pair]), lds_addr(flag_mem[pair]), silent_scorer);
 
-    const int slice = blockIdx.x * kPairsPerBlock + pair;
-    if (slice >= n_slices_total) return;
-    const int units = n_slices_total / n_splits;
-    const int bh = slice % units, split = slice / units;
+    // grid (planes / 4, slices): workgroups are handed out x first, so the plane index runs fastest
+    const int bh = blockIdx.x * kPairsPerBlock + pair, split = blockIdx.y;
+    if (bh >= B * Nk) return;
     const int b = bh / Nk, kvh = bh - b * Nk;
     const V4Args v4none = v4;
     const SeqCounts sc = seq_counts<false>(p, v4none, b);
@@ -499,7 +500,10 @@ int launch_pair_tb(const AttnArgs& a, int total, hipStream_t st) {
 #define PQ_LAUNCH_PAIR_P(REPP, PK6)                                                                                  \
     do {                                                                                                             \
         if (a.balanced) PQ_LAUNCH_PAIR_K(attn_pair_balanced_kernel, REPP, PK6);                                      \
-        else PQ_LAUNCH_PAIR_K(attn_pair_kernel, REPP, PK6, static_cast<uint16_t*>(a.out));                           \
+        else {                                                                                                       \
+            const dim3 grid((a.B * a.Nk + kPairsPerBlock - 1) / kPairsPerBlock, a.n_splits);                         \
+            PQ_LAUNCH_PAIR_K(attn_pair_kernel, REPP, PK6, static_cast<uint16_t*>(a.out));                            \
+        }                                                                                                            \
     } while (0)
     // packed 6-bit code rows exist for tbits == 3 only (the 3/3 configuration)
 #define PQ_LAUNCH_PAIR(REPP)                                                                                         \
