@@ -17,8 +17,8 @@ __global__ __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(Lut<TB, R
     const uint32_t lut = lds_addr(lut_mem);
     const int lane = threadIdx.x;
     const int grp = blockIdx.x;
-    const int bh = blockIdx.y;             // b*Nk + kvh
-    const int b = bh / Nk, kvh = bh - b * Nk;
+    const int kvh = blockIdx.y, b = blockIdx.z;      // (grid dimensions of their own: no division ahead of the first loads)
+    const int bh = b * Nk + kvh;
     const size_t gidx = static_cast<size_t>(bh) * Nb + grp;
 
     // token codes of tile 0 and 1 (issued first: longest latency); rows of 64 bytes, or 48 when the
@@ -126,7 +126,7 @@ static int launch_tb(const void* q, const uint8_t* codes, const void* rscale, co
     int rep = rep_stride;
     const uint16_t* qp = static_cast<const uint16_t*>(q);
     float* op = out;
-    const dim3 grid(Nb, B * Nk);
+    const dim3 grid(Nb, Nk, B);
     if constexpr (TB == 7) {
         // 128 angle bins: a table holds four query heads at most (128 KiB); more heads per KV head go in two
         // launches, heads [0, 4) here and [4, rep) below
